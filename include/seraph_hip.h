@@ -1,0 +1,188 @@
+/*
+ * seraph_hip.h - C ABI of libseraph_hip.so: hand-written gfx950 (MI355X)
+ * kernels for the backward pass and optimizer of Seraph's training engine,
+ * plus the forward ops and the small device runtime a training step needs.
+ *
+ * Plain C: raw device pointers, sizes, and a stream handle (a hipStream_t
+ * passed as void*; NULL = the default stream).  No HIP types appear here, so
+ * the host side (src/hip_backend*.c, or the reference's own C code) compiles
+ * with any C compiler and without ROCm headers.
+ *
+ * Every entry point returns SERAPH_OK (0) or a negative error code and never
+ * aborts; seraph_hip_last_error() describes the most recent failure on the
+ * calling thread.  All launches are asynchronous on `stream`; ordering is the
+ * stream's in-order guarantee, which is the guarantee the reference gives
+ * between recorded ops (src/vulkan_backend_backward.c:124-142).
+ *
+ * Layouts (row-major FP32): activations [T, width] token-major with heads
+ * interleaved per token; projections [out, in]; seq_starts is a DEVICE array
+ * of batch+1 prefix offsets of the packed sequences, or NULL for one sequence.
+ * "ws"/"ws_bytes" is caller-owned device scratch; the matching *_ws_bytes()
+ * query gives the size an op needs (0 = none).  Scratch contents need not be
+ * preserved or initialised between calls.
+ *
+ * Each declaration cites the reference interface it stands in for
+ * (paths relative to the Seraph source tree).
+ */
+#ifndef SERAPH_HIP_H
+#define SERAPH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SERAPH_OK             0
+#define SERAPH_ERR_INVALID   -1   /* NULL pointer, bad shape, misaligned buffer */
+#define SERAPH_ERR_HIP       -2   /* a HIP runtime call or launch failed        */
+#define SERAPH_ERR_WORKSPACE -3   /* ws missing or smaller than *_ws_bytes()    */
+#define SERAPH_ERR_NODEVICE  -4   /* no gfx950 device visible                   */
+
+typedef void* seraph_stream_t;
+
+/* ---------------------------------------------------------------- runtime
+ * Stands in for the device half of vulkan_init_ex / vulkan_buffer_* /
+ * vulkan_cmd_end_submit (include/vulkan_backend.h:357-420). */
+typedef struct {
+    char     name[256];
+    char     arch[64];            /* "gfx950..."                          */
+    uint64_t hbm_bytes;
+    uint32_t compute_units;
+    uint32_t wavefront_size;
+    uint32_t lds_bytes_per_block;
+    uint32_t clock_khz;
+} seraph_device_info_t;
+
+const char* seraph_hip_last_error(void);
+int  seraph_hip_init(int device_index);                 /* -1 = device 0 */
+int  seraph_hip_device_info(seraph_device_info_t* out);
+int  seraph_hip_malloc(void** out, size_t bytes);
+int  seraph_hip_free(void* p);
+int  seraph_hip_host_alloc(void** out, size_t bytes);   /* pinned host memory */
+int  seraph_hip_host_free(void* p);
+int  seraph_hip_h2d(void* dst, const void* src, size_t bytes, seraph_stream_t s);
+int  seraph_hip_d2h(void* dst, const void* src, size_t bytes, seraph_stream_t s);
+int  seraph_hip_d2d(void* dst, const void* src, size_t bytes, seraph_stream_t s);
+int  seraph_hip_stream_create(seraph_stream_t* out);
+int  seraph_hip_stream_destroy(seraph_stream_t s);
+int  seraph_hip_stream_sync(seraph_stream_t s);
+int  seraph_hip_device_sync(void);
+/* event pair timing on a stream (vulkan_profiler_* stand-in, include/vulkan_backend.h:638-642) */
+int  seraph_hip_event_create(void** out);
+int  seraph_hip_event_destroy(void* ev);
+int  seraph_hip_event_record(void* ev, seraph_stream_t s);
+int  seraph_hip_event_elapsed_ms(void* start, void* stop, float* ms);  /* waits for stop */
+
+/* ---------------------------------------------------------------- utility ops */
+/* vulkan_fill_buffer / vulkan_fill_buffer_range, include/vulkan_backend.h:411-415,525-528 */
+int seraph_fill_u32(void* dst, uint32_t value, size_t count, seraph_stream_t s);
+/* vulkan_add / vulkan_mul / vulkan_scale, include/vulkan_backend.h:461-473 (shaders/add.comp, mul.comp, scale.comp) */
+int seraph_add(const float* a, const float* b, float* c, size_t n, seraph_stream_t s);
+int seraph_mul(const float* a, const float* b, float* c, size_t n, seraph_stream_t s);
+int seraph_scale(float* a, size_t n, float alpha, seraph_stream_t s);
+/* vulkan_nan_check, include/vulkan_backend.h:419-423 (shaders/nan_check.comp): flags[flag_index] |= 1 */
+int seraph_nan_check(const float* x, size_t n, uint32_t* flags, uint32_t flag_index, seraph_stream_t s);
+/* vulkan_reduce_sum, include/vulkan_backend.h:546-549 (shaders/reduce_sum.comp): out[g] = sum of 512 inputs */
+int seraph_reduce_sum(const float* in, float* out, size_t count, seraph_stream_t s);
+
+/* ---------------------------------------------------------------- loss */
+/* vulkan_cross_entropy_grad, include/vulkan_backend.h:538-543 (shaders/cross_entropy_grad.comp:33-99).
+ * seq_starts != NULL selects the packed form of cuda_train_cross_entropy_grad_packed
+ * (include/cuda_train_context.h:288): the last token of every sequence gives a zero row.
+ * valid_rows is the divisor (0 -> all gradients 0).  grad may alias logits. */
+int seraph_cross_entropy_grad(const float* logits, const uint32_t* targets, float* grad, float* loss_rows,
+                              const uint32_t* seq_starts, int batch,
+                              int64_t rows, int64_t cols, int64_t valid_rows, seraph_stream_t s);
+
+/* ---------------------------------------------------------------- GEMM family */
+/* vulkan_matmul (include/vulkan_backend.h:431-433, shaders/matmul.comp) and
+ * vulkan_matmul_transpose (include/vulkan_backend.h:439-442, shaders/matmul_transpose.comp:35-169):
+ * C[M,N] (+)= op(A) op(B); transposed A is stored [K,M], transposed B is stored [N,K]. */
+int seraph_gemm(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
+                int transpose_A, int transpose_B, int accumulate, seraph_stream_t s);
+
+/* ---------------------------------------------------------------- attention */
+/* vulkan_batch_attention (include/vulkan_backend.h:485-488, shaders/batch_attention_stream.comp)
+ * and cuda_train_batch_attention_packed (include/cuda_train_context.h:273): causal, GQA,
+ * block-diagonal over packed sequences; lse (optional, [T,H]) = logsumexp of the scaled scores. */
+int seraph_attention_forward(const float* Q, const float* K, const float* V, float* out, float* lse,
+                             const uint32_t* seq_starts, int batch, int64_t T,
+                             int heads, int kv_heads, int head_dim, float scale, seraph_stream_t s);
+/* vulkan_batch_attention_backward (include/vulkan_backend.h:566-572;
+ * shaders/batch_attention_backward.comp:50-196 and ..._stream.comp:34-202, no sequence cap) and
+ * cuda_train_batch_attention_backward_packed (include/cuda_train_context.h:285).
+ * attn_out and lse are optional saved forward results; when either is NULL both are
+ * recomputed from Q, K, V.  dQ is overwritten; dK/dV are ADDED into (the caller zeroes
+ * them first, src/train.c:5221-5222).  Deterministic: no atomics. */
+size_t seraph_attention_backward_ws_bytes(int64_t T, int heads, int kv_heads, int head_dim);
+int seraph_attention_backward(const float* Q, const float* K, const float* V, const float* dO,
+                              const float* attn_out, const float* lse,
+                              float* dQ, float* dK, float* dV,
+                              const uint32_t* seq_starts, int batch, int64_t T,
+                              int heads, int kv_heads, int head_dim, float scale,
+                              void* ws, size_t ws_bytes, seraph_stream_t s);
+
+/* ---------------------------------------------------------------- norm / position */
+/* vulkan_rmsnorm, include/vulkan_backend.h:499-503 (shaders/rmsnorm.comp) */
+int seraph_rmsnorm(const float* x, const float* scale, float* y, int64_t rows, int64_t cols, float eps,
+                   seraph_stream_t s);
+/* vulkan_rmsnorm_backward_batch, include/vulkan_backend.h:552-558
+ * (shaders/rmsnorm_backward_batch.comp:34-100): FP64 intermediates, rms floor 0.01,
+ * grad_scale accumulated (+=) with a deterministic two-stage column reduction. */
+size_t seraph_rmsnorm_backward_ws_bytes(int64_t rows, int64_t cols);
+int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy, float* dx, float* grad_scale,
+                            int64_t rows, int64_t cols, float eps, void* ws, size_t ws_bytes, seraph_stream_t s);
+/* vulkan_rope / vulkan_rope_backward, include/vulkan_backend.h:493-495,561-563
+ * (shaders/rope.comp, rope_backward.comp:26-59) and the packed forms
+ * (include/cuda_train_context.h:275,286).  in and out may alias.  backward != 0 applies
+ * the inverse rotation. */
+int seraph_rope(const float* in, float* out, const uint32_t* seq_starts, int batch, int64_t T,
+                int heads, int head_dim, float theta, int backward, seraph_stream_t s);
+/* vulkan_qk_norm, include/vulkan_backend.h:600-603 (shaders/qk_norm.comp:30-76): in place,
+ * no-op when use_qk_norm == 0.  The backward has no reference counterpart. */
+int seraph_qk_norm(float* qk, int64_t T, int heads, int head_dim, int use_qk_norm, float eps, seraph_stream_t s);
+int seraph_qk_norm_backward(const float* x_pre, const float* dy, float* dx, int64_t T, int heads, int head_dim,
+                            float eps, seraph_stream_t s);
+
+/* ---------------------------------------------------------------- element-wise */
+/* vulkan_silu, include/vulkan_backend.h:476-478 (shaders/silu.comp) */
+int seraph_silu(const float* x, float* y, size_t n, seraph_stream_t s);
+/* vulkan_silu_backward, include/vulkan_backend.h:582-586 (shaders/silu_backward.comp:26-41); dx may alias dy */
+int seraph_silu_backward(const float* x, const float* dy, float* dx, size_t n, seraph_stream_t s);
+/* vulkan_elementwise_mul_backward, include/vulkan_backend.h:591-597 (shaders/elementwise_mul_backward.comp:24-35) */
+int seraph_mul_backward(const float* A, const float* B, const float* dC, float* dA, float* dB, size_t n,
+                        seraph_stream_t s);
+/* The pair above fused as src/train.c:5131-5140 composes it, in one pass and without the
+ * cached silu(gate): dUp = dH*silu(gate), dGate = dH*up*silu'(gate). */
+int seraph_swiglu_backward(const float* gate, const float* up, const float* dH, float* dGate, float* dUp,
+                           size_t n, seraph_stream_t s);
+/* silu.comp then mul.comp in one pass (src/train.c:4726-4732): out = silu(gate)*up */
+int seraph_swiglu(const float* gate, const float* up, float* out, size_t n, seraph_stream_t s);
+
+/* ---------------------------------------------------------------- embedding */
+/* vulkan_embed_lookup, include/vulkan_backend.h:531-535 (shaders/embed_lookup.comp) */
+int seraph_embed_lookup(const uint32_t* tokens, const float* embed, float* out,
+                        int64_t T, int64_t hidden, int64_t vocab, seraph_stream_t s);
+/* vulkan_embedding_backward, include/vulkan_backend.h:575-579 (shaders/embedding_backward.comp:22-44):
+ * grad_embed[tok[p]] += dH[p], ids >= vocab skipped.  Deterministic: positions are grouped
+ * by token and each touched row is summed in position order by one workgroup. */
+size_t seraph_embedding_backward_ws_bytes(int64_t T, int64_t vocab);
+int seraph_embedding_backward(const uint32_t* tokens, const float* dH, float* grad_embed,
+                              int64_t T, int64_t hidden, int64_t vocab,
+                              void* ws, size_t ws_bytes, seraph_stream_t s);
+
+/* ---------------------------------------------------------------- optimizer */
+/* vulkan_adamw_update, include/vulkan_backend.h:445-452 (shaders/adamw.comp:36-61); bias
+ * corrections 1-powf(beta,step) on the host as src/vulkan_backend.c:2151-2152.
+ * clip <= 0: the reference formula.  clip > 0: each gradient element is first clamped to
+ * [-clip, clip] (an extension; the reference never clips). */
+int seraph_adamw(float* w, const float* g, float* m, float* v, size_t n,
+                 float lr, float beta1, float beta2, float weight_decay, float eps, int step, float clip,
+                 seraph_stream_t s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,544 @@
+// attention.hip - causal, grouped-query, packed-sequence attention on the FP32 matrix
+// cores: forward (with log-sum-exp) and a deterministic backward.
+//
+// Mathematics (shaders/batch_attention_backward.comp:50-196, ..._stream.comp:34-202):
+//   S = scale Q K^T (causal, block-diagonal over packed sequences), P = softmax(S),
+//   dV = P^T dO, dP = dO V^T, dS = P (dP - rowsum(P dP)), dQ = scale dS K, dK = scale dS^T Q.
+// rowsum(P dP) equals rowsum(dO O), so the backward takes the forward's O and LSE (saved
+// by the caller, or recomputed here) and never rebuilds the softmax statistics.
+//
+// All matrix products run on v_mfma_f32_32x32x2_f32.  Tiles sit in LDS as [row][D+4] in
+// their memory orientation and nothing is ever transposed through LDS: the accumulator
+// layout of the instruction (lane = column, registers = rows 8(v/4)+4(l/32)+v%4) is
+// exactly the operand layout of the next product when that product contracts over the
+// accumulator's row index, because both half-waves may supply any k as long as the two
+// operands agree.  Hence
+//   forward :  S^T = K Q^T  (lane = query)  ->  O^T += V^T P^T   (P straight from registers)
+//   dK/dV   :  S = Q K^T    (lane = key)    ->  dV += P^T dO, dK += dS^T Q
+//   dQ      :  S^T = K Q^T  (lane = query)  ->  dQ += dS K
+// The softmax statistics of a query are therefore per-lane scalars in the forward and dQ
+// kernels, and per-register values (read from LDS) in the dK/dV kernel.
+//
+// No atomics: one workgroup owns a key/value tile (for all query heads of its group) or a
+// query tile, so every output element is written by exactly one lane in a fixed order.
+// The price is that S and dP are formed twice (7 products instead of 5).
+//
+// Packed sequences: each lane looks up the start of its token's sequence once (binary
+// search over the batch+1 offsets); a score (i, j) is kept when start[i] <= j <= i.  Tiles are anchored on the global token
+// axis at multiples of 32/128, so ragged sequence lengths need no padding.
+#include <limits.h>
+
+#include "common.hpp"
+
+namespace seraph {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kAttnThreads = 256;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ v16f mfma(float a, float b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
+// row index inside a 32x32 accumulator block held by register v of a lane in half-wave h
+__device__ __forceinline__ int acc_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3); }
+
+// ---------------------------------------------------------------- sequence bounds of a token
+__device__ __forceinline__ int seq_start_of(const uint32_t* __restrict__ ss, int batch, int64_t t) {
+    return ss ? (int)ss[find_seq(ss, batch, t)] : 0;
+}
+__device__ __forceinline__ int seq_end_of(const uint32_t* __restrict__ ss, int batch, int64_t t, int64_t T) {
+    if (!ss) return (int)T;
+    const int64_t e = (int64_t)ss[find_seq(ss, batch, t) + 1];
+    return (int)(e < T ? e : T);
+}
+
+// ---------------------------------------------------------------- tile staging (32 rows x D)
+template <int D>
+struct Tile32 {
+    static constexpr int LD = D + 4;
+    static constexpr int kSlots = 32 * D / 4 / kAttnThreads;
+    float4 r[kSlots];
+    // rows row0..row0+31 of a token-major matrix with `stride` floats per token, columns col0..col0+D-1
+    __device__ __forceinline__ void gload(const float* __restrict__ base, int64_t row0, int64_t T, int64_t stride, int col0) {
+#pragma unroll
+        for (int u = 0; u < kSlots; u++) {
+            const int f = threadIdx.x + kAttnThreads * u;
+            const int row = f / (D / 4), c4 = f % (D / 4);
+            const int64_t t = row0 + row;
+            r[u] = t < T ? *reinterpret_cast<const float4*>(base + t * stride + col0 + 4 * c4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    __device__ __forceinline__ void sstore(float* __restrict__ lds) const {
+#pragma unroll
+        for (int u = 0; u < kSlots; u++) {
+            const int f = threadIdx.x + kAttnThreads * u;
+            *reinterpret_cast<float4*>(lds + (f / (D / 4)) * LD + 4 * (f % (D / 4))) = r[u];
+        }
+    }
+};
+
+// ---------------------------------------------------------------- forward
+// grid (query tiles of 128, heads); wave w owns queries i0+32w .. +31; key/value tiles of 32.
+template <int D>
+__global__ __launch_bounds__(kAttnThreads) void attn_fwd_kernel(const float* __restrict__ Q, const float* __restrict__ K,
+                                                                const float* __restrict__ V, float* __restrict__ O,
+                                                                float* __restrict__ LSE, const uint32_t* __restrict__ seq_starts, int batch,
+                                                                int64_t T, int H, int KVH, float scale_log2e) {
+    constexpr int LD = D + 4, DB = D / 32;
+    __shared__ __attribute__((aligned(16))) float sK[2][32 * LD];
+    __shared__ __attribute__((aligned(16))) float sV[2][32 * LD];
+    const int head = blockIdx.y, kvh = head / (H / KVH);
+    const int qt = gridDim.x - 1 - blockIdx.x;                 // long rows first
+    const int64_t i0 = (int64_t)qt * 128;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
+    const int64_t iw0 = i0 + 32 * w, i_lane = iw0 + r;
+    const bool row_ok = i_lane < T;
+    const int ss_lane = row_ok ? seq_start_of(seq_starts, batch, i_lane) : INT_MAX;
+    const int64_t qw = (int64_t)H * D, kw = (int64_t)KVH * D;
+
+    float4 qf[D / 8];
+#pragma unroll
+    for (int s8 = 0; s8 < D / 8; s8++)
+        qf[s8] = row_ok ? *reinterpret_cast<const float4*>(Q + i_lane * qw + head * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
+
+    const int64_t i_last = (i0 + 127 < T - 1) ? i0 + 127 : T - 1;
+    const int64_t jbeg = (seq_start_of(seq_starts, batch, i0) / 32) * 32;
+    const int ntiles = (int)((i_last + 1 - jbeg + 31) / 32);
+
+    float m = -INFINITY, l = 0.0f;
+    v16f o[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) o[db][v] = 0.0f;
+
+    Tile32<D> tk, tv;
+    tk.gload(K, jbeg, T, kw, kvh * D);
+    tv.gload(V, jbeg, T, kw, kvh * D);
+    tk.sstore(sK[0]);
+    tv.sstore(sV[0]);
+    __syncthreads();
+
+    for (int t = 0; t < ntiles; t++) {
+        const int cur = t & 1;
+        const int64_t j0 = jbeg + 32 * (int64_t)t;
+        if (t + 1 < ntiles) {
+            tk.gload(K, j0 + 32, T, kw, kvh * D);
+            tv.gload(V, j0 + 32, T, kw, kvh * D);
+        }
+        if (j0 <= iw0 + 31 && iw0 < T) {                        // some query of this wave can see this tile
+            v16f s;
+#pragma unroll
+            for (int v = 0; v < 16; v++) s[v] = 0.0f;
+#pragma unroll
+            for (int s8 = 0; s8 < D / 8; s8++) {
+                const float4 a = *reinterpret_cast<const float4*>(&sK[cur][r * LD + s8 * 8 + 4 * h]);
+                s = mfma(a.x, qf[s8].x, s); s = mfma(a.y, qf[s8].y, s);
+                s = mfma(a.z, qf[s8].z, s); s = mfma(a.w, qf[s8].w, s);
+            }
+            float mloc = -INFINITY;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int64_t j = j0 + acc_row(v, h);
+                const bool valid = (j >= ss_lane) && (j <= i_lane);
+                s[v] = valid ? s[v] * scale_log2e : -INFINITY;
+                mloc = fmaxf(mloc, s[v]);
+            }
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+            const float mnew = fmaxf(m, mloc);
+            const float msafe = mnew == -INFINITY ? 0.0f : mnew;
+            const float alpha = fast_exp2(m - msafe);
+            float lsum = 0.0f;
+#pragma unroll
+            for (int v = 0; v < 16; v++) { s[v] = fast_exp2(s[v] - msafe); lsum += s[v]; }
+            lsum += __shfl_xor(lsum, 32, 64);
+            l = l * alpha + lsum;
+            m = mnew;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) o[db][v] *= alpha;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int jl = acc_row(v, h);
+#pragma unroll
+                for (int db = 0; db < DB; db++) o[db] = mfma(sV[cur][jl * LD + db * 32 + r], s[v], o[db]);
+            }
+        }
+        if (t + 1 < ntiles) {
+            tk.sstore(sK[cur ^ 1]);
+            tv.sstore(sV[cur ^ 1]);
+        }
+        __syncthreads();
+    }
+
+    if (row_ok) {
+        const float inv = 1.0f / l;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                float4 out = make_float4(o[db][4 * g] * inv, o[db][4 * g + 1] * inv, o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
+                *reinterpret_cast<float4*>(O + i_lane * qw + head * D + db * 32 + 8 * g + 4 * h) = out;
+            }
+        if (LSE && h == 0) LSE[i_lane * H + head] = (m + __log2f(l)) * kLn2;
+    }
+}
+
+// ---------------------------------------------------------------- delta = rowsum(dO * O)
+// one wave per token; a head's D values are spread over D/4 consecutive lanes
+template <int D>
+__global__ __launch_bounds__(256) void attn_delta_kernel(const float* __restrict__ dO, const float* __restrict__ O,
+                                                         float* __restrict__ delta, int64_t T, int H) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= T) return;
+    const int64_t qw = (int64_t)H * D;
+    constexpr int LPH = D / 4;                                  // lanes per head
+    for (int64_t c = lane * 4; c < qw; c += 256) {
+        const float4 a = *reinterpret_cast<const float4*>(dO + t * qw + c);
+        const float4 b = *reinterpret_cast<const float4*>(O + t * qw + c);
+        float s = a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w;
+#pragma unroll
+        for (int o = LPH / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+        if ((lane % LPH) == 0) delta[t * H + c / D] = s;
+    }
+}
+
+// ---------------------------------------------------------------- backward: dK, dV
+// grid (key tiles of 128, kv heads); wave w owns keys j0+32w .. +31 for every query head of the group.
+template <int D>
+__global__ __launch_bounds__(kAttnThreads) void attn_bwd_dkv_kernel(const float* __restrict__ Q, const float* __restrict__ K,
+                                                                    const float* __restrict__ V, const float* __restrict__ dO,
+                                                                    const float* __restrict__ LSE, const float* __restrict__ DELTA,
+                                                                    float* __restrict__ dK, float* __restrict__ dV,
+                                                                    const uint32_t* __restrict__ seq_starts, int batch,
+                                                                    int64_t T, int H, int KVH, float scale, float scale_log2e) {
+    constexpr int LD = D + 4, DB = D / 32;
+    __shared__ __attribute__((aligned(16))) float sQ[2][32 * LD];
+    __shared__ __attribute__((aligned(16))) float sG[2][32 * LD];     // dO
+    __shared__ __attribute__((aligned(16))) float sLse[2][32];
+    __shared__ __attribute__((aligned(16))) float sDel[2][32];
+    __shared__ __attribute__((aligned(16))) int sSS[2][32];
+    const int kvh = blockIdx.y, G = H / KVH;
+    const int64_t j0 = (int64_t)blockIdx.x * 128;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
+    const int64_t jw0 = j0 + 32 * w, j_lane = jw0 + r;
+    const bool col_ok = j_lane < T;
+    const int64_t qw = (int64_t)H * D, kw = (int64_t)KVH * D;
+
+    float4 kf[D / 8], vf[D / 8];
+#pragma unroll
+    for (int s8 = 0; s8 < D / 8; s8++) {
+        kf[s8] = col_ok ? *reinterpret_cast<const float4*>(K + j_lane * kw + kvh * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
+        vf[s8] = col_ok ? *reinterpret_cast<const float4*>(V + j_lane * kw + kvh * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    v16f dk[DB], dv[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) { dk[db][v] = 0.0f; dv[db][v] = 0.0f; }
+
+    const int64_t j_last = (j0 + 127 < T - 1) ? j0 + 127 : T - 1;
+    const int64_t i_end = seq_end_of(seq_starts, batch, j_last, T);                         // queries of the last key's sequence
+    const int nq = (int)((i_end - j0 + 31) / 32);
+    const int iters = nq * G;
+
+    Tile32<D> tq, tg;
+    float st_lse = 0.f, st_del = 0.f;
+    int st_ss = INT_MAX;
+    auto stats_load = [&](int it) {
+        const int head = kvh * G + it / nq;
+        const int64_t i = j0 + 32 * (int64_t)(it % nq) + (threadIdx.x & 31);
+        if (threadIdx.x < 32) {
+            st_lse = i < T ? LSE[i * H + head] * kLog2e : 0.f;
+            st_del = i < T ? DELTA[i * H + head] : 0.f;
+            st_ss = i < T ? seq_start_of(seq_starts, batch, i) : INT_MAX;
+        }
+    };
+    auto stats_store = [&](int buf) {
+        if (threadIdx.x < 32) { sLse[buf][threadIdx.x] = st_lse; sDel[buf][threadIdx.x] = st_del; sSS[buf][threadIdx.x] = st_ss; }
+    };
+    auto tiles_load = [&](int it) {
+        const int head = kvh * G + it / nq;
+        const int64_t i0 = j0 + 32 * (int64_t)(it % nq);
+        tq.gload(Q, i0, T, qw, head * D);
+        tg.gload(dO, i0, T, qw, head * D);
+    };
+
+    tiles_load(0); stats_load(0);
+    tq.sstore(sQ[0]); tg.sstore(sG[0]); stats_store(0);
+    __syncthreads();
+
+    for (int it = 0; it < iters; it++) {
+        const int cur = it & 1;
+        const int64_t i0 = j0 + 32 * (int64_t)(it % nq);
+        if (it + 1 < iters) { tiles_load(it + 1); stats_load(it + 1); }
+        if (i0 + 31 >= jw0 && jw0 < T) {                        // some query of the tile can see this wave's keys
+            v16f s, dp;
+#pragma unroll
+            for (int v = 0; v < 16; v++) { s[v] = 0.0f; dp[v] = 0.0f; }
+#pragma unroll
+            for (int s8 = 0; s8 < D / 8; s8++) {
+                const float4 a = *reinterpret_cast<const float4*>(&sQ[cur][r * LD + s8 * 8 + 4 * h]);
+                const float4 b = *reinterpret_cast<const float4*>(&sG[cur][r * LD + s8 * 8 + 4 * h]);
+                s = mfma(a.x, kf[s8].x, s); dp = mfma(b.x, vf[s8].x, dp);
+                s = mfma(a.y, kf[s8].y, s); dp = mfma(b.y, vf[s8].y, dp);
+                s = mfma(a.z, kf[s8].z, s); dp = mfma(b.z, vf[s8].z, dp);
+                s = mfma(a.w, kf[s8].w, s); dp = mfma(b.w, vf[s8].w, dp);
+            }
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const float4 lse4 = *reinterpret_cast<const float4*>(&sLse[cur][8 * g + 4 * h]);
+                const float4 del4 = *reinterpret_cast<const float4*>(&sDel[cur][8 * g + 4 * h]);
+                const int4 ss4 = *reinterpret_cast<const int4*>(&sSS[cur][8 * g + 4 * h]);
+                const float* lse_p = &lse4.x; const float* del_p = &del4.x; const int* ss_p = &ss4.x;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int v = 4 * g + e;
+                    const int64_t i = i0 + 8 * g + 4 * h + e;
+                    const bool valid = (j_lane <= i) && (j_lane >= ss_p[e]);       // ss = INT_MAX for i >= T
+                    const float p = valid ? fast_exp2(s[v] * scale_log2e - lse_p[e]) : 0.0f;
+                    s[v] = p;
+                    dp[v] = p * (dp[v] - del_p[e]);
+                }
+            }
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int il = acc_row(v, h);
+#pragma unroll
+                for (int db = 0; db < DB; db++) {
+                    dv[db] = mfma(s[v], sG[cur][il * LD + db * 32 + r], dv[db]);
+                    dk[db] = mfma(dp[v], sQ[cur][il * LD + db * 32 + r], dk[db]);
+                }
+            }
+        }
+        if (it + 1 < iters) { tq.sstore(sQ[cur ^ 1]); tg.sstore(sG[cur ^ 1]); stats_store(cur ^ 1); }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int64_t j = jw0 + acc_row(v, h);
+            if (j < T) {
+                const int64_t off = j * kw + kvh * D + db * 32 + r;
+                dK[off] += dk[db][v] * scale;
+                dV[off] += dv[db][v];
+            }
+        }
+}
+
+// ---------------------------------------------------------------- backward: dQ
+// grid (query tiles of 128, heads); wave w owns queries i0+32w .. +31; key/value tiles of 32.
+template <int D>
+__global__ __launch_bounds__(kAttnThreads) void attn_bwd_dq_kernel(const float* __restrict__ Q, const float* __restrict__ K,
+                                                                   const float* __restrict__ V, const float* __restrict__ dO,
+                                                                   const float* __restrict__ LSE, const float* __restrict__ DELTA,
+                                                                   float* __restrict__ dQ, const uint32_t* __restrict__ seq_starts, int batch,
+                                                                   int64_t T, int H, int KVH, float scale, float scale_log2e) {
+    constexpr int LD = D + 4, DB = D / 32;
+    __shared__ __attribute__((aligned(16))) float sK[2][32 * LD];
+    __shared__ __attribute__((aligned(16))) float sV[2][32 * LD];
+    const int head = blockIdx.y, kvh = head / (H / KVH);
+    const int qt = gridDim.x - 1 - blockIdx.x;
+    const int64_t i0 = (int64_t)qt * 128;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
+    const int64_t iw0 = i0 + 32 * w, i_lane = iw0 + r;
+    const bool row_ok = i_lane < T;
+    const int ss_lane = row_ok ? seq_start_of(seq_starts, batch, i_lane) : INT_MAX;
+    const float lse_i = row_ok ? LSE[i_lane * H + head] * kLog2e : 0.0f;
+    const float del_i = row_ok ? DELTA[i_lane * H + head] : 0.0f;
+    const int64_t qw = (int64_t)H * D, kw = (int64_t)KVH * D;
+
+    float4 qf[D / 8], gf[D / 8];
+#pragma unroll
+    for (int s8 = 0; s8 < D / 8; s8++) {
+        qf[s8] = row_ok ? *reinterpret_cast<const float4*>(Q + i_lane * qw + head * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
+        gf[s8] = row_ok ? *reinterpret_cast<const float4*>(dO + i_lane * qw + head * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    v16f dq[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) dq[db][v] = 0.0f;
+
+    const int64_t i_last = (i0 + 127 < T - 1) ? i0 + 127 : T - 1;
+    const int64_t jbeg = (seq_start_of(seq_starts, batch, i0) / 32) * 32;
+    const int ntiles = (int)((i_last + 1 - jbeg + 31) / 32);
+
+    Tile32<D> tk, tv;
+    tk.gload(K, jbeg, T, kw, kvh * D);
+    tv.gload(V, jbeg, T, kw, kvh * D);
+    tk.sstore(sK[0]);
+    tv.sstore(sV[0]);
+    __syncthreads();
+
+    for (int t = 0; t < ntiles; t++) {
+        const int cur = t & 1;
+        const int64_t j0 = jbeg + 32 * (int64_t)t;
+        if (t + 1 < ntiles) {
+            tk.gload(K, j0 + 32, T, kw, kvh * D);
+            tv.gload(V, j0 + 32, T, kw, kvh * D);
+        }
+        if (j0 <= iw0 + 31 && iw0 < T) {
+            v16f s, dp;
+#pragma unroll
+            for (int v = 0; v < 16; v++) { s[v] = 0.0f; dp[v] = 0.0f; }
+#pragma unroll
+            for (int s8 = 0; s8 < D / 8; s8++) {
+                const float4 a = *reinterpret_cast<const float4*>(&sK[cur][r * LD + s8 * 8 + 4 * h]);
+                const float4 b = *reinterpret_cast<const float4*>(&sV[cur][r * LD + s8 * 8 + 4 * h]);
+                s = mfma(a.x, qf[s8].x, s); dp = mfma(b.x, gf[s8].x, dp);
+                s = mfma(a.y, qf[s8].y, s); dp = mfma(b.y, gf[s8].y, dp);
+                s = mfma(a.z, qf[s8].z, s); dp = mfma(b.z, gf[s8].z, dp);
+                s = mfma(a.w, qf[s8].w, s); dp = mfma(b.w, gf[s8].w, dp);
+            }
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int64_t j = j0 + acc_row(v, h);
+                const bool valid = (j >= ss_lane) && (j <= i_lane);
+                const float p = valid ? fast_exp2(s[v] * scale_log2e - lse_i) : 0.0f;
+                dp[v] = p * (dp[v] - del_i);
+            }
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int jl = acc_row(v, h);
+#pragma unroll
+                for (int db = 0; db < DB; db++) dq[db] = mfma(dp[v], sK[cur][jl * LD + db * 32 + r], dq[db]);
+            }
+        }
+        if (t + 1 < ntiles) {
+            tk.sstore(sK[cur ^ 1]);
+            tv.sstore(sV[cur ^ 1]);
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int64_t i = iw0 + acc_row(v, h);
+            if (i < T) dQ[i * qw + head * D + db * 32 + r] = dq[db][v] * scale;
+        }
+}
+
+// ---------------------------------------------------------------- host side
+struct AttnWs { float* lse; float* delta; float* out; };
+
+static size_t a256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+static size_t attn_ws_layout(int64_t T, int H, int D, char* base, AttnWs* w) {
+    size_t o = 0;
+    auto take = [&](size_t bytes) { char* p = base ? base + o : nullptr; o += a256(bytes); return p; };
+    char* c = take((size_t)T * H * 4); char* d = take((size_t)T * H * 4);
+    char* e = take((size_t)T * H * D * 4);
+    if (w) { w->lse = (float*)c; w->delta = (float*)d; w->out = (float*)e; }
+    return o;
+}
+
+static int check_attn_shape(const char* who, int64_t T, int H, int KVH, int D) {
+    SERAPH_REQUIRE(T > 0 && T < 0x7fffff00LL, "%s: bad token count %lld", who, (long long)T);
+    SERAPH_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "%s: heads (%d) must be a multiple of kv_heads (%d)", who, H, KVH);
+    SERAPH_REQUIRE(D == 32 || D == 64 || D == 128, "%s: head_dim %d not supported (32, 64, 128)", who, D);
+    return SERAPH_OK;
+}
+
+template <int D>
+static int run_forward(const float* Q, const float* K, const float* V, float* O, float* lse, const uint32_t* seq_starts, int batch,
+                       int64_t T, int H, int KVH, float scale, hipStream_t st) {
+    dim3 grid((unsigned)ceil_div(T, 128), (unsigned)H);
+    hipLaunchKernelGGL(attn_fwd_kernel<D>, grid, dim3(kAttnThreads), 0, st, Q, K, V, O, lse, seq_starts, batch, T, H, KVH, scale * kLog2e);
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
+}
+
+template <int D>
+static int run_backward(const float* Q, const float* K, const float* V, const float* dO, const float* O, const float* lse,
+                        float* delta, float* dQ, float* dK, float* dV, const uint32_t* seq_starts, int batch,
+                        int64_t T, int H, int KVH, float scale, hipStream_t st) {
+    hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)ceil_div(T, 4)), dim3(256), 0, st, dO, O, delta, T, H);
+    SERAPH_LAUNCH_CHECK();
+    dim3 gkv((unsigned)ceil_div(T, 128), (unsigned)KVH), gq((unsigned)ceil_div(T, 128), (unsigned)H);
+    hipLaunchKernelGGL(attn_bwd_dkv_kernel<D>, gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dK, dV, seq_starts, batch,
+                       T, H, KVH, scale, scale * kLog2e);
+    SERAPH_LAUNCH_CHECK();
+    hipLaunchKernelGGL(attn_bwd_dq_kernel<D>, gq, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dQ, seq_starts, batch,
+                       T, H, KVH, scale, scale * kLog2e);
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
+}
+
+}  // namespace seraph
+
+using namespace seraph;
+
+extern "C" {
+
+size_t seraph_attention_backward_ws_bytes(int64_t T, int heads, int kv_heads, int head_dim) {
+    (void)kv_heads;
+    if (T <= 0 || heads <= 0 || head_dim <= 0) return 0;
+    return attn_ws_layout(T, heads, head_dim, nullptr, nullptr);
+}
+
+int seraph_attention_forward(const float* Q, const float* K, const float* V, float* out, float* lse,
+                             const uint32_t* seq_starts, int batch, int64_t T,
+                             int heads, int kv_heads, int head_dim, float scale, seraph_stream_t s) {
+    if (T == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(Q && K && V && out, "attention_forward: NULL pointer");
+    int rc = check_attn_shape("attention_forward", T, heads, kv_heads, head_dim);
+    if (rc != SERAPH_OK) return rc;
+    SERAPH_REQUIRE(aligned16(Q) && aligned16(K) && aligned16(V) && aligned16(out), "attention_forward: buffers must be 16-byte aligned");
+    SERAPH_REQUIRE(!seq_starts || batch >= 1, "attention_forward: packed call needs batch >= 1");
+    hipStream_t st = as_stream(s);
+    switch (head_dim) {
+        case 32: rc = run_forward<32>(Q, K, V, out, lse, seq_starts, batch, T, heads, kv_heads, scale, st); break;
+        case 64: rc = run_forward<64>(Q, K, V, out, lse, seq_starts, batch, T, heads, kv_heads, scale, st); break;
+        default: rc = run_forward<128>(Q, K, V, out, lse, seq_starts, batch, T, heads, kv_heads, scale, st); break;
+    }
+    return rc;
+}
+
+int seraph_attention_backward(const float* Q, const float* K, const float* V, const float* dO,
+                              const float* attn_out, const float* lse,
+                              float* dQ, float* dK, float* dV,
+                              const uint32_t* seq_starts, int batch, int64_t T,
+                              int heads, int kv_heads, int head_dim, float scale,
+                              void* ws, size_t ws_bytes, seraph_stream_t s) {
+    if (T == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(Q && K && V && dO && dQ && dK && dV, "attention_backward: NULL pointer");
+    int rc = check_attn_shape("attention_backward", T, heads, kv_heads, head_dim);
+    if (rc != SERAPH_OK) return rc;
+    SERAPH_REQUIRE(aligned16(Q) && aligned16(K) && aligned16(V) && aligned16(dO) && (!attn_out || aligned16(attn_out)),
+                   "attention_backward: buffers must be 16-byte aligned");
+    SERAPH_REQUIRE(!seq_starts || batch >= 1, "attention_backward: packed call needs batch >= 1");
+    if (!ws || !aligned16(ws) || ws_bytes < seraph_attention_backward_ws_bytes(T, heads, kv_heads, head_dim)) {
+        set_error("attention_backward: 16-byte aligned scratch of %zu bytes required",
+                  seraph_attention_backward_ws_bytes(T, heads, kv_heads, head_dim));
+        return SERAPH_ERR_WORKSPACE;
+    }
+    AttnWs w;
+    attn_ws_layout(T, heads, head_dim, (char*)ws, &w);
+    hipStream_t st = as_stream(s);
+    const float* O = attn_out;
+    const float* L = lse;
+    if (!O || !L) {                                              // recompute the forward results
+        switch (head_dim) {
+            case 32: rc = run_forward<32>(Q, K, V, w.out, w.lse, seq_starts, batch, T, heads, kv_heads, scale, st); break;
+            case 64: rc = run_forward<64>(Q, K, V, w.out, w.lse, seq_starts, batch, T, heads, kv_heads, scale, st); break;
+            default: rc = run_forward<128>(Q, K, V, w.out, w.lse, seq_starts, batch, T, heads, kv_heads, scale, st); break;
+        }
+        if (rc != SERAPH_OK) return rc;
+        O = w.out; L = w.lse;
+    }
+    switch (head_dim) {
+        case 32: return run_backward<32>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, st);
+        case 64: return run_backward<64>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, st);
+        default: return run_backward<128>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, st);
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,294 @@
+// elementwise.hip - bandwidth-bound streaming kernels: fill, add, mul, scale, silu,
+// silu/mul backward, fused SwiGLU forward/backward, nan check, 512-wide reduce, AdamW.
+//
+// All of them are one pass over HBM: every input element is read once and every
+// output element written once, 16 bytes per lane per access, several independent
+// accesses in flight per lane, grid sized to a few waves per SIMD and strided.
+#include "common.hpp"
+
+namespace seraph {
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;      // independent float4 accesses in flight per lane and stream
+
+static inline int stream_grid(size_t n4) {
+    int64_t want = ceil_div((int64_t)n4, (int64_t)kBlock * kUnroll);
+    int64_t cap = (int64_t)num_compute_units() * 16;
+    if (want < 1) want = 1;
+    return (int)(want < cap ? want : cap);
+}
+
+// F provides:  void vec(size_t i4) const   - one float4 slot
+//              void one(size_t i)  const   - one scalar element
+template <typename F>
+__global__ __launch_bounds__(kBlock) void stream_kernel(F f, size_t n4, size_t n, int vec_ok) {
+    const size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    if (vec_ok) {
+        size_t i = tid;
+        for (; i + (kUnroll - 1) * stride < n4; i += kUnroll * stride) {
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) f.vec(i + u * stride);
+        }
+        for (; i < n4; i += stride) f.vec(i);
+        for (size_t j = n4 * 4 + tid; j < n; j += stride) f.one(j);
+    } else {
+        for (size_t j = tid; j < n; j += stride) f.one(j);
+    }
+}
+
+template <typename F>
+static int launch_stream(F f, size_t n, bool vec_ok, hipStream_t st) {
+    if (n == 0) return SERAPH_OK;
+    size_t n4 = vec_ok ? n / 4 : 0;
+    int grid = stream_grid(vec_ok ? n4 : n / 4 + 1);
+    hipLaunchKernelGGL(stream_kernel<F>, dim3(grid), dim3(kBlock), 0, st, f, n4, n, vec_ok ? 1 : 0);
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
+}
+
+__device__ __forceinline__ float4 ld4(const float* p, size_t i4) { return reinterpret_cast<const float4*>(p)[i4]; }
+__device__ __forceinline__ void st4(float* p, size_t i4, float4 v) { reinterpret_cast<float4*>(p)[i4] = v; }
+
+#define MAP4(expr_x, expr_y, expr_z, expr_w) make_float4(expr_x, expr_y, expr_z, expr_w)
+
+// ---------------------------------------------------------------- functors
+struct FillOp {
+    uint32_t* dst; uint32_t value;
+    __device__ void vec(size_t i) const { reinterpret_cast<uint4*>(dst)[i] = make_uint4(value, value, value, value); }
+    __device__ void one(size_t i) const { dst[i] = value; }
+};
+
+struct AddOp {
+    const float* a; const float* b; float* c;
+    __device__ void vec(size_t i) const {
+        float4 x = ld4(a, i), y = ld4(b, i);
+        st4(c, i, MAP4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w));
+    }
+    __device__ void one(size_t i) const { c[i] = a[i] + b[i]; }
+};
+
+struct MulOp {
+    const float* a; const float* b; float* c;
+    __device__ void vec(size_t i) const {
+        float4 x = ld4(a, i), y = ld4(b, i);
+        st4(c, i, MAP4(x.x * y.x, x.y * y.y, x.z * y.z, x.w * y.w));
+    }
+    __device__ void one(size_t i) const { c[i] = a[i] * b[i]; }
+};
+
+struct ScaleOp {
+    float* a; float alpha;
+    __device__ void vec(size_t i) const {
+        float4 x = ld4(a, i);
+        st4(a, i, MAP4(x.x * alpha, x.y * alpha, x.z * alpha, x.w * alpha));
+    }
+    __device__ void one(size_t i) const { a[i] *= alpha; }
+};
+
+// shaders/silu.comp: x / (1 + exp(-x))
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+// shaders/silu_backward.comp:33-40: s*(1 + x*(1-s)), s = 1/(1+exp(-x))
+__device__ __forceinline__ float silu_grad_f(float x) {
+    float s = 1.0f / (1.0f + __expf(-x));
+    return s * (1.0f + x * (1.0f - s));
+}
+
+struct SiluOp {
+    const float* x; float* y;
+    __device__ void vec(size_t i) const {
+        float4 v = ld4(x, i);
+        st4(y, i, MAP4(silu_f(v.x), silu_f(v.y), silu_f(v.z), silu_f(v.w)));
+    }
+    __device__ void one(size_t i) const { y[i] = silu_f(x[i]); }
+};
+
+struct SiluBwdOp {
+    const float* x; const float* dy; float* dx;
+    __device__ void vec(size_t i) const {
+        float4 v = ld4(x, i), g = ld4(dy, i);
+        st4(dx, i, MAP4(g.x * silu_grad_f(v.x), g.y * silu_grad_f(v.y), g.z * silu_grad_f(v.z), g.w * silu_grad_f(v.w)));
+    }
+    __device__ void one(size_t i) const { dx[i] = dy[i] * silu_grad_f(x[i]); }
+};
+
+struct MulBwdOp {
+    const float* A; const float* B; const float* dC; float* dA; float* dB;
+    __device__ void vec(size_t i) const {
+        float4 a = ld4(A, i), b = ld4(B, i), g = ld4(dC, i);
+        st4(dA, i, MAP4(g.x * b.x, g.y * b.y, g.z * b.z, g.w * b.w));
+        st4(dB, i, MAP4(g.x * a.x, g.y * a.y, g.z * a.z, g.w * a.w));
+    }
+    __device__ void one(size_t i) const { float a = A[i], b = B[i], g = dC[i]; dA[i] = g * b; dB[i] = g * a; }
+};
+
+// dUp = dH * silu(gate); dGate = (dH * up) * silu'(gate): 3 reads + 2 writes per element.
+struct SwigluBwdOp {
+    const float* gate; const float* up; const float* dH; float* dGate; float* dUp;
+    __device__ __forceinline__ void elem(float x, float u, float g, float& dg, float& du) const {
+        float s = 1.0f / (1.0f + __expf(-x));
+        du = g * (x * s);
+        dg = (g * u) * (s * (1.0f + x * (1.0f - s)));
+    }
+    __device__ void vec(size_t i) const {
+        float4 x = ld4(gate, i), u = ld4(up, i), g = ld4(dH, i), dg, du;
+        elem(x.x, u.x, g.x, dg.x, du.x); elem(x.y, u.y, g.y, dg.y, du.y);
+        elem(x.z, u.z, g.z, dg.z, du.z); elem(x.w, u.w, g.w, dg.w, du.w);
+        st4(dGate, i, dg); st4(dUp, i, du);
+    }
+    __device__ void one(size_t i) const { float dg, du; elem(gate[i], up[i], dH[i], dg, du); dGate[i] = dg; dUp[i] = du; }
+};
+
+struct SwigluOp {
+    const float* gate; const float* up; float* out;
+    __device__ void vec(size_t i) const {
+        float4 x = ld4(gate, i), u = ld4(up, i);
+        st4(out, i, MAP4(silu_f(x.x) * u.x, silu_f(x.y) * u.y, silu_f(x.z) * u.z, silu_f(x.w) * u.w));
+    }
+    __device__ void one(size_t i) const { out[i] = silu_f(gate[i]) * up[i]; }
+};
+
+// shaders/adamw.comp:43-60 in its own expression order.  Divisions and the square root
+// are the IEEE-rounded ones; clip > 0 clamps the gradient first.
+struct AdamWOp {
+    float* w; const float* g; float* m; float* v;
+    float lr, beta1, beta2, wd, eps, bc1, bc2, clip;
+    __device__ __forceinline__ void elem(float& wi, float gi, float& mi, float& vi) const {
+        if (clip > 0.0f) gi = fminf(fmaxf(gi, -clip), clip);
+        float mn = beta1 * mi + (1.0f - beta1) * gi;
+        float vn = beta2 * vi + (1.0f - beta2) * gi * gi;
+        mi = mn; vi = vn;
+        float mh = mn / bc1, vh = vn / bc2;
+        wi = wi * (1.0f - lr * wd) - lr * mh / (sqrtf(vh) + eps);
+    }
+    __device__ void vec(size_t i) const {
+        float4 W = ld4(w, i), G = ld4(g, i), M = ld4(m, i), V = ld4(v, i);
+        elem(W.x, G.x, M.x, V.x); elem(W.y, G.y, M.y, V.y); elem(W.z, G.z, M.z, V.z); elem(W.w, G.w, M.w, V.w);
+        st4(m, i, M); st4(v, i, V); st4(w, i, W);
+    }
+    __device__ void one(size_t i) const { float W = w[i], M = m[i], V = v[i]; elem(W, g[i], M, V); m[i] = M; v[i] = V; w[i] = W; }
+};
+
+// ---------------------------------------------------------------- nan check, reduce
+__global__ __launch_bounds__(kBlock) void nan_check_kernel(const float* __restrict__ x, size_t n,
+                                                           uint32_t* flags, uint32_t flag_index) {
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    int bad = 0;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+        uint32_t bits = __float_as_uint(x[i]);
+        bad |= ((bits & 0x7f800000u) == 0x7f800000u) ? 1 : 0;     // exponent all ones: Inf or NaN
+    }
+    if (__any(bad) && (threadIdx.x & 63) == 0) atomicOr(&flags[flag_index], 1u);
+}
+
+// out[g] = sum of in[512 g .. 512 g + 511]
+__global__ __launch_bounds__(kBlock) void reduce_sum_512_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                                size_t count) {
+    __shared__ float part[kBlock / kWave];
+    size_t base = (size_t)blockIdx.x * 512;
+    size_t i0 = base + threadIdx.x, i1 = i0 + kBlock;
+    float v = (i0 < count ? in[i0] : 0.0f) + (i1 < count ? in[i1] : 0.0f);
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) out[blockIdx.x] = (part[0] + part[1]) + (part[2] + part[3]);
+}
+
+}  // namespace seraph
+
+using namespace seraph;
+
+#define ALL_ALIGNED(...) ([&] { const void* ps_[] = {__VA_ARGS__}; for (const void* p_ : ps_) if (!aligned16(p_)) return false; return true; }())
+
+extern "C" {
+
+int seraph_fill_u32(void* dst, uint32_t value, size_t count, seraph_stream_t s) {
+    if (count == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(dst, "fill_u32: NULL dst");
+    return launch_stream(FillOp{(uint32_t*)dst, value}, count, aligned16(dst), as_stream(s));
+}
+
+int seraph_add(const float* a, const float* b, float* c, size_t n, seraph_stream_t s) {
+    if (n == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(a && b && c, "add: NULL pointer");
+    return launch_stream(AddOp{a, b, c}, n, ALL_ALIGNED(a, b, c), as_stream(s));
+}
+
+int seraph_mul(const float* a, const float* b, float* c, size_t n, seraph_stream_t s) {
+    if (n == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(a && b && c, "mul: NULL pointer");
+    return launch_stream(MulOp{a, b, c}, n, ALL_ALIGNED(a, b, c), as_stream(s));
+}
+
+int seraph_scale(float* a, size_t n, float alpha, seraph_stream_t s) {
+    if (n == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(a, "scale: NULL pointer");
+    return launch_stream(ScaleOp{a, alpha}, n, aligned16(a), as_stream(s));
+}
+
+int seraph_silu(const float* x, float* y, size_t n, seraph_stream_t s) {
+    if (n == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(x && y, "silu: NULL pointer");
+    return launch_stream(SiluOp{x, y}, n, ALL_ALIGNED(x, y), as_stream(s));
+}
+
+int seraph_silu_backward(const float* x, const float* dy, float* dx, size_t n, seraph_stream_t s) {
+    if (n == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(x && dy && dx, "silu_backward: NULL pointer");
+    return launch_stream(SiluBwdOp{x, dy, dx}, n, ALL_ALIGNED(x, dy, dx), as_stream(s));
+}
+
+int seraph_mul_backward(const float* A, const float* B, const float* dC, float* dA, float* dB, size_t n,
+                        seraph_stream_t s) {
+    if (n == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(A && B && dC && dA && dB, "mul_backward: NULL pointer");
+    return launch_stream(MulBwdOp{A, B, dC, dA, dB}, n, ALL_ALIGNED(A, B, dC, dA, dB), as_stream(s));
+}
+
+int seraph_swiglu_backward(const float* gate, const float* up, const float* dH, float* dGate, float* dUp,
+                           size_t n, seraph_stream_t s) {
+    if (n == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(gate && up && dH && dGate && dUp, "swiglu_backward: NULL pointer");
+    return launch_stream(SwigluBwdOp{gate, up, dH, dGate, dUp}, n, ALL_ALIGNED(gate, up, dH, dGate, dUp), as_stream(s));
+}
+
+int seraph_swiglu(const float* gate, const float* up, float* out, size_t n, seraph_stream_t s) {
+    if (n == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(gate && up && out, "swiglu: NULL pointer");
+    return launch_stream(SwigluOp{gate, up, out}, n, ALL_ALIGNED(gate, up, out), as_stream(s));
+}
+
+int seraph_adamw(float* w, const float* g, float* m, float* v, size_t n,
+                 float lr, float beta1, float beta2, float weight_decay, float eps, int step, float clip,
+                 seraph_stream_t s) {
+    if (n == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(w && g && m && v, "adamw: NULL pointer");
+    SERAPH_REQUIRE(step >= 1, "adamw: step must be >= 1 (got %d)", step);
+    float bc1 = 1.0f - powf(beta1, (float)step);      // src/vulkan_backend.c:2151-2152
+    float bc2 = 1.0f - powf(beta2, (float)step);
+    return launch_stream(AdamWOp{w, g, m, v, lr, beta1, beta2, weight_decay, eps, bc1, bc2, clip}, n,
+                         ALL_ALIGNED(w, g, m, v), as_stream(s));
+}
+
+int seraph_nan_check(const float* x, size_t n, uint32_t* flags, uint32_t flag_index, seraph_stream_t s) {
+    if (n == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(x && flags, "nan_check: NULL pointer");
+    int64_t want = ceil_div((int64_t)n, kBlock * 8);
+    int64_t cap = (int64_t)num_compute_units() * 16;
+    int grid = (int)(want < cap ? want : cap);
+    hipLaunchKernelGGL(nan_check_kernel, dim3(grid), dim3(kBlock), 0, as_stream(s), x, n, flags, flag_index);
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
+}
+
+int seraph_reduce_sum(const float* in, float* out, size_t count, seraph_stream_t s) {
+    if (count == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(in && out, "reduce_sum: NULL pointer");
+    size_t groups = (count + 511) / 512;
+    SERAPH_REQUIRE(groups <= 0x7fffffffu, "reduce_sum: count too large");
+    hipLaunchKernelGGL(reduce_sum_512_kernel, dim3((unsigned)groups), dim3(kBlock), 0, as_stream(s), in, out, count);
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,242 @@
+// gemm.hip - FP32 GEMM family on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32):
+//   C[M,N] (+)= op(A) * op(B)      NN = dgrad, TN(+=) = wgrad, NT = forward, TT for completeness.
+//
+// Shape of the kernel
+//   * 256 lanes = 4 wavefronts in a 2x2 grid; each wave owns TM x TN MFMA blocks of 32x32,
+//     so the workgroup tile is (64 TM) x (64 TN): 128x128 for the large backward GEMMs and
+//     64x64 when a 128x128 grid would leave most of the 256 CUs idle.
+//   * K advances 32 at a time through a double-buffered LDS stage; the next stage's global
+//     loads are issued into registers before the current stage's MFMAs and written to the
+//     other LDS buffer afterwards, so one barrier per stage is enough.
+//   * An operand keeps the orientation it has in memory.  "k-contiguous" operands
+//     (A in NN/NT, B in NT) sit in LDS as [mn][32+4]; a lane fetches four consecutive k
+//     with one 16-byte LDS read and feeds them to four successive MFMA steps.
+//     "mn-contiguous" operands (A in TN, B in NN/TN) sit as [k][tile+4] and are fetched
+//     four bytes at a time, 32 consecutive lanes on 32 consecutive addresses.  Within a
+//     step the two half-waves supply k = 4h+s and both operands use that same mapping,
+//     so no transpose is ever materialised.
+//   * Workgroup ids are first regrouped per XCD (ids are dealt round-robin to the 8 XCDs,
+//     each with a private L2), then walked in bands 8 tiles tall so the tiles an XCD holds
+//     at one time share operand panels in its L2.
+// Accumulator layout of the 32x32x2 instruction: lane l, register v holds
+//   row 8*(v/4) + 4*(l/32) + v%4, column l%32.
+#include "common.hpp"
+
+namespace seraph {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kBK = 32;                 // K extent of one LDS stage
+constexpr int kPadK = 4;                // [mn][kBK + kPadK]: 16-byte reads of 8 lanes fall on distinct banks
+constexpr int kPadM = 4;                // [k][tile + kPadM]
+constexpr int kGemmThreads = 256;
+constexpr int kGroupM = 8;
+
+__device__ __forceinline__ int xcd_regroup(int bid, int total) {
+    // Contiguous range of logical ids per XCD; a bijection on [0,total) for any total.
+    const int per = (total + kNumXcd - 1) / kNumXcd;
+    int tall = total % kNumXcd;
+    if (tall == 0) tall = kNumXcd;
+    const int xcd = bid % kNumXcd, local = bid / kNumXcd;
+    return xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+}
+
+// One operand tile (TILE rows of mn, kBK of k) from global memory into registers.
+// KC: the operand is stored [mn_total, K] (k contiguous); otherwise [K, mn_total].
+template <int TILE, bool KC, bool VEC>
+struct TileLoader {
+    static constexpr int kSlots = TILE * kBK / 4 / kGemmThreads;      // float4 slots per lane
+    float4 r[kSlots];
+
+    __device__ __forceinline__ void load(const float* __restrict__ P, int64_t ld, int64_t mn0, int64_t mn_total,
+                                         int64_t k0, int64_t K) {
+#pragma unroll
+        for (int u = 0; u < kSlots; u++) {
+            const int f = threadIdx.x + kGemmThreads * u;
+            int64_t mn, k;
+            if (KC) { mn = mn0 + f / (kBK / 4); k = k0 + 4 * (f % (kBK / 4)); }
+            else    { k = k0 + f / (TILE / 4);  mn = mn0 + 4 * (f % (TILE / 4)); }
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (VEC) {
+                // ld % 4 == 0 and both origins are multiples of 4: a slot is wholly inside or wholly outside
+                if (mn < mn_total && k < K)
+                    v = *reinterpret_cast<const float4*>(P + (KC ? mn * ld + k : k * ld + mn));
+            } else {
+                float* e = &v.x;
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    int64_t mq = KC ? mn : mn + q, kq = KC ? k + q : k;
+                    if (mq < mn_total && kq < K) e[q] = P[KC ? mq * ld + kq : kq * ld + mq];
+                }
+            }
+            r[u] = v;
+        }
+    }
+
+    __device__ __forceinline__ void store(float* __restrict__ lds) const {
+#pragma unroll
+        for (int u = 0; u < kSlots; u++) {
+            const int f = threadIdx.x + kGemmThreads * u;
+            int off;
+            if (KC) off = (f / (kBK / 4)) * (kBK + kPadK) + 4 * (f % (kBK / 4));
+            else    off = (f / (TILE / 4)) * (TILE + kPadM) + 4 * (f % (TILE / 4));
+            *reinterpret_cast<float4*>(lds + off) = r[u];
+        }
+    }
+};
+
+template <int TILE, bool KC>
+constexpr int lds_floats() { return KC ? TILE * (kBK + kPadK) : kBK * (TILE + kPadM); }
+
+template <int TM, int TN, bool A_KC, bool B_KC, bool VEC>
+__global__ __launch_bounds__(kGemmThreads) void gemm_f32_mfma_kernel(const float* __restrict__ A,
+                                                                     const float* __restrict__ B,
+                                                                     float* __restrict__ C,
+                                                                     int64_t M, int64_t N, int64_t K,
+                                                                     int accumulate, int nbm, int nbn) {
+    constexpr int BM = 64 * TM, BN = 64 * TN;
+    constexpr int A_FLOATS = lds_floats<BM, A_KC>(), B_FLOATS = lds_floats<BN, B_KC>();
+    __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
+    __shared__ __attribute__((aligned(16))) float lds_b[2][B_FLOATS];
+
+    // ---- tile assignment
+    const int total = nbm * nbn;
+    const int pid = xcd_regroup(blockIdx.x, total);
+    const int width = kGroupM * nbn;
+    const int group = pid / width;
+    const int first_m = group * kGroupM;
+    const int gsize = (nbm - first_m) < kGroupM ? (nbm - first_m) : kGroupM;
+    const int pm = first_m + (pid % width) % gsize;
+    const int pn = (pid % width) / gsize;
+    const int64_t m0 = (int64_t)pm * BM, n0 = (int64_t)pn * BN;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int wm0 = (wave >> 1) * (32 * TM), wn0 = (wave & 1) * (32 * TN);
+
+    const int64_t lda = A_KC ? K : M, ldb = B_KC ? K : N;
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    TileLoader<BM, A_KC, VEC> la;
+    TileLoader<BN, B_KC, VEC> lb;
+    const int nk = (int)((K + kBK - 1) / kBK);
+
+    la.load(A, lda, m0, M, 0, K);
+    lb.load(B, ldb, n0, N, 0, K);
+    la.store(lds_a[0]);
+    lb.store(lds_b[0]);
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; kt++) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) {
+            la.load(A, lda, m0, M, (int64_t)(kt + 1) * kBK, K);
+            lb.load(B, ldb, n0, N, (int64_t)(kt + 1) * kBK, K);
+        }
+        const float* sa = lds_a[cur];
+        const float* sb = lds_b[cur];
+#pragma unroll
+        for (int slab = 0; slab < kBK / 8; slab++) {
+            float fa[TM][4], fb[TN][4];
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                if (A_KC) {
+                    const float4 t = *reinterpret_cast<const float4*>(sa + (wm0 + 32 * i + r) * (kBK + kPadK) + slab * 8 + 4 * h);
+                    fa[i][0] = t.x; fa[i][1] = t.y; fa[i][2] = t.z; fa[i][3] = t.w;
+                } else {
+#pragma unroll
+                    for (int s = 0; s < 4; s++) fa[i][s] = sa[(slab * 8 + 4 * h + s) * (BM + kPadM) + wm0 + 32 * i + r];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                if (B_KC) {
+                    const float4 t = *reinterpret_cast<const float4*>(sb + (wn0 + 32 * j + r) * (kBK + kPadK) + slab * 8 + 4 * h);
+                    fb[j][0] = t.x; fb[j][1] = t.y; fb[j][2] = t.z; fb[j][3] = t.w;
+                } else {
+#pragma unroll
+                    for (int s = 0; s < 4; s++) fb[j][s] = sb[(slab * 8 + 4 * h + s) * (BN + kPadM) + wn0 + 32 * j + r];
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) {
+            la.store(lds_a[cur ^ 1]);
+            lb.store(lds_b[cur ^ 1]);
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int64_t col = n0 + wn0 + 32 * j + r;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int64_t row = m0 + wm0 + 32 * i + 8 * (v >> 2) + 4 * h + (v & 3);
+                if (row < M && col < N) {
+                    float* dst = C + row * N + col;
+                    *dst = accumulate ? *dst + acc[i][j][v] : acc[i][j][v];
+                }
+            }
+        }
+}
+
+template <int TM, int TN>
+static int launch_gemm(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
+                       int tA, int tB, int accumulate, bool vec, hipStream_t st) {
+    const int64_t nbm = ceil_div(M, 64 * TM), nbn = ceil_div(N, 64 * TN);
+    SERAPH_REQUIRE(nbm * nbn <= 0x7fffffff, "gemm: too many tiles");
+    const dim3 grid((unsigned)(nbm * nbn)), block(kGemmThreads);
+#define GO(AKC, BKC, V) \
+    hipLaunchKernelGGL((gemm_f32_mfma_kernel<TM, TN, AKC, BKC, V>), grid, block, 0, st, A, B, C, M, N, K, accumulate, (int)nbm, (int)nbn)
+    // A is k-contiguous unless transposed; B is k-contiguous when transposed.
+    if (vec) {
+        if (!tA && !tB) GO(true, false, true);
+        else if (!tA && tB) GO(true, true, true);
+        else if (tA && !tB) GO(false, false, true);
+        else GO(false, true, true);
+    } else {
+        if (!tA && !tB) GO(true, false, false);
+        else if (!tA && tB) GO(true, true, false);
+        else if (tA && !tB) GO(false, false, false);
+        else GO(false, true, false);
+    }
+#undef GO
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
+}
+
+}  // namespace seraph
+
+using namespace seraph;
+
+extern "C" int seraph_gemm(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
+                           int transpose_A, int transpose_B, int accumulate, seraph_stream_t s) {
+    if (M == 0 || N == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(A && B && C, "gemm: NULL pointer");
+    SERAPH_REQUIRE(M > 0 && N > 0 && K >= 0, "gemm: bad shape %lld x %lld x %lld", (long long)M, (long long)N, (long long)K);
+    const int64_t lda = transpose_A ? M : K, ldb = transpose_B ? K : N;
+    const bool vec = (lda % 4 == 0) && (ldb % 4 == 0) && aligned16(A) && aligned16(B);
+    hipStream_t st = as_stream(s);
+    // 128x128 tiles when they fill the machine at least once, else 64x64.
+    const int64_t big_tiles = ceil_div(M, 128) * ceil_div(N, 128);
+    if (big_tiles >= num_compute_units())
+        return launch_gemm<2, 2>(A, B, C, M, N, K, transpose_A, transpose_B, accumulate, vec, st);
+    return launch_gemm<1, 1>(A, B, C, M, N, K, transpose_A, transpose_B, accumulate, vec, st);
+}

@@ -1,0 +1,361 @@
+// rmsnorm.hip - RMSNorm forward, batched RMSNorm backward with FP64 intermediates,
+// and the gain-less all-heads qk_norm with its derivative.
+//
+// One wavefront owns one row: the row (and, going backward, dy) lives in registers as
+// float4 slots, the two row sums are wave reductions (no LDS, no barrier), and each
+// byte of x / dy / dx crosses HBM exactly once.  The column reduction for grad_scale is
+// deterministic: lanes keep per-column partial sums over the rows their wave visits,
+// the block's four waves are combined through LDS, each block writes one partial row
+// to scratch, and a second small kernel adds the partial rows in a fixed order.
+#include "common.hpp"
+
+namespace seraph {
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+
+// ---------------------------------------------------------------- forward
+template <int VPL>
+__global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const float* __restrict__ x,
+                                                             const float* __restrict__ scale,
+                                                             float* __restrict__ y,
+                                                             int64_t rows, int cols, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+    const int n4 = cols >> 2;
+    float4 sc[VPL];
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+        int i4 = lane + 64 * k;
+        sc[k] = i4 < n4 ? reinterpret_cast<const float4*>(scale)[i4] : make_float4(0, 0, 0, 0);
+    }
+    for (int64_t row = wave; row < rows; row += nwaves) {
+        const float4* xr = reinterpret_cast<const float4*>(x + row * cols);
+        float4 v[VPL];
+        float ss = 0.0f;
+#pragma unroll
+        for (int k = 0; k < VPL; k++) {
+            int i4 = lane + 64 * k;
+            v[k] = i4 < n4 ? xr[i4] : make_float4(0, 0, 0, 0);
+            ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+        }
+        ss = wave_sum(ss);
+        float inv = rsqrtf(ss / (float)cols + eps);       // shaders/rmsnorm.comp: inversesqrt(mean_sq + eps)
+        float4* yr = reinterpret_cast<float4*>(y + row * cols);
+#pragma unroll
+        for (int k = 0; k < VPL; k++) {
+            int i4 = lane + 64 * k;
+            if (i4 < n4)
+                yr[i4] = make_float4(v[k].x * inv * sc[k].x, v[k].y * inv * sc[k].y,
+                                     v[k].z * inv * sc[k].z, v[k].w * inv * sc[k].w);
+        }
+    }
+}
+
+// Any cols / alignment: the row is read twice (the second read is served by cache).
+__global__ __launch_bounds__(kBlock) void rmsnorm_fwd_generic_kernel(const float* __restrict__ x,
+                                                                     const float* __restrict__ scale,
+                                                                     float* __restrict__ y,
+                                                                     int64_t rows, int64_t cols, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+    for (int64_t row = wave; row < rows; row += nwaves) {
+        const float* xr = x + row * cols;
+        float ss = 0.0f;
+        for (int64_t c = lane; c < cols; c += 64) ss += xr[c] * xr[c];
+        ss = wave_sum(ss);
+        float inv = rsqrtf(ss / (float)cols + eps);
+        for (int64_t c = lane; c < cols; c += 64) y[row * cols + c] = xr[c] * inv * scale[c];
+    }
+}
+
+// ---------------------------------------------------------------- backward
+// Row statistics of shaders/rmsnorm_backward_batch.comp:44-79 in double.
+struct RowStats { double inv, k; };     // 1/rms and coupled/rms^3
+__device__ __forceinline__ RowStats row_stats(double ssq, double cp, int64_t cols, float eps) {
+    double denom = cols > 1 ? (double)cols : 1.0;         // max(1.0, cols)
+    double rms = sqrt(ssq / denom + (double)eps);
+    rms = fmax(rms, 0.01);                                // floor, :59
+    double inv = 1.0 / rms;
+    RowStats r;
+    r.inv = inv;
+    r.k = (cp / denom) * (inv * inv * inv);               // coupled * inv_rms3, :79,:98
+    return r;
+}
+
+template <int VPL>
+__global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const float* __restrict__ x,
+                                                             const float* __restrict__ scale,
+                                                             const float* __restrict__ dy,
+                                                             float* __restrict__ dx,
+                                                             float* __restrict__ partial,   // [gridDim.x, cols]
+                                                             int64_t rows, int cols, float eps) {
+    extern __shared__ float lds[];                        // [kWavesPerBlock, cols]
+    const int lane = threadIdx.x & 63;
+    const int wv = threadIdx.x >> 6;
+    const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + wv;
+    const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+    const int n4 = cols >> 2;
+
+    float4 sc[VPL], gs[VPL];
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+        int i4 = lane + 64 * k;
+        sc[k] = i4 < n4 ? reinterpret_cast<const float4*>(scale)[i4] : make_float4(0, 0, 0, 0);
+        gs[k] = make_float4(0, 0, 0, 0);
+    }
+
+    for (int64_t row = wave; row < rows; row += nwaves) {
+        const float4* xr = reinterpret_cast<const float4*>(x + row * cols);
+        const float4* gr = reinterpret_cast<const float4*>(dy + row * cols);
+        float4 xv[VPL], gv[VPL];
+#pragma unroll
+        for (int k = 0; k < VPL; k++) {
+            int i4 = lane + 64 * k;
+            xv[k] = i4 < n4 ? xr[i4] : make_float4(0, 0, 0, 0);
+            gv[k] = i4 < n4 ? gr[i4] : make_float4(0, 0, 0, 0);
+        }
+        double ssq = 0.0, cp = 0.0;
+#pragma unroll
+        for (int k = 0; k < VPL; k++) {
+            const float* xs = &xv[k].x; const float* g = &gv[k].x; const float* s = &sc[k].x;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                double xd = (double)xs[e];
+                ssq += xd * xd;
+                cp += (double)g[e] * (double)s[e] * xd;
+            }
+        }
+        ssq = wave_sum(ssq);
+        cp = wave_sum(cp);
+        RowStats st = row_stats(ssq, cp, cols, eps);
+        float4* dr = reinterpret_cast<float4*>(dx + row * cols);
+#pragma unroll
+        for (int k = 0; k < VPL; k++) {
+            int i4 = lane + 64 * k;
+            const float* xs = &xv[k].x; const float* g = &gv[k].x; const float* s = &sc[k].x;
+            float o[4]; float* acc = &gs[k].x;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                double xd = (double)xs[e], gd = (double)g[e];
+                acc[e] += (float)(gd * xd * st.inv);                                 // :90
+                o[e] = (float)(gd * (double)s[e] * st.inv - xd * st.k);              // :98
+            }
+            if (i4 < n4) dr[i4] = make_float4(o[0], o[1], o[2], o[3]);
+        }
+    }
+
+    // combine the block's waves, then one partial row per block
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+        int i4 = lane + 64 * k;
+        if (i4 < n4) reinterpret_cast<float4*>(lds + (size_t)wv * cols)[i4] = gs[k];
+    }
+    __syncthreads();
+    for (int i4 = threadIdx.x; i4 < n4; i4 += kBlock) {
+        float4 a = reinterpret_cast<float4*>(lds)[i4];
+#pragma unroll
+        for (int w = 1; w < kWavesPerBlock; w++) {
+            float4 b = reinterpret_cast<float4*>(lds + (size_t)w * cols)[i4];
+            a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+        }
+        reinterpret_cast<float4*>(partial + (size_t)blockIdx.x * cols)[i4] = a;
+    }
+}
+
+// Generic shape: one wave per row, scalar accesses, per-wave partial rows in scratch.
+__global__ __launch_bounds__(kBlock) void rmsnorm_bwd_generic_kernel(const float* __restrict__ x,
+                                                                     const float* __restrict__ scale,
+                                                                     const float* __restrict__ dy,
+                                                                     float* __restrict__ dx,
+                                                                     float* __restrict__ partial,   // [nwaves, cols], zeroed
+                                                                     int64_t rows, int64_t cols, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+    float* mine = partial + wave * cols;
+    for (int64_t row = wave; row < rows; row += nwaves) {
+        const float* xr = x + row * cols;
+        const float* gr = dy + row * cols;
+        double ssq = 0.0, cp = 0.0;
+        for (int64_t c = lane; c < cols; c += 64) {
+            double xd = (double)xr[c];
+            ssq += xd * xd;
+            cp += (double)gr[c] * (double)scale[c] * xd;
+        }
+        ssq = wave_sum(ssq);
+        cp = wave_sum(cp);
+        RowStats st = row_stats(ssq, cp, cols, eps);
+        for (int64_t c = lane; c < cols; c += 64) {
+            double xd = (double)xr[c], gd = (double)gr[c];
+            mine[c] += (float)(gd * xd * st.inv);          // same lane revisits the same column: no race
+            dx[row * cols + c] = (float)(gd * (double)scale[c] * st.inv - xd * st.k);
+        }
+    }
+}
+
+// grad_scale[c] += sum over partial rows, fixed order, double accumulator
+__global__ __launch_bounds__(kBlock) void colsum_add_kernel(const float* __restrict__ partial, int nparts,
+                                                            int64_t cols, float* __restrict__ grad_scale) {
+    int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (c >= cols) return;
+    double s = 0.0;
+    for (int p = 0; p < nparts; p++) s += (double)partial[(size_t)p * cols + c];
+    grad_scale[c] = (float)((double)grad_scale[c] + s);
+}
+
+// ---------------------------------------------------------------- qk_norm
+// shaders/qk_norm.comp:38-75: y = x / max(sqrt(mean(x^2)), eps) over all heads of a token.
+__global__ __launch_bounds__(kBlock) void qk_norm_kernel(float* __restrict__ qk, int64_t T, int64_t n, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+    for (int64_t t = wave; t < T; t += nwaves) {
+        float* xr = qk + t * n;
+        float ss = 0.0f;
+        for (int64_t c = lane; c < n; c += 64) ss += xr[c] * xr[c];
+        ss = wave_sum(ss);
+        float rms = fmaxf(sqrtf(ss / (float)n), eps);
+        float inv = 1.0f / rms;
+        for (int64_t c = lane; c < n; c += 64) xr[c] *= inv;
+    }
+}
+
+// d/dx of the above: dx = dy/r - x (dy.x)/(n r^3) while r = rms > eps; dx = dy/eps when clamped.
+__global__ __launch_bounds__(kBlock) void qk_norm_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+                                                             float* __restrict__ dx, int64_t T, int64_t n, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+    for (int64_t t = wave; t < T; t += nwaves) {
+        const float* xr = x + t * n;
+        const float* gr = dy + t * n;
+        float ss = 0.0f, gx = 0.0f;
+        for (int64_t c = lane; c < n; c += 64) { ss += xr[c] * xr[c]; gx += gr[c] * xr[c]; }
+        ss = wave_sum(ss);
+        gx = wave_sum(gx);
+        float rms = sqrtf(ss / (float)n);
+        if (rms < eps) {
+            float inv = 1.0f / eps;
+            for (int64_t c = lane; c < n; c += 64) dx[t * n + c] = gr[c] * inv;
+        } else {
+            float inv = 1.0f / rms;
+            float k = gx / ((float)n * rms * rms * rms);
+            for (int64_t c = lane; c < n; c += 64) dx[t * n + c] = gr[c] * inv - xr[c] * k;
+        }
+    }
+}
+
+// ---------------------------------------------------------------- host side
+static int pick_vpl(int64_t cols) {
+    if (cols % 4 != 0) return 0;
+    int64_t n4 = cols / 4;
+    for (int v = 1; v <= 16; v *= 2) if (n4 <= 64 * v) return v;
+    return 0;
+}
+
+static int bwd_grid(int64_t rows) {
+    int64_t want = ceil_div(rows, kWavesPerBlock * 2);          // at least two rows per wave
+    int64_t cap = (int64_t)num_compute_units() * 3;
+    if (want < 1) want = 1;
+    return (int)(want < cap ? want : cap);
+}
+
+}  // namespace seraph
+
+using namespace seraph;
+
+extern "C" {
+
+int seraph_rmsnorm(const float* x, const float* scale, float* y, int64_t rows, int64_t cols, float eps,
+                   seraph_stream_t s) {
+    if (rows == 0 || cols == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(x && scale && y, "rmsnorm: NULL pointer");
+    SERAPH_REQUIRE(rows > 0 && cols > 0, "rmsnorm: bad shape %lld x %lld", (long long)rows, (long long)cols);
+    int64_t want = ceil_div(rows, kWavesPerBlock);
+    int64_t cap = (int64_t)num_compute_units() * 8;
+    int grid = (int)(want < cap ? want : cap);
+    int vpl = (aligned16(x) && aligned16(scale) && aligned16(y)) ? pick_vpl(cols) : 0;
+    hipStream_t st = as_stream(s);
+#define FWD(V) hipLaunchKernelGGL(rmsnorm_fwd_kernel<V>, dim3(grid), dim3(kBlock), 0, st, x, scale, y, rows, (int)cols, eps)
+    switch (vpl) {
+        case 1: FWD(1); break;
+        case 2: FWD(2); break;
+        case 4: FWD(4); break;
+        case 8: FWD(8); break;
+        case 16: FWD(16); break;
+        default:
+            hipLaunchKernelGGL(rmsnorm_fwd_generic_kernel, dim3(grid), dim3(kBlock), 0, st, x, scale, y, rows, cols, eps);
+    }
+#undef FWD
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
+}
+
+size_t seraph_rmsnorm_backward_ws_bytes(int64_t rows, int64_t cols) {
+    if (rows <= 0 || cols <= 0) return 0;
+    // the generic path needs one partial row per wave, the register path one per block
+    return (size_t)bwd_grid(rows) * kWavesPerBlock * (size_t)cols * sizeof(float);
+}
+
+int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy, float* dx, float* grad_scale,
+                            int64_t rows, int64_t cols, float eps, void* ws, size_t ws_bytes, seraph_stream_t s) {
+    if (rows == 0 || cols == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(x && scale && dy && dx && grad_scale, "rmsnorm_backward: NULL pointer");
+    SERAPH_REQUIRE(rows > 0 && cols > 0, "rmsnorm_backward: bad shape");
+    if (!ws || ws_bytes < seraph_rmsnorm_backward_ws_bytes(rows, cols)) {
+        set_error("rmsnorm_backward: scratch of %zu bytes required", seraph_rmsnorm_backward_ws_bytes(rows, cols));
+        return SERAPH_ERR_WORKSPACE;
+    }
+    hipStream_t st = as_stream(s);
+    int grid = bwd_grid(rows);
+    float* partial = (float*)ws;
+    int vpl = (aligned16(x) && aligned16(scale) && aligned16(dy) && aligned16(dx) && aligned16(ws)) ? pick_vpl(cols) : 0;
+    size_t lds = (size_t)kWavesPerBlock * cols * sizeof(float);
+    int nparts;
+#define BWD(V) hipLaunchKernelGGL(rmsnorm_bwd_kernel<V>, dim3(grid), dim3(kBlock), lds, st, x, scale, dy, dx, partial, rows, (int)cols, eps)
+    switch (vpl) {
+        case 1: BWD(1); nparts = grid; break;
+        case 2: BWD(2); nparts = grid; break;
+        case 4: BWD(4); nparts = grid; break;
+        case 8: BWD(8); nparts = grid; break;
+        case 16: BWD(16); nparts = grid; break;
+        default: {
+            nparts = grid * kWavesPerBlock;
+            int rc = seraph_fill_u32(partial, 0u, (size_t)nparts * cols, s);
+            if (rc != SERAPH_OK) return rc;
+            hipLaunchKernelGGL(rmsnorm_bwd_generic_kernel, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, dx, partial, rows, cols, eps);
+        }
+    }
+#undef BWD
+    SERAPH_LAUNCH_CHECK();
+    hipLaunchKernelGGL(colsum_add_kernel, dim3((unsigned)ceil_div(cols, kBlock)), dim3(kBlock), 0, st,
+                       partial, nparts, cols, grad_scale);
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
+}
+
+int seraph_qk_norm(float* qk, int64_t T, int heads, int head_dim, int use_qk_norm, float eps, seraph_stream_t s) {
+    if (!use_qk_norm || T == 0) return SERAPH_OK;                 // shaders/qk_norm.comp:32
+    SERAPH_REQUIRE(qk && heads > 0 && head_dim > 0, "qk_norm: bad argument");
+    int64_t want = ceil_div(T, kWavesPerBlock), cap = (int64_t)num_compute_units() * 8;
+    hipLaunchKernelGGL(qk_norm_kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(kBlock), 0, as_stream(s),
+                       qk, T, (int64_t)heads * head_dim, eps);
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
+}
+
+int seraph_qk_norm_backward(const float* x_pre, const float* dy, float* dx, int64_t T, int heads, int head_dim,
+                            float eps, seraph_stream_t s) {
+    if (T == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(x_pre && dy && dx && heads > 0 && head_dim > 0, "qk_norm_backward: bad argument");
+    int64_t want = ceil_div(T, kWavesPerBlock), cap = (int64_t)num_compute_units() * 8;
+    hipLaunchKernelGGL(qk_norm_bwd_kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(kBlock), 0, as_stream(s),
+                       x_pre, dy, dx, T, (int64_t)heads * head_dim, eps);
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
+}
+
+}  // extern "C"

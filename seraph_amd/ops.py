@@ -1,0 +1,211 @@
+"""Thin Python mirror of the C-ABI kernel library over torch CUDA tensors.
+
+torch supplies device memory and the stream only; every computation goes through
+libseraph_hip.so.  Names and argument meaning follow the backend ops of the reference
+(include/vulkan_backend.h:431-603), with the packed-batch arguments of
+include/cuda_train_context.h:273-288 where they apply.
+"""
+import ctypes as C
+
+import torch
+
+from ._lib import check, kernels
+
+i64, f32, sz = C.c_int64, C.c_float, C.c_size_t
+
+
+def _p(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "expected a contiguous CUDA tensor"
+    return C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+_ws = {}
+
+
+def _workspace(nbytes):
+    dev = torch.cuda.current_device()
+    t = _ws.get(dev)
+    if t is None or t.numel() < nbytes:
+        t = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device="cuda")
+        _ws[dev] = t
+    return t
+
+
+def init(device=0):
+    check(kernels().seraph_hip_init(C.c_int(device)), "seraph_hip_init")
+
+
+def _batch(seq_starts):
+    return 1 if seq_starts is None else seq_starts.numel() - 1
+
+
+def fill_u32(t, value):
+    check(kernels().seraph_fill_u32(_p(t), C.c_uint32(value), sz(t.numel()), _stream()), "fill_u32")
+
+
+def add(a, b, out):
+    check(kernels().seraph_add(_p(a), _p(b), _p(out), sz(a.numel()), _stream()), "add")
+    return out
+
+
+def mul(a, b, out):
+    check(kernels().seraph_mul(_p(a), _p(b), _p(out), sz(a.numel()), _stream()), "mul")
+    return out
+
+
+def scale_(a, alpha):
+    check(kernels().seraph_scale(_p(a), sz(a.numel()), f32(alpha), _stream()), "scale")
+    return a
+
+
+def nan_check(x, flags, flag_index):
+    check(kernels().seraph_nan_check(_p(x), sz(x.numel()), _p(flags), C.c_uint32(flag_index), _stream()), "nan_check")
+
+
+def reduce_sum(x):
+    out = torch.empty((x.numel() + 511) // 512, dtype=torch.float32, device=x.device)
+    check(kernels().seraph_reduce_sum(_p(x), _p(out), sz(x.numel()), _stream()), "reduce_sum")
+    return out
+
+
+def cross_entropy_grad(logits, targets, valid_rows, seq_starts=None, grad=None):
+    rows, cols = logits.shape
+    grad = torch.empty_like(logits) if grad is None else grad
+    loss = torch.empty(rows, dtype=torch.float32, device=logits.device)
+    check(kernels().seraph_cross_entropy_grad(_p(logits), _p(targets), _p(grad), _p(loss), _p(seq_starts),
+                                              C.c_int(_batch(seq_starts)), i64(rows), i64(cols), i64(valid_rows),
+                                              _stream()), "cross_entropy_grad")
+    return grad, loss
+
+
+def gemm(A, B, M, N, K, tA=0, tB=0, out=None, accumulate=False):
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=A.device)
+    check(kernels().seraph_gemm(_p(A), _p(B), _p(out), i64(M), i64(N), i64(K), C.c_int(tA), C.c_int(tB),
+                                C.c_int(1 if accumulate else 0), _stream()), "gemm")
+    return out
+
+
+def attention_forward(Q, K, V, heads, kv_heads, head_dim, seq_starts=None, scale=None, want_lse=True):
+    T = Q.shape[0]
+    out = torch.empty_like(Q)
+    lse = torch.empty((T, heads), dtype=torch.float32, device=Q.device) if want_lse else None
+    scale = head_dim ** -0.5 if scale is None else scale
+    check(kernels().seraph_attention_forward(_p(Q), _p(K), _p(V), _p(out), _p(lse), _p(seq_starts),
+                                             C.c_int(_batch(seq_starts)), i64(T), C.c_int(heads), C.c_int(kv_heads),
+                                             C.c_int(head_dim), f32(scale), _stream()), "attention_forward")
+    return out, lse
+
+
+def attention_backward(Q, K, V, dO, heads, kv_heads, head_dim, seq_starts=None, scale=None, out=None, lse=None,
+                       dK=None, dV=None):
+    T = Q.shape[0]
+    dQ = torch.empty_like(Q)
+    dK = torch.zeros_like(K) if dK is None else dK
+    dV = torch.zeros_like(V) if dV is None else dV
+    scale = head_dim ** -0.5 if scale is None else scale
+    nbytes = kernels().seraph_attention_backward_ws_bytes(i64(T), C.c_int(heads), C.c_int(kv_heads), C.c_int(head_dim))
+    ws = _workspace(nbytes)
+    check(kernels().seraph_attention_backward(_p(Q), _p(K), _p(V), _p(dO), _p(out), _p(lse), _p(dQ), _p(dK), _p(dV),
+                                              _p(seq_starts), C.c_int(_batch(seq_starts)), i64(T), C.c_int(heads),
+                                              C.c_int(kv_heads), C.c_int(head_dim), f32(scale), _p(ws), sz(nbytes),
+                                              _stream()), "attention_backward")
+    return dQ, dK, dV
+
+
+def rmsnorm(x, scale, eps):
+    y = torch.empty_like(x)
+    check(kernels().seraph_rmsnorm(_p(x), _p(scale), _p(y), i64(x.shape[0]), i64(x.shape[1]), f32(eps), _stream()),
+          "rmsnorm")
+    return y
+
+
+def rmsnorm_backward(x, scale, dy, eps, grad_scale=None):
+    dx = torch.empty_like(x)
+    gs = torch.zeros_like(scale) if grad_scale is None else grad_scale
+    rows, cols = x.shape
+    nbytes = kernels().seraph_rmsnorm_backward_ws_bytes(i64(rows), i64(cols))
+    ws = _workspace(nbytes)
+    check(kernels().seraph_rmsnorm_backward(_p(x), _p(scale), _p(dy), _p(dx), _p(gs), i64(rows), i64(cols), f32(eps),
+                                            _p(ws), sz(nbytes), _stream()), "rmsnorm_backward")
+    return dx, gs
+
+
+def rope(x, heads, head_dim, theta, seq_starts=None, backward=False, out=None):
+    out = torch.empty_like(x) if out is None else out
+    check(kernels().seraph_rope(_p(x), _p(out), _p(seq_starts), C.c_int(_batch(seq_starts)), i64(x.shape[0]),
+                                C.c_int(heads), C.c_int(head_dim), f32(theta), C.c_int(1 if backward else 0),
+                                _stream()), "rope")
+    return out
+
+
+def qk_norm_(x, heads, head_dim, eps, use_qk_norm=1):
+    check(kernels().seraph_qk_norm(_p(x), i64(x.shape[0]), C.c_int(heads), C.c_int(head_dim), C.c_int(use_qk_norm),
+                                   f32(eps), _stream()), "qk_norm")
+    return x
+
+
+def qk_norm_backward(x_pre, dy, heads, head_dim, eps):
+    dx = torch.empty_like(x_pre)
+    check(kernels().seraph_qk_norm_backward(_p(x_pre), _p(dy), _p(dx), i64(x_pre.shape[0]), C.c_int(heads),
+                                            C.c_int(head_dim), f32(eps), _stream()), "qk_norm_backward")
+    return dx
+
+
+def silu(x):
+    y = torch.empty_like(x)
+    check(kernels().seraph_silu(_p(x), _p(y), sz(x.numel()), _stream()), "silu")
+    return y
+
+
+def silu_backward(x, dy, out=None):
+    dx = torch.empty_like(x) if out is None else out
+    check(kernels().seraph_silu_backward(_p(x), _p(dy), _p(dx), sz(x.numel()), _stream()), "silu_backward")
+    return dx
+
+
+def mul_backward(A, B, dC):
+    dA, dB = torch.empty_like(A), torch.empty_like(A)
+    check(kernels().seraph_mul_backward(_p(A), _p(B), _p(dC), _p(dA), _p(dB), sz(A.numel()), _stream()), "mul_backward")
+    return dA, dB
+
+
+def swiglu_backward(gate, up, dH):
+    dG, dU = torch.empty_like(gate), torch.empty_like(gate)
+    check(kernels().seraph_swiglu_backward(_p(gate), _p(up), _p(dH), _p(dG), _p(dU), sz(gate.numel()), _stream()),
+          "swiglu_backward")
+    return dG, dU
+
+
+def swiglu(gate, up):
+    out = torch.empty_like(gate)
+    check(kernels().seraph_swiglu(_p(gate), _p(up), _p(out), sz(gate.numel()), _stream()), "swiglu")
+    return out
+
+
+def embed_lookup(tokens, embed):
+    T, (V, h) = tokens.numel(), embed.shape
+    out = torch.empty((T, h), dtype=torch.float32, device=embed.device)
+    check(kernels().seraph_embed_lookup(_p(tokens), _p(embed), _p(out), i64(T), i64(h), i64(V), _stream()), "embed_lookup")
+    return out
+
+
+def embedding_backward(tokens, dH, grad_embed):
+    T, (V, h) = tokens.numel(), grad_embed.shape
+    nbytes = kernels().seraph_embedding_backward_ws_bytes(i64(T), i64(V))
+    ws = _workspace(nbytes)
+    check(kernels().seraph_embedding_backward(_p(tokens), _p(dH), _p(grad_embed), i64(T), i64(h), i64(V), _p(ws),
+                                              sz(nbytes), _stream()), "embedding_backward")
+    return grad_embed
+
+
+def adamw_(w, g, m, v, lr, beta1, beta2, weight_decay, eps, step, clip=0.0):
+    check(kernels().seraph_adamw(_p(w), _p(g), _p(m), _p(v), sz(w.numel()), f32(lr), f32(beta1), f32(beta2),
+                                 f32(weight_decay), f32(eps), C.c_int(step), f32(clip), _stream()), "adamw")
+    return w, m, v

@@ -1,0 +1,325 @@
+"""Parity of every HIP op against the CPU oracle, through the C ABI, on the same seeded
+inputs.  Bar: bit-exact for token / index handling and the set of embedding rows
+touched; |got - ref| <= 1e-5 + 1e-4 |ref| element-wise for FP32 results."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-4, 1e-5
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from seraph_amd import ops as o
+    o.init(0)
+    return o
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def parity(got, ref, what="", rtol=RTOL, atol=ATOL):
+    got = np.asarray(host(got) if isinstance(got, torch.Tensor) else got, np.float64)
+    ref = np.asarray(ref, np.float64)
+    assert got.shape == ref.shape, (what, got.shape, ref.shape)
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    err = np.abs(got - ref)
+    bad = err > atol + rtol * np.abs(ref)
+    if bad.any():
+        i = np.unravel_index(np.argmax(err - rtol * np.abs(ref)), err.shape)
+        raise AssertionError(f"{what}: {bad.sum()} of {bad.size} outside tolerance; worst at {i}: "
+                             f"got {got[i]:.8g} ref {ref[i]:.8g}; rel-L2 {np.linalg.norm(got - ref) / (np.linalg.norm(ref) + 1e-30):.3e}")
+
+
+# ------------------------------------------------------------------ element-wise
+@pytest.mark.parametrize("n", [1, 3, 1023, 4096, 100003])
+def test_elementwise_family(ops, orc, n):
+    r = rng(n)
+    a, b, g = (3 * r.standard_normal(n).astype(np.float32) for _ in range(3))
+    A, B, G = dev(a), dev(b), dev(g)
+    assert (host(ops.add(A, B, torch.empty_like(A))) == a + b).all()
+    assert (host(ops.mul(A, B, torch.empty_like(A))) == a * b).all()
+    assert (host(ops.scale_(A.clone(), 0.37)) == a * np.float32(0.37)).all()
+    parity(ops.silu(A), orc.silu(a), "silu")
+    parity(ops.silu_backward(A, G), orc.silu_backward(a, g), "silu_backward")
+    dA, dB = ops.mul_backward(A, B, G)
+    ra, rb = orc.mul_backward(a, b, g)
+    assert (host(dA) == ra).all() and (host(dB) == rb).all()
+    dG, dU = ops.swiglu_backward(A, B, G)
+    rg, ru = orc.swiglu_backward(a, b, g)
+    parity(dG, rg, "swiglu dGate"); parity(dU, ru, "swiglu dUp")
+    parity(ops.swiglu(A, B), orc.silu(a) * b, "swiglu fwd")
+    # in place, as src/train.c:5140 calls it (grad_input aliases grad_output)
+    G2 = G.clone()
+    ops.silu_backward(A, G2, out=G2)
+    parity(G2, orc.silu_backward(a, g), "silu_backward in place")
+
+
+def test_elementwise_unaligned_views(ops, orc):
+    r = rng(7)
+    base = r.standard_normal(5000).astype(np.float32)
+    t = dev(base)
+    a, b = t[1:3001], t[1002:4002]                      # 4-byte aligned only
+    out = torch.empty(3001, dtype=torch.float32, device="cuda")[1:]
+    ops.add(a, b, out)
+    assert (host(out) == base[1:3001] + base[1002:4002]).all()
+
+
+def test_fill_nan_reduce(ops, orc):
+    t = torch.empty(1001, dtype=torch.int32, device="cuda")
+    ops.fill_u32(t, 0xDEADBEEF)
+    assert (host(t).view(np.uint32) == 0xDEADBEEF).all()
+    flags = torch.zeros(8, dtype=torch.int32, device="cuda")
+    x = dev(rng(1).standard_normal(70000).astype(np.float32))
+    ops.nan_check(x, flags, 3)
+    assert host(flags).sum() == 0
+    x[69999] = float("inf")
+    ops.nan_check(x, flags, 3)
+    x[5] = float("nan")
+    ops.nan_check(x, flags, 6)
+    assert host(flags).tolist() == [0, 0, 0, 1, 0, 0, 1, 0]
+    v = rng(2).standard_normal(1300).astype(np.float32)
+    parity(ops.reduce_sum(dev(v)), orc.reduce_sum(v), "reduce_sum", atol=1e-4)
+
+
+# ------------------------------------------------------------------ cross entropy
+@pytest.mark.parametrize("rows,cols", [(9, 8192), (5, 1000), (4, 40000), (3, 33001), (2, 151936), (6, 4)])
+def test_cross_entropy_grad(ops, orc, rows, cols):
+    r = rng(rows * 100003 + cols)
+    x = (2 * r.standard_normal((rows, cols))).astype(np.float32)
+    t = r.integers(0, cols, rows).astype(np.uint32)
+    if rows > 2:
+        t[1] = cols                                      # no supervision for this row
+    rg, rl = orc.cross_entropy_grad(x, t, valid_rows=rows - 1)
+    g, l = ops.cross_entropy_grad(dev(x), dev(t.view(np.int32)), rows - 1)
+    parity(l, rl, "loss", atol=1e-5)
+    parity(g, rg, "grad", atol=1e-7)
+    if rows > 2:
+        assert (host(g)[1] == 0).all() and host(l)[1] == 0
+    # in place (grad aliases logits)
+    X = dev(x)
+    g2, l2 = ops.cross_entropy_grad(X, dev(t.view(np.int32)), rows - 1, grad=X)
+    parity(g2, rg, "grad in place", atol=1e-7); parity(l2, rl, "loss in place")
+    g0, _ = ops.cross_entropy_grad(dev(x), dev(t.view(np.int32)), 0)
+    assert (host(g0) == 0).all()
+
+
+def test_cross_entropy_grad_packed(ops, orc):
+    r = rng(11)
+    starts = np.array([0, 3, 4, 20], np.uint32)
+    x = r.standard_normal((20, 8192)).astype(np.float32)
+    t = r.integers(0, 8192, 20).astype(np.uint32)
+    rg, rl = orc.cross_entropy_grad_packed(x, t, starts, 17)
+    g, l = ops.cross_entropy_grad(dev(x), dev(t.view(np.int32)), 17, seq_starts=dev(starts.view(np.int32)))
+    parity(g, rg, "packed grad", atol=1e-7); parity(l, rl, "packed loss")
+    for last in (2, 3, 19):
+        assert (host(g)[last] == 0).all() and host(l)[last] == 0
+
+
+# ------------------------------------------------------------------ GEMM
+@pytest.mark.parametrize("tA,tB", [(0, 0), (1, 0), (0, 1), (1, 1)])
+@pytest.mark.parametrize("M,N,K", [(256, 384, 512), (67, 35, 129), (300, 16, 260), (16, 520, 300), (130, 140, 16),
+                                   (1024, 2048, 96), (1, 1, 1)])
+def test_gemm_forms(ops, orc, tA, tB, M, N, K):
+    r = rng(M * 7 + N * 3 + K + 2 * tA + tB)
+    A = r.standard_normal((K, M) if tA else (M, K)).astype(np.float32)
+    B = r.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+    C0 = r.standard_normal((M, N)).astype(np.float32)
+    ref = orc.matmul(A, B, M, N, K, tA, tB)
+    parity(ops.gemm(dev(A), dev(B), M, N, K, tA, tB), ref, f"gemm tA={tA} tB={tB}", atol=1e-4)
+    out = dev(C0)
+    ops.gemm(dev(A), dev(B), M, N, K, tA, tB, out=out, accumulate=True)
+    parity(out, orc.matmul(A, B, M, N, K, tA, tB, C0), "gemm accumulate", atol=1e-4)
+
+
+def test_gemm_reference_recipe_is_exact(ops):
+    # tests/test_matmul.c:47-49 of the reference: 64^3, integers in [-5, 4]; exact in FP32
+    r = rng(64)
+    A = r.integers(-5, 5, (64, 64)).astype(np.float32)
+    B = r.integers(-5, 5, (64, 64)).astype(np.float32)
+    assert (host(ops.gemm(dev(A), dev(B), 64, 64, 64)) == (A.astype(np.int64) @ B.astype(np.int64))).all()
+    A = r.integers(-5, 5, (300, 200)).astype(np.float32)
+    B = r.integers(-5, 5, (300, 260)).astype(np.float32)      # TN, as the weight gradient uses it
+    assert (host(ops.gemm(dev(A), dev(B), 200, 260, 300, 1, 0)) == (A.T.astype(np.int64) @ B.astype(np.int64))).all()
+
+
+def test_gemm_wgrad_shape_long_k(ops, orc):
+    r = rng(5)
+    T, out_d, in_d = 4096, 192, 160
+    dY = (1e-2 * r.standard_normal((T, out_d))).astype(np.float32)
+    X = r.standard_normal((T, in_d)).astype(np.float32)
+    G0 = (1e-2 * r.standard_normal((out_d, in_d))).astype(np.float32)
+    out = dev(G0)
+    ops.gemm(dev(dY), dev(X), out_d, in_d, T, 1, 0, out=out, accumulate=True)
+    parity(out, orc.matmul(dY, X, out_d, in_d, T, 1, 0, G0), "wgrad")
+
+
+# ------------------------------------------------------------------ rmsnorm
+@pytest.mark.parametrize("rows,cols", [(33, 512), (17, 2048), (5, 4096), (9, 100), (4, 8192), (1, 4)])
+def test_rmsnorm_forward_backward(ops, orc, rows, cols):
+    r = rng(rows + cols)
+    x = r.standard_normal((rows, cols)).astype(np.float32)
+    s = (1 + 0.02 * r.standard_normal(cols)).astype(np.float32)
+    dy = (1e-2 * r.standard_normal((rows, cols))).astype(np.float32)
+    g0 = r.standard_normal(cols).astype(np.float32)
+    for eps in (1e-5, 1e-6):
+        parity(ops.rmsnorm(dev(x), dev(s), eps), orc.rmsnorm(x, s, eps), "rmsnorm")
+        rdx, rgs = orc.rmsnorm_backward_batch(x, s, dy, eps, g0)
+        dx, gs = ops.rmsnorm_backward(dev(x), dev(s), dev(dy), eps, grad_scale=dev(g0))
+        parity(dx, rdx, "rmsnorm dx", atol=1e-7); parity(gs, rgs, "rmsnorm grad_scale")
+
+
+def test_rmsnorm_backward_clamp_branch(ops, orc):
+    r = rng(3)
+    x = (1e-4 * r.standard_normal((6, 512))).astype(np.float32)       # sqrt(ms + 1e-5) < 0.01
+    x[0] = 0
+    s = r.standard_normal(512).astype(np.float32)
+    dy = r.standard_normal((6, 512)).astype(np.float32)
+    rdx, rgs = orc.rmsnorm_backward_batch(x, s, dy, 1e-5)
+    dx, gs = ops.rmsnorm_backward(dev(x), dev(s), dev(dy), 1e-5)
+    parity(dx, rdx, "clamped dx"); parity(gs, rgs, "clamped grad_scale")
+    parity(host(dx)[0], dy[0].astype(np.float64) * s * 100.0, "x=0 row")
+
+
+def test_qk_norm(ops, orc):
+    r = rng(4)
+    x = r.standard_normal((37, 4 * 64)).astype(np.float32)
+    dy = r.standard_normal((37, 4 * 64)).astype(np.float32)
+    parity(ops.qk_norm_(dev(x), 4, 64, 1e-6), orc.qk_norm(x, 4, 64, 1e-6), "qk_norm")
+    assert (host(ops.qk_norm_(dev(x), 4, 64, 1e-6, use_qk_norm=0)) == x).all()     # disabled: untouched
+    parity(ops.qk_norm_backward(dev(x), dev(dy), 4, 64, 1e-6), orc.qk_norm_backward(x, dy, 4, 64, 1e-6), "qk_norm bwd")
+
+
+# ------------------------------------------------------------------ rope
+@pytest.mark.parametrize("heads,D,theta,starts", [(8, 64, 10000.0, [0, 256, 300]), (16, 128, 1e6, [0, 4096]),
+                                                  (3, 16, 10000.0, [0, 1, 2, 50])])
+def test_rope_forward_backward(ops, orc, heads, D, theta, starts):
+    r = rng(heads * D)
+    T = starts[-1]
+    x = r.standard_normal((T, heads * D)).astype(np.float32)
+    su = np.array(starts, np.uint32)
+    sd = dev(su.view(np.int32))
+    # angles reach thousands of radians at theta = 1e6: FP32 sincos argument reduction sets the floor
+    parity(ops.rope(dev(x), heads, D, theta, sd), orc.rope(x, heads, D, theta, su), "rope", atol=2e-5)
+    parity(ops.rope(dev(x), heads, D, theta, sd, backward=True), orc.rope(x, heads, D, theta, su, backward=True),
+           "rope backward", atol=2e-5)
+    X = dev(x)
+    ops.rope(X, heads, D, theta, sd, backward=True, out=X)                       # in place (src/train.c:5253)
+    parity(X, orc.rope(x, heads, D, theta, su, backward=True), "rope backward in place", atol=2e-5)
+    if len(starts) == 2:
+        parity(ops.rope(dev(x), heads, D, theta, None), orc.rope(x, heads, D, theta, None), "rope unpacked", atol=2e-5)
+
+
+# ------------------------------------------------------------------ embedding
+def test_embedding_lookup_and_backward_bit_exact(ops, orc):
+    r = rng(6)
+    T, h, V = 3000, 512, 700
+    tok = r.integers(0, V + 40, T).astype(np.uint32)
+    tok[:50] = 13                                              # a heavily repeated token
+    tok[77] = 4000000000
+    dH = r.integers(-8, 9, (T, h)).astype(np.float32)          # integer-valued: any order sums exactly
+    base = r.integers(-3, 4, (V, h)).astype(np.float32)
+    ref = orc.embedding_backward(tok, dH, base)
+    got = host(ops.embedding_backward(dev(tok.view(np.int32)), dev(dH), dev(base)))
+    assert (got == ref).all()
+    touched = set(np.nonzero((got != base).any(1))[0].tolist())
+    assert touched <= set(np.unique(tok[tok < V]).tolist())
+    E = r.standard_normal((V, h)).astype(np.float32)
+    assert (host(ops.embed_lookup(dev(tok.view(np.int32)), dev(E))) == orc.embed_lookup(tok, E)).all()
+
+
+def test_embedding_backward_float_and_odd_hidden(ops, orc):
+    r = rng(8)
+    T, h, V = 500, 70, 90
+    tok = r.integers(0, V, T).astype(np.uint32)
+    dH = r.standard_normal((T, h)).astype(np.float32)
+    base = r.standard_normal((V, h)).astype(np.float32)
+    parity(ops.embedding_backward(dev(tok.view(np.int32)), dev(dH), dev(base)), orc.embedding_backward(tok, dH, base),
+           "embedding backward")
+    # deterministic: two runs give identical bits
+    a = host(ops.embedding_backward(dev(tok.view(np.int32)), dev(dH), dev(base)))
+    b = host(ops.embedding_backward(dev(tok.view(np.int32)), dev(dH), dev(base)))
+    assert (a == b).all()
+
+
+# ------------------------------------------------------------------ AdamW
+@pytest.mark.parametrize("n", [1, 1000, 100003])
+@pytest.mark.parametrize("clip", [0.0, 1.0])
+def test_adamw(ops, orc, n, clip):
+    r = rng(n)
+    w = r.standard_normal(n).astype(np.float32)
+    m = (1e-3 * r.standard_normal(n)).astype(np.float32)
+    v = (1e-6 * r.random(n)).astype(np.float32)
+    g = (1e-3 * r.standard_normal(n)).astype(np.float32)
+    g[r.random(n) < 0.01] = 10.0
+    for step in (1, 7):
+        rw, rm, rv = orc.adamw(w, g, m, v, 3.14e-4, 0.9, 0.999, 0.01, 1e-8, step, clip)
+        W, M, V = dev(w), dev(m), dev(v)
+        ops.adamw_(W, dev(g), M, V, 3.14e-4, 0.9, 0.999, 0.01, 1e-8, step, clip)
+        parity(W, rw, "adamw w", atol=1e-7); parity(M, rm, "adamw m", atol=1e-9); parity(V, rv, "adamw v", atol=1e-12)
+
+
+# ------------------------------------------------------------------ attention
+ATTN_CASES = [([0, 200], 4, 4, 64), ([0, 5, 6, 133, 300], 4, 2, 32), ([0, 257], 4, 2, 128), ([0, 128, 256], 2, 1, 64),
+              ([0, 1], 2, 2, 64), ([0, 31, 64, 97, 161], 8, 2, 128)]
+
+
+def _attn_inputs(seed, starts, H, KVH, D):
+    r = rng(seed)
+    T = starts[-1]
+    mk = lambda w: (r.standard_normal((T, w)) / np.sqrt(np.sqrt(D))).astype(np.float32)
+    return mk(H * D), mk(KVH * D), mk(KVH * D), mk(H * D)
+
+
+@pytest.mark.parametrize("starts,H,KVH,D", ATTN_CASES)
+def test_attention_forward(ops, orc, starts, H, KVH, D):
+    Q, K, V, _ = _attn_inputs(1, starts, H, KVH, D)
+    su = np.array(starts, np.uint32)
+    ro, rl = orc.attention_forward(Q, K, V, H, KVH, D, su)
+    o, l = ops.attention_forward(dev(Q), dev(K), dev(V), H, KVH, D, dev(su.view(np.int32)))
+    parity(o, ro, "attention out"); parity(l, rl, "attention lse")
+    if len(starts) == 2:
+        o2, _ = ops.attention_forward(dev(Q), dev(K), dev(V), H, KVH, D, None)
+        parity(o2, ro, "attention out, unpacked call")
+
+
+@pytest.mark.parametrize("starts,H,KVH,D", ATTN_CASES)
+@pytest.mark.parametrize("saved", [False, True])
+def test_attention_backward(ops, orc, starts, H, KVH, D, saved):
+    Q, K, V, dO = _attn_inputs(2, starts, H, KVH, D)
+    su = np.array(starts, np.uint32)
+    sd = dev(su.view(np.int32))
+    base = rng(3).standard_normal(K.shape).astype(np.float32)
+    rdQ, rdK, rdV = orc.attention_backward(Q, K, V, dO, H, KVH, D, su, dK0=base, dV0=base)
+    out = lse = None
+    if saved:
+        out, lse = ops.attention_forward(dev(Q), dev(K), dev(V), H, KVH, D, sd)
+    dQ, dK, dV = ops.attention_backward(dev(Q), dev(K), dev(V), dev(dO), H, KVH, D, sd, out=out, lse=lse,
+                                        dK=dev(base), dV=dev(base))
+    parity(dQ, rdQ, "dQ"); parity(dK, rdK, "dK"); parity(dV, rdV, "dV")
+
+
+def test_attention_backward_is_deterministic(ops):
+    Q, K, V, dO = _attn_inputs(4, [0, 300, 700], 4, 2, 64)
+    sd = dev(np.array([0, 300, 700], np.int32))
+    a = [host(t) for t in ops.attention_backward(dev(Q), dev(K), dev(V), dev(dO), 4, 2, 64, sd)]
+    b = [host(t) for t in ops.attention_backward(dev(Q), dev(K), dev(V), dev(dO), 4, 2, 64, sd)]
+    assert all((x == y).all() for x, y in zip(a, b))
+
+
+def test_attention_rejects_unsupported_head_dim(ops):
+    from seraph_amd._lib import SeraphError
+    Q = torch.zeros(8, 48, device="cuda")
+    with pytest.raises(SeraphError):
+        ops.attention_forward(Q, Q, Q, 2, 2, 24)
