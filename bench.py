@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Headline benchmark: training tokens/s (forward + backward + AdamW) of the packed-batch
+training step on ONE MI355X, with the dominant kernel's roofline fraction measured live and
+the CPU oracle timed beside it.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c1]
+
+Workloads (BASELINE.json configs): c5 = Qwen3-1.7B-shape full-weight FP32 training,
+4 x 4096 tokens (default); c4 = the same model, LoRA r16 on q/k/v/o, 1 x 2048; c1 = the
+33M Seraph-native model, 8 x 256.  Synthetic data: uniform token ids, N(0, 0.02) weights,
+norm gains 1, fixed seeds.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3      # MI355X dense FP32 matrix peak
+PEAK_HBM_GBS = 8000.0              # MI355X HBM3E peak
+
+WORKLOADS = {
+    "c5": dict(name="qwen3-1.7b-shape full-weight fp32, 4x4096 packed", hidden=2048, layers=28, heads=16, kv_heads=8,
+               head_dim=128, ffn=6144, vocab=151936, rms_eps=1e-6, rope_theta=1e6, batch=4, seq=4096, lr=3.14e-4,
+               clip=0.0, lora=None),
+    "c4": dict(name="qwen3-1.7b-shape LoRA r16 a32 on q/k/v/o fp32, 1x2048", hidden=2048, layers=28, heads=16, kv_heads=8,
+               head_dim=128, ffn=6144, vocab=151936, rms_eps=1e-6, rope_theta=1e6, batch=1, seq=2048, lr=3.14e-4,
+               clip=0.0, lora=dict(rank=16, alpha=32.0, mask=0b1111)),
+    "c1": dict(name="seraph-native 33M full-weight fp32, 8x256 packed", hidden=512, layers=8, heads=8, kv_heads=8,
+               head_dim=64, ffn=1408, vocab=8192, rms_eps=1e-6, rope_theta=10000.0, batch=8, seq=256, lr=3.14e-4,
+               clip=1.0, lora=None),
+}
+
+
+def norm_gain_slices(w):
+    """(start, stop) of every RMSNorm gain inside the flat parameter arena."""
+    h, qd, kv, f, V = w["hidden"], w["heads"] * w["head_dim"], w["kv_heads"] * w["head_dim"], w["ffn"], w["vocab"]
+    out = [(V * h, V * h + h)]
+    stride = h + qd * h + 2 * kv * h + h * qd + h + 3 * f * h
+    for l in range(w["layers"]):
+        base = V * h + h + l * stride
+        out.append((base, base + h))
+        pn = base + h + qd * h + 2 * kv * h + h * qd
+        out.append((pn, pn + h))
+    return out
+
+
+def cpu_baseline(w, budget_tokens=192):
+    """The CPU oracle's own step (same mathematics, OpenMP over rows/heads, double accumulation)
+    on a bounded sample: the real widths and vocabulary, `budget_tokens` tokens in one sequence,
+    with one and with three layers (best of two runs each, the first run also warms the
+    allocator); the per-layer and the head costs are then scaled to the full depth."""
+    from oracle import oracle as orc
+    T = min(budget_tokens, w["seq"])
+    tok = np.random.default_rng(0).integers(0, w["vocab"], T).astype(np.int32)
+    best = {}
+    for L in (1, 1, 3, 3):
+        kw = dict(hidden=w["hidden"], layers=L, heads=w["heads"], kv_heads=w["kv_heads"], head_dim=w["head_dim"],
+                  ffn=w["ffn"], vocab=w["vocab"], rms_eps=w["rms_eps"], rope_theta=w["rope_theta"])
+        if w["lora"]:
+            kw.update(lora_rank=w["lora"]["rank"], lora_alpha=w["lora"]["alpha"], lora_mask=w["lora"]["mask"])
+        cfg = orc.make_config(**kw)
+        p = np.full(orc.param_count(cfg), 0.01, np.float32)
+        lo = np.full(max(orc.lora_param_count(cfg), 1), 0.01, np.float32)
+        t0 = time.perf_counter()
+        if w["lora"]:
+            orc.step_lora(cfg, p, lo, tok)
+        else:
+            orc.step_full(cfg, p, tok)
+        dt = time.perf_counter() - t0
+        best[L] = min(best.get(L, dt), dt)
+        del p
+    per_layer = max((best[3] - best[1]) / 2.0, 1e-9)
+    head = max(best[1] - per_layer, 0.0)
+    full = head + per_layer * w["layers"]
+    return dict(value=round(T / full, 3), unit="tok/s", cores=orc.num_threads(), kind="port",
+                sample=(f"oracle step (fwd+loss+bwd, no AdamW) on {T} tokens in 1 sequence at full width and vocabulary, "
+                        f"1 layer {best[1]:.2f}s and 3 layers {best[3]:.2f}s (best of 2); LM-head/embedding cost "
+                        f"{head:.2f}s + {per_layer:.2f}s per layer scaled to {w['layers']} layers"))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
+                 "(value is the one GPU's throughput)")
+
+    import torch
+    from seraph_amd import trainer as tr
+
+    w = WORKLOADS[args.workload]
+    T = w["batch"] * w["seq"]
+    lora = w["lora"] or dict(rank=0, alpha=0.0, mask=0)
+    cfg = tr.model_config(w["hidden"], w["layers"], w["heads"], w["kv_heads"], w["head_dim"], w["ffn"], w["vocab"],
+                          w["rms_eps"], w["rope_theta"], lora["rank"], lora["alpha"], lora["mask"])
+    opt = tr.optim_config(w["lr"], clip=w["clip"])
+    n = tr.param_count(cfg)
+
+    torch.manual_seed(1234)
+    dev = torch.device("cuda:0")
+    params = torch.empty(n, dtype=torch.float32, device=dev).normal_(0.0, 0.02)
+    for a, b in norm_gain_slices(w):
+        params[a:b] = 1.0
+    if w["lora"]:
+        ext = (params, None, None, None)
+    else:
+        ext = (params, torch.zeros(n, dtype=torch.float32, device=dev), torch.zeros(n, dtype=torch.float32, device=dev),
+               torch.zeros(n, dtype=torch.float32, device=dev))
+    torch.cuda.synchronize()
+    t = tr.Trainer(cfg, opt, max_tokens=T, max_batch=w["batch"], device=0, ext=ext)
+    if w["lora"]:
+        nl = tr.lora_param_count(cfg)
+        lo = (0.01 * np.random.default_rng(5).standard_normal(nl)).astype(np.float32)     # A ~ N(0, 0.01)
+        h, qd, kv, r = w["hidden"], w["heads"] * w["head_dim"], w["kv_heads"] * w["head_dim"], lora["rank"]
+        o = 0
+        for _ in range(w["layers"]):                                                    # B = 0
+            for i, oo in ((h, qd), (h, kv), (h, kv), (qd, h)):
+                o += r * i
+                lo[o:o + oo * r] = 0
+                o += oo * r
+        t.upload(tr.LORA_PARAMS, lo)
+
+    rng = np.random.default_rng(99)
+    starts = np.arange(0, T + 1, w["seq"], dtype=np.int32)
+    batches = [rng.integers(0, w["vocab"], T).astype(np.int32) for _ in range(args.warmup + args.steps)]
+
+    losses = []
+    for i in range(args.warmup):
+        losses.append(t.step(batches[i], starts))
+    t.enable_op_timing(True)
+    t.reset_op_stats()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        losses.append(t.step(batches[args.warmup + i], starts))
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    timing = t.last_timing()
+
+    stats = t.op_stats()
+    total_ms = sum(s["ms"] for s in stats) or 1.0
+    kernels = {}
+    for s in sorted(stats, key=lambda s: -s["ms"]):
+        avg = s["ms"] / max(s["launches"], 1)
+        e = dict(launches=s["launches"], avg_ms=round(avg, 4), share=round(s["ms"] / total_ms, 4))
+        if s["flops"] > 0:
+            e["tflops"] = round(s["flops"] / s["ms"] / 1e9, 2)
+            e["frac_mfma_peak"] = round(s["flops"] / s["ms"] / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)
+        elif s["bytes"] > 0:
+            e["gbs"] = round(s["bytes"] / s["ms"] / 1e6, 1)
+            e["frac_hbm_peak"] = round(s["bytes"] / s["ms"] / 1e6 / PEAK_HBM_GBS, 4)
+        kernels[s["name"]] = e
+    dom = max(stats, key=lambda s: s["ms"])
+    if dom["flops"] > 0:
+        achieved = dom["flops"] / dom["ms"] / 1e9
+        roofline = dict(bound="mfma", kernel=dom["name"], achieved=round(achieved, 2), peak=PEAK_FP32_MFMA_TFLOPS,
+                        unit="TFLOP/s", frac=round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), traffic=None,
+                        launches=dom["launches"], avg_launch_ms=round(dom["ms"] / dom["launches"], 4),
+                        flops_per_launch=dom["flops"] / dom["launches"])
+    else:
+        achieved = dom["bytes"] / dom["ms"] / 1e6
+        roofline = dict(bound="hbm", kernel=dom["name"], achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                        frac=round(achieved / PEAK_HBM_GBS, 4), traffic=None, launches=dom["launches"],
+                        avg_launch_ms=round(dom["ms"] / dom["launches"], 4), bytes_per_launch=dom["bytes"] / dom["launches"])
+
+    out = {
+        "metric": "train tok/s (fwd+bwd+AdamW)", "value": round(args.steps * T / elapsed, 2), "unit": "tok/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(1000.0 * elapsed / args.steps, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": w["name"], "tokens_per_step": T, "batch": w["batch"], "seq_len": w["seq"],
+                   "params": n, "device_bytes": t.device_bytes + sum(x.numel() * 4 for x in ext if x is not None),
+                   "rms_eps": w["rms_eps"], "adamw_clip": w["clip"], "seed": 1234},
+        "loss_first_last": [round(losses[0], 5), round(losses[-1], 5)],
+        "phase_ms_last_step": {k: round(v, 3) for k, v in timing.items()},
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    t.close()
+    del params, ext
+    torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,105 @@
+/*
+ * hip_train.h - packed-batch training steps for Seraph-shaped decoder models on one
+ * MI355X: forward, loss, backward and AdamW, all device resident.
+ *
+ * Stands in for cuda_train_step_gpu_full_batch / cuda_train_step_gpu_lora_batch
+ * (include/train_cuda.h:41-49): same arguments (a packed token stream plus seq_starts
+ * prefix offsets), same return value (mean loss over total_tokens - batch_size
+ * predictions), same accumulation / warm-up / optimizer-step bookkeeping as
+ * src/train.c:5439-5463.  The mathematics of every op is the Vulkan path's
+ * (shaders/ *.comp in the op order of src/train.c:4365-5763 and :5847-6719); the LoRA step
+ * follows train_step_gpu_lora, not the approximate CUDA variant.
+ *
+ * What differs from the reference is layout and fusion only: parameters, gradients and
+ * the two Adam moments are four flat arenas (one AdamW launch covers the model),
+ * activations are written once where the backward reads them (no cache copies),
+ * silu*mul and its backward are single passes, the attention backward reuses the
+ * forward's output and log-sum-exp, and sums of weight-side gradients use GEMM
+ * accumulation instead of a temporary and an add.
+ *
+ * Arena layout (floats): embed[V,h], final_norm[h], then per layer
+ *   in_norm[h], q[q,h], k[kv,h], v[kv,h], o[h,q], post_norm[h], gate[f,h], up[f,h], down[h,f].
+ * LoRA arena: per layer, for each of q,k,v,o selected by lora_mask (bit 0..3): A[r,in], B[out,r].
+ */
+#ifndef HIP_TRAIN_H
+#define HIP_TRAIN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct {
+    int32_t hidden, layers, heads, kv_heads, head_dim, ffn, vocab;
+    float   rms_eps;        /* the reference's step hard-codes 1e-5 (src/train.c:4378) */
+    float   rope_theta;
+    int32_t lora_rank;      /* 0 = full-weight training */
+    float   lora_alpha;
+    int32_t lora_mask;      /* bit0 q, bit1 k, bit2 v, bit3 o */
+} hip_model_config_t;
+
+typedef struct {
+    float   learning_rate;
+    float   beta1, beta2, weight_decay, eps;     /* reference: 0.9, 0.999, 0.01, 1e-8 (src/train.c:5449-5452) */
+    float   clip;                                /* per-element gradient clamp; <= 0 = off (the reference) */
+    int32_t warmup_steps;                        /* reference: 100 (src/train.c:5456) */
+    int32_t gradient_accumulation_steps;
+} hip_optim_config_t;
+
+typedef struct hip_trainer hip_trainer_t;
+
+int64_t hip_param_count(const hip_model_config_t* cfg);
+int64_t hip_lora_param_count(const hip_model_config_t* cfg);
+
+/* ext_* are optional caller-owned DEVICE arenas of hip_param_count floats (NULL: allocated
+ * here).  In LoRA mode (cfg->lora_rank > 0) only ext_params is used: the base model is frozen
+ * and the adapter arenas are always owned by the trainer.  Returns NULL on failure with the
+ * reason on stderr. */
+hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim_config_t* opt,
+                                  int max_tokens, int max_batch, int device_index,
+                                  float* ext_params, float* ext_grads, float* ext_m, float* ext_v);
+void hip_trainer_free(hip_trainer_t* t);
+
+/* host <-> device transfers of whole arenas; `which`: 0 params, 1 grads, 2 m, 3 v,
+ * 4 lora params, 5 lora grads, 6 lora m, 7 lora v.  Return 0 on success. */
+int hip_trainer_upload(hip_trainer_t* t, int which, const float* host, int64_t count);
+int hip_trainer_download(hip_trainer_t* t, int which, float* host, int64_t count);
+void* hip_trainer_device_ptr(hip_trainer_t* t, int which);
+
+/* One packed step.  tokens_packed[total_tokens]; seq_starts[batch_size + 1] (NULL with
+ * batch_size 1 = one sequence).  Negative ids are treated as 0 (src/train.c:4473).
+ * run_optimizer = 0 leaves the weights untouched (gradients only).  Returns the mean loss,
+ * or -1 on error. */
+float hip_train_step_full_batch(hip_trainer_t* t, const int* tokens_packed, int total_tokens,
+                                const int* seq_starts, int batch_size, int run_optimizer);
+float hip_train_step_lora_batch(hip_trainer_t* t, const int* tokens_packed, int total_tokens,
+                                const int* seq_starts, int batch_size, int run_optimizer);
+
+int   hip_trainer_optimizer_step(const hip_trainer_t* t);
+float hip_trainer_last_lr(const hip_trainer_t* t);
+/* device time of the phases of the last step, in ms: [0] forward+loss, [1] backward, [2] optimizer */
+void  hip_trainer_last_timing(const hip_trainer_t* t, float ms[3]);
+size_t hip_trainer_device_bytes(const hip_trainer_t* t);
+
+/* Optional per-kernel accounting (the counterpart of the reference's per-op profilers,
+ * src/vulkan_backend.c:105-210, include/cuda_profiler.h:18-28): with timing on, every
+ * kernel-library call of a step is bracketed by an event pair on the step's stream and
+ * folded per kernel class with its algorithmic work (flops for the matrix-core kernels,
+ * compulsory HBM bytes for the streaming ones). */
+typedef struct {
+    const char* name;      /* GEMMs: the kernel instantiation, as a profiler names it */
+    int64_t     launches;
+    double      ms;        /* summed device time */
+    double      flops;     /* summed algorithmic flops (0 for bandwidth-bound classes) */
+    double      bytes;     /* summed algorithmic bytes (0 for matrix-core classes)     */
+} hip_op_stat_t;
+void hip_trainer_enable_op_timing(hip_trainer_t* t, int on);
+void hip_trainer_reset_op_stats(hip_trainer_t* t);
+int  hip_trainer_op_stats(const hip_trainer_t* t, hip_op_stat_t* out, int max);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

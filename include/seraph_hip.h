@@ -102,6 +102,9 @@ int seraph_cross_entropy_grad(const float* logits, const uint32_t* targets, floa
  * C[M,N] (+)= op(A) op(B); transposed A is stored [K,M], transposed B is stored [N,K]. */
 int seraph_gemm(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
                 int transpose_A, int transpose_B, int accumulate, seraph_stream_t s);
+/* Name of the kernel instantiation seraph_gemm launches for this shape with 16-byte aligned
+ * operands, as a profiler prints it (no reference counterpart; used to label timings). */
+const char* seraph_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int transpose_A, int transpose_B);
 
 /* ---------------------------------------------------------------- attention */
 /* vulkan_batch_attention (include/vulkan_backend.h:485-488, shaders/batch_attention_stream.comp)

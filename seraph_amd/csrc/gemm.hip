@@ -226,6 +226,21 @@ static int launch_gemm(const float* A, const float* B, float* C, int64_t M, int6
 
 using namespace seraph;
 
+// 128x128 tiles when they fill the machine at least once, else 64x64.
+static bool use_big_tiles(int64_t M, int64_t N) {
+    return ceil_div(M, 128) * ceil_div(N, 128) >= num_compute_units();
+}
+
+extern "C" const char* seraph_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int transpose_A, int transpose_B) {
+    (void)K;
+    static const char* names[2][4] = {
+        {"seraph::gemm_f32_mfma_kernel<1, 1, true, false, true>", "seraph::gemm_f32_mfma_kernel<1, 1, true, true, true>",
+         "seraph::gemm_f32_mfma_kernel<1, 1, false, false, true>", "seraph::gemm_f32_mfma_kernel<1, 1, false, true, true>"},
+        {"seraph::gemm_f32_mfma_kernel<2, 2, true, false, true>", "seraph::gemm_f32_mfma_kernel<2, 2, true, true, true>",
+         "seraph::gemm_f32_mfma_kernel<2, 2, false, false, true>", "seraph::gemm_f32_mfma_kernel<2, 2, false, true, true>"}};
+    return names[use_big_tiles(M, N) ? 1 : 0][(transpose_A ? 2 : 0) + (transpose_B ? 1 : 0)];
+}
+
 extern "C" int seraph_gemm(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
                            int transpose_A, int transpose_B, int accumulate, seraph_stream_t s) {
     if (M == 0 || N == 0) return SERAPH_OK;
@@ -234,9 +249,7 @@ extern "C" int seraph_gemm(const float* A, const float* B, float* C, int64_t M, 
     const int64_t lda = transpose_A ? M : K, ldb = transpose_B ? K : N;
     const bool vec = (lda % 4 == 0) && (ldb % 4 == 0) && aligned16(A) && aligned16(B);
     hipStream_t st = as_stream(s);
-    // 128x128 tiles when they fill the machine at least once, else 64x64.
-    const int64_t big_tiles = ceil_div(M, 128) * ceil_div(N, 128);
-    if (big_tiles >= num_compute_units())
+    if (use_big_tiles(M, N))
         return launch_gemm<2, 2>(A, B, C, M, N, K, transpose_A, transpose_B, accumulate, vec, st);
     return launch_gemm<1, 1>(A, B, C, M, N, K, transpose_A, transpose_B, accumulate, vec, st);
 }

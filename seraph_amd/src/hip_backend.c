@@ -1,0 +1,414 @@
+/*
+ * hip_backend.c - runtime, buffers, forward ops and the optimizer op of the backend API
+ * (the counterpart of Seraph's src/vulkan_backend.c), over the MI355X kernel library.
+ * Plain C, no HIP headers: everything device-side goes through include/seraph_hip.h.
+ *
+ * One in-order HIP stream replaces the command buffer: ops are enqueued as they are
+ * called, vulkan_cmd_end_submit waits for the stream, and transfers from or to host
+ * memory wait for the work queued before them - which is the ordering the reference
+ * gets from its barrier after every recorded op (src/vulkan_backend_backward.c:124-142).
+ */
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "hip_backend_internal.h"
+
+/* ------------------------------------------------------------------ helpers */
+void hip_backend_report(vulkan_context_t* ctx, const char* op, int rc) {
+    hip_state_t* st = hip_state(ctx);
+    if (st) st->errors++;
+    fprintf(stderr, "ERROR: %s failed (%d): %s\n", op, rc, seraph_hip_last_error());
+}
+
+int hip_backend_error_count(vulkan_context_t* ctx) {
+    hip_state_t* st = hip_state(ctx);
+    return st ? st->errors : -1;
+}
+
+void* hip_backend_scratch(vulkan_context_t* ctx, size_t bytes) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st) return NULL;
+    if (bytes <= st->ws_bytes && st->ws) return st->ws;
+    /* queued kernels may still read the old block */
+    if (seraph_hip_stream_sync(st->stream) != SERAPH_OK) return NULL;
+    seraph_hip_free(st->ws);
+    st->ws = NULL;
+    st->ws_bytes = 0;
+    size_t want = bytes + bytes / 4 + (1u << 20);
+    void* p = NULL;
+    if (seraph_hip_malloc(&p, want) != SERAPH_OK) {
+        hip_backend_report(ctx, "scratch allocation", SERAPH_ERR_HIP);
+        return NULL;
+    }
+    st->ws = p;
+    st->ws_bytes = want;
+    return p;
+}
+
+/* ------------------------------------------------------------------ profiler
+ * hipEvent pairs per op; vulkan_profiler_end_step prints the per-op table and a roll-up
+ * by op-name substring, like src/vulkan_backend.c:105-210. */
+void hip_prof_begin(vulkan_context_t* ctx, const char* name) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !ctx->profiling || st->prof_count >= HIP_PROF_MAX_OPS) return;
+    if (!st->prof_ops) st->prof_ops = (hip_prof_op_t*)calloc(HIP_PROF_MAX_OPS, sizeof(hip_prof_op_t));
+    if (!st->prof_ops) return;
+    hip_prof_op_t* op = &st->prof_ops[st->prof_count];
+    if (st->prof_count >= st->prof_events_made) {
+        if (seraph_hip_event_create(&op->ev_start) != SERAPH_OK || seraph_hip_event_create(&op->ev_stop) != SERAPH_OK) return;
+        st->prof_events_made = st->prof_count + 1;
+    }
+    op->name = name;
+    seraph_hip_event_record(op->ev_start, st->stream);
+}
+
+void hip_prof_end(vulkan_context_t* ctx) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !ctx->profiling || !st->prof_ops || st->prof_count >= st->prof_events_made) return;
+    seraph_hip_event_record(st->prof_ops[st->prof_count].ev_stop, st->stream);
+    st->prof_count++;
+    ctx->prof_num_ops = st->prof_count;
+}
+
+void vulkan_profiler_enable(vulkan_context_t* ctx) { if (ctx) ctx->profiling = 1; }
+void vulkan_profiler_disable(vulkan_context_t* ctx) { if (ctx) ctx->profiling = 0; }
+void vulkan_profiler_set_log(vulkan_context_t* ctx, void* file_ptr) { if (ctx) ctx->prof_log = file_ptr; }
+
+void vulkan_profiler_begin_step(vulkan_context_t* ctx) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st) return;
+    st->prof_count = 0;
+    ctx->prof_num_ops = 0;
+}
+
+void vulkan_profiler_end_step(vulkan_context_t* ctx, int step, int seq_len, float loss) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !ctx->profiling || st->prof_count == 0) return;
+    FILE* out = ctx->prof_log ? (FILE*)ctx->prof_log : stderr;
+    static const char* cats[] = {"matmul", "attention", "rmsnorm", "rope", "cross_entropy", "adamw", "embed", "silu", "mul", "add", "copy", "fill"};
+    enum { NCAT = sizeof(cats) / sizeof(cats[0]) };
+    double cat_ms[NCAT + 1] = {0}, total = 0.0;
+    seraph_hip_stream_sync(st->stream);
+    fprintf(out, "[HIP PROFILE] step=%d seq=%d loss=%.6f ops=%d\n", step, seq_len, loss, st->prof_count);
+    for (int i = 0; i < st->prof_count; i++) {
+        float ms = 0.f;
+        seraph_hip_event_elapsed_ms(st->prof_ops[i].ev_start, st->prof_ops[i].ev_stop, &ms);
+        total += ms;
+        int c = NCAT;
+        for (int k = 0; k < NCAT; k++) if (strstr(st->prof_ops[i].name, cats[k])) { c = k; break; }
+        cat_ms[c] += ms;
+        fprintf(out, "  %4d %-32s %9.3f ms\n", i, st->prof_ops[i].name, ms);
+    }
+    for (int k = 0; k <= NCAT; k++)
+        if (cat_ms[k] > 0) fprintf(out, "  [%s] %.3f ms (%.1f%%)\n", k < NCAT ? cats[k] : "other", cat_ms[k], 100.0 * cat_ms[k] / total);
+    fprintf(out, "  [total] %.3f ms\n", total);
+    fflush(out);
+}
+
+/* ------------------------------------------------------------------ init / free */
+vulkan_context_t* vulkan_init_ex(int pool_size_hint, int device_index) {
+    (void)pool_size_hint;
+    if (seraph_hip_init(device_index) != SERAPH_OK) {
+        fprintf(stderr, "ERROR: HIP backend init failed: %s\n", seraph_hip_last_error());
+        return NULL;
+    }
+    vulkan_context_t* ctx = (vulkan_context_t*)calloc(1, sizeof(vulkan_context_t));
+    hip_state_t* st = (hip_state_t*)calloc(1, sizeof(hip_state_t));
+    if (!ctx || !st) { free(ctx); free(st); return NULL; }
+    if (seraph_hip_stream_create(&st->stream) != SERAPH_OK) {
+        fprintf(stderr, "ERROR: HIP stream creation failed: %s\n", seraph_hip_last_error());
+        free(ctx); free(st);
+        return NULL;
+    }
+    seraph_device_info_t info;
+    if (seraph_hip_device_info(&info) == SERAPH_OK) {
+        snprintf(ctx->gpu_name, sizeof(ctx->gpu_name), "%.180s (%.60s)", info.name, info.arch);
+        ctx->vram_bytes = info.hbm_bytes;
+        ctx->max_compute_units = info.compute_units;
+        ctx->subgroup_size = ctx->min_subgroup_size = ctx->max_subgroup_size = info.wavefront_size;
+        ctx->max_shared_memory = info.lds_bytes_per_block;
+    }
+    ctx->device_type = 2;                         /* discrete */
+    ctx->vendor_id = 0x1002;
+    ctx->max_workgroup_invocations = 1024;
+    ctx->max_workgroup_size[0] = 1024; ctx->max_workgroup_size[1] = 1024; ctx->max_workgroup_size[2] = 1024;
+    ctx->max_workgroup_count[0] = 0x7fffffffu; ctx->max_workgroup_count[1] = 65535; ctx->max_workgroup_count[2] = 65535;
+    ctx->max_storage_buffer_range = 0xffffffffu;
+    ctx->has_shader_atomic_float = 1;
+    ctx->wg_size_1d = 256;                        /* vulkan_reduce_sum's caller assumes 512 inputs per output */
+    ctx->wg_size_attn = 64;
+    ctx->wg_size_matmul = 128; ctx->matmul_reg = 32; ctx->matmul_bk = 32;
+    ctx->device = st;
+    ctx->queue = st->stream;
+    ctx->initialized = 1;
+    return ctx;
+}
+
+vulkan_context_t* vulkan_init(int pool_size_hint) { return vulkan_init_ex(pool_size_hint, -1); }
+
+void vulkan_free(vulkan_context_t* ctx) {
+    if (!ctx) return;
+    hip_state_t* st = hip_state(ctx);
+    if (st) {
+        seraph_hip_stream_sync(st->stream);
+        seraph_hip_free(st->ws);
+        if (st->prof_ops) {
+            for (int i = 0; i < st->prof_events_made; i++) {
+                seraph_hip_event_destroy(st->prof_ops[i].ev_start);
+                seraph_hip_event_destroy(st->prof_ops[i].ev_stop);
+            }
+            free(st->prof_ops);
+        }
+        seraph_hip_stream_destroy(st->stream);
+        free(st);
+    }
+    /* Buffers parked in the context's slot table belong to the caller (train.c frees them). */
+    free(ctx);
+}
+
+int vulkan_cmd_begin(vulkan_context_t* ctx) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || st->recording) return 0;
+    st->recording = 1;
+    return 1;
+}
+
+int vulkan_cmd_end_submit(vulkan_context_t* ctx) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !st->recording) return 0;
+    st->recording = 0;
+    int rc = seraph_hip_stream_sync(st->stream);
+    if (rc != SERAPH_OK) { hip_backend_report(ctx, "vulkan_cmd_end_submit", rc); return 0; }
+    return 1;
+}
+
+/* ------------------------------------------------------------------ buffers */
+vulkan_buffer_t* vulkan_buffer_create(vulkan_context_t* ctx, size_t size) {
+    if (!hip_state(ctx)) return NULL;
+    vulkan_buffer_t* buf = (vulkan_buffer_t*)calloc(1, sizeof(vulkan_buffer_t));
+    if (!buf) return NULL;
+    if (seraph_hip_malloc(&buf->buffer, size) != SERAPH_OK) {
+        hip_backend_report(ctx, "vulkan_buffer_create", SERAPH_ERR_HIP);
+        free(buf);
+        return NULL;
+    }
+    buf->memory = buf->buffer;
+    buf->size = size;
+    buf->mapped = NULL;
+    return buf;
+}
+
+void vulkan_buffer_free(vulkan_context_t* ctx, vulkan_buffer_t* buf) {
+    hip_state_t* st = hip_state(ctx);
+    if (!buf) return;
+    if (st) seraph_hip_stream_sync(st->stream);           /* queued ops may still use it */
+    seraph_hip_free(buf->buffer);
+    free(buf);
+}
+
+void vulkan_buffer_upload_bytes(vulkan_context_t* ctx, vulkan_buffer_t* buf, const void* data, size_t bytes) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !buf || !data) return;
+    if (bytes > buf->size) bytes = buf->size;
+    int rc = seraph_hip_h2d(DPTR(buf), data, bytes, st->stream);
+    if (rc != SERAPH_OK) hip_backend_report(ctx, "vulkan_buffer_upload", rc);
+}
+
+void vulkan_buffer_upload(vulkan_context_t* ctx, vulkan_buffer_t* buf, const float* data, size_t count) {
+    vulkan_buffer_upload_bytes(ctx, buf, data, count * sizeof(float));
+}
+
+void vulkan_buffer_upload_u32(vulkan_context_t* ctx, vulkan_buffer_t* buf, const uint32_t* data, size_t count) {
+    vulkan_buffer_upload_bytes(ctx, buf, data, count * sizeof(uint32_t));
+}
+
+void vulkan_buffer_download_bytes(vulkan_context_t* ctx, vulkan_buffer_t* buf, void* data, size_t bytes) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !buf || !data) return;
+    if (bytes > buf->size) bytes = buf->size;
+    int rc = seraph_hip_d2h(data, DPTR(buf), bytes, st->stream);
+    if (rc != SERAPH_OK) hip_backend_report(ctx, "vulkan_buffer_download", rc);
+}
+
+void vulkan_buffer_download(vulkan_context_t* ctx, vulkan_buffer_t* buf, float* data, size_t count) {
+    vulkan_buffer_download_bytes(ctx, buf, data, count * sizeof(float));
+}
+
+void vulkan_fill_buffer_range(vulkan_context_t* ctx, vulkan_buffer_t* buf, size_t offset_bytes, uint32_t value, size_t bytes) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !buf || bytes == 0) return;
+    if (offset_bytes >= buf->size) return;
+    if (bytes > buf->size - offset_bytes) bytes = buf->size - offset_bytes;
+    offset_bytes &= ~(size_t)3;                           /* as src/vulkan_backend.c:1216-1223 */
+    bytes &= ~(size_t)3;
+    if (bytes == 0) return;
+    HIP_OP(ctx, "fill_buffer", seraph_fill_u32((char*)DPTR(buf) + offset_bytes, value, bytes / 4, st->stream));
+}
+
+void vulkan_fill_buffer(vulkan_context_t* ctx, vulkan_buffer_t* buf, uint32_t value, size_t bytes) {
+    vulkan_fill_buffer_range(ctx, buf, 0, value, bytes);
+}
+
+void vulkan_copy_buffer(vulkan_context_t* ctx, vulkan_buffer_t* src, vulkan_buffer_t* dst, size_t bytes) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !src || !dst || bytes == 0) return;
+    if (bytes > src->size) bytes = src->size;
+    if (bytes > dst->size) bytes = dst->size;
+    HIP_OP(ctx, "copy_buffer", seraph_hip_d2d(DPTR(dst), DPTR(src), bytes, st->stream));
+}
+
+void vulkan_copy_buffer_cache(vulkan_context_t* ctx, vulkan_buffer_t* src, vulkan_buffer_t* dst, size_t bytes) {
+    vulkan_copy_buffer(ctx, src, dst, bytes);             /* the stream already orders it */
+}
+
+void vulkan_barrier_transfer_to_compute(vulkan_context_t* ctx) { (void)ctx; }
+
+void vulkan_nan_check(vulkan_context_t* ctx, vulkan_buffer_t* input, size_t count_floats, vulkan_buffer_t* flags_u32, uint32_t flag_index) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !input || !flags_u32 || count_floats == 0) return;
+    if ((size_t)(flag_index + 1) * 4 > flags_u32->size) return;
+    HIP_OP(ctx, "nan_check", seraph_nan_check(FPTR(input), count_floats, UPTR(flags_u32), flag_index, st->stream));
+}
+
+/* ------------------------------------------------------------------ forward ops */
+void vulkan_matmul(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C, int M, int N, int K) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !A || !B || !C) return;
+    HIP_OP(ctx, "matmul", seraph_gemm(FPTR(A), FPTR(B), FPTR(C), M, N, K, 0, 0, 0, st->stream));
+}
+
+void vulkan_matmul_transpose(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C,
+                             int M, int N, int K, int transpose_A, int transpose_B, int accumulate) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !A || !B || !C) return;
+    HIP_OP(ctx, "matmul_transpose", seraph_gemm(FPTR(A), FPTR(B), FPTR(C), M, N, K, transpose_A, transpose_B, accumulate, st->stream));
+}
+
+void vulkan_add(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C, size_t count) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !A || !B || !C) return;
+    HIP_OP(ctx, "add", seraph_add(FPTR(A), FPTR(B), FPTR(C), count, st->stream));
+}
+
+void vulkan_mul(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C, size_t count) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !A || !B || !C) return;
+    HIP_OP(ctx, "mul", seraph_mul(FPTR(A), FPTR(B), FPTR(C), count, st->stream));
+}
+
+void vulkan_scale(vulkan_context_t* ctx, vulkan_buffer_t* A, size_t count, float alpha) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !A) return;
+    HIP_OP(ctx, "scale", seraph_scale(FPTR(A), count, alpha, st->stream));
+}
+
+void vulkan_silu(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* output, size_t count) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !input || !output) return;
+    HIP_OP(ctx, "silu", seraph_silu(FPTR(input), FPTR(output), count, st->stream));
+}
+
+void hip_swiglu(vulkan_context_t* ctx, vulkan_buffer_t* gate, vulkan_buffer_t* up, vulkan_buffer_t* out, size_t count) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !gate || !up || !out) return;
+    HIP_OP(ctx, "silu_mul", seraph_swiglu(FPTR(gate), FPTR(up), FPTR(out), count, st->stream));
+}
+
+void vulkan_rmsnorm(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* scale, vulkan_buffer_t* output,
+                    int rows, int cols, float eps) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !input || !scale || !output) return;
+    HIP_OP(ctx, "rmsnorm", seraph_rmsnorm(FPTR(input), FPTR(scale), FPTR(output), rows, cols, eps, st->stream));
+}
+
+void vulkan_rope(vulkan_context_t* ctx, vulkan_buffer_t* x_in, vulkan_buffer_t* x_out,
+                 int seq_len, int num_heads, int head_dim, float rope_theta) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !x_in || !x_out) return;
+    HIP_OP(ctx, "rope", seraph_rope(FPTR(x_in), FPTR(x_out), NULL, 1, seq_len, num_heads, head_dim, rope_theta, 0, st->stream));
+}
+
+void hip_rope_packed(vulkan_context_t* ctx, vulkan_buffer_t* x_in, vulkan_buffer_t* x_out, vulkan_buffer_t* seq_starts,
+                     int total_tokens, int batch_size, int num_heads, int head_dim, float rope_theta) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !x_in || !x_out || !seq_starts) return;
+    HIP_OP(ctx, "rope_packed", seraph_rope(FPTR(x_in), FPTR(x_out), UPTR(seq_starts), batch_size, total_tokens, num_heads, head_dim, rope_theta, 0, st->stream));
+}
+
+void vulkan_batch_attention(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulkan_buffer_t* K, vulkan_buffer_t* V,
+                            vulkan_buffer_t* out, int seq_len, int num_heads, int kv_heads, int head_dim) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !Q || !K || !V || !out) return;
+    float scale = 1.0f / sqrtf((float)head_dim);          /* src/vulkan_backend.c:2980-2984 */
+    HIP_OP(ctx, "batch_attention", seraph_attention_forward(FPTR(Q), FPTR(K), FPTR(V), FPTR(out), NULL, NULL, 1, seq_len,
+                                                            num_heads, kv_heads, head_dim, scale, st->stream));
+}
+
+void hip_batch_attention_packed(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulkan_buffer_t* K, vulkan_buffer_t* V,
+                                vulkan_buffer_t* out, vulkan_buffer_t* lse_out, vulkan_buffer_t* seq_starts,
+                                int total_tokens, int batch_size, int num_heads, int kv_heads, int head_dim) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !Q || !K || !V || !out || !seq_starts) return;
+    float scale = 1.0f / sqrtf((float)head_dim);
+    HIP_OP(ctx, "batch_attention_packed", seraph_attention_forward(FPTR(Q), FPTR(K), FPTR(V), FPTR(out), lse_out ? FPTR(lse_out) : NULL,
+                                                                   UPTR(seq_starts), batch_size, total_tokens,
+                                                                   num_heads, kv_heads, head_dim, scale, st->stream));
+}
+
+void vulkan_embed_lookup(vulkan_context_t* ctx, vulkan_buffer_t* tokens_u32, vulkan_buffer_t* embed_weight,
+                         vulkan_buffer_t* out_hidden, int seq_len, int hidden_size, int vocab_size) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !tokens_u32 || !embed_weight || !out_hidden) return;
+    HIP_OP(ctx, "embed_lookup", seraph_embed_lookup(UPTR(tokens_u32), FPTR(embed_weight), FPTR(out_hidden), seq_len, hidden_size, vocab_size, st->stream));
+}
+
+void vulkan_qk_norm(vulkan_context_t* ctx, vulkan_buffer_t* qk, int seq_len, int num_heads, int head_dim, int use_qk_norm, float eps) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !qk || !use_qk_norm) return;               /* src/vulkan_backend.c:3481 */
+    HIP_OP(ctx, "qk_norm", seraph_qk_norm(FPTR(qk), seq_len, num_heads, head_dim, use_qk_norm, eps, st->stream));
+}
+
+/* ------------------------------------------------------------------ optimizer */
+void hip_adamw_update_clipped(vulkan_context_t* ctx, vulkan_buffer_t* weight, vulkan_buffer_t* grad, vulkan_buffer_t* m,
+                              vulkan_buffer_t* v, float lr, float beta1, float beta2, float weight_decay, float eps,
+                              int step, size_t size, float clip) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !weight || !grad || !m || !v || size == 0) return;
+    HIP_OP(ctx, "adamw", seraph_adamw(FPTR(weight), FPTR(grad), FPTR(m), FPTR(v), size, lr, beta1, beta2, weight_decay, eps, step, clip, st->stream));
+}
+
+void vulkan_adamw_update(vulkan_context_t* ctx, vulkan_buffer_t* weight, vulkan_buffer_t* grad, vulkan_buffer_t* m,
+                         vulkan_buffer_t* v, float lr, float beta1, float beta2, float weight_decay, float eps,
+                         int step, size_t size) {
+    hip_adamw_update_clipped(ctx, weight, grad, m, v, lr, beta1, beta2, weight_decay, eps, step, size, 0.0f);
+}
+
+/* ------------------------------------------------------------------ video-mode ops
+ * Not on the LLM training path (reached only when num_queries > 0). */
+static void video_op_unsupported(vulkan_context_t* ctx, const char* name) {
+    static int warned = 0;
+    if (!warned) fprintf(stderr, "ERROR: %s: video-mode ops are not provided by the HIP backend\n", name);
+    warned = 1;
+    hip_state_t* st = hip_state(ctx);
+    if (st) st->errors++;
+}
+
+void vulkan_patch_extract(vulkan_context_t* ctx, vulkan_buffer_t* frame, vulkan_buffer_t* patches,
+                          int frame_h, int frame_w, int channels, int patch_t, int patch_h, int patch_w) {
+    (void)frame; (void)patches; (void)frame_h; (void)frame_w; (void)channels; (void)patch_t; (void)patch_h; (void)patch_w;
+    video_op_unsupported(ctx, "vulkan_patch_extract");
+}
+void vulkan_add_bias(vulkan_context_t* ctx, vulkan_buffer_t* data, vulkan_buffer_t* bias, int rows, int cols) {
+    (void)data; (void)bias; (void)rows; (void)cols;
+    video_op_unsupported(ctx, "vulkan_add_bias");
+}
+void vulkan_bce_loss_grad(vulkan_context_t* ctx, vulkan_buffer_t* logits, vulkan_buffer_t* targets,
+                          vulkan_buffer_t* grad_logits, vulkan_buffer_t* loss_out, size_t count) {
+    (void)logits; (void)targets; (void)grad_logits; (void)loss_out; (void)count;
+    video_op_unsupported(ctx, "vulkan_bce_loss_grad");
+}
+void vulkan_sum_cols(vulkan_context_t* ctx, vulkan_buffer_t* data, vulkan_buffer_t* out, int rows, int cols) {
+    (void)data; (void)out; (void)rows; (void)cols;
+    video_op_unsupported(ctx, "vulkan_sum_cols");
+}

@@ -1,0 +1,139 @@
+/*
+ * hip_backend_backward.c - loss, backward and scatter ops of the backend API (the
+ * counterpart of Seraph's src/vulkan_backend_backward.c) over the MI355X kernel library.
+ * Each function keeps the reference's signature and conventions: void return, NULL
+ * arguments ignored, outputs that the reference accumulates into are accumulated into.
+ */
+#include <math.h>
+
+#include "hip_backend_internal.h"
+
+/* src/vulkan_backend_backward.c:571-689 */
+void vulkan_cross_entropy_grad(vulkan_context_t* ctx, vulkan_buffer_t* logits, vulkan_buffer_t* targets_u32,
+                               vulkan_buffer_t* grad_logits, vulkan_buffer_t* loss_rows, int rows, int cols, int valid_rows) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !logits || !targets_u32 || !grad_logits || !loss_rows) return;
+    HIP_OP(ctx, "cross_entropy_grad", seraph_cross_entropy_grad(FPTR(logits), UPTR(targets_u32), FPTR(grad_logits), FPTR(loss_rows),
+                                                               NULL, 1, rows, cols, valid_rows, st->stream));
+}
+
+void hip_cross_entropy_grad_packed(vulkan_context_t* ctx, vulkan_buffer_t* logits, vulkan_buffer_t* targets_u32,
+                                   vulkan_buffer_t* grad_logits, vulkan_buffer_t* loss_rows, vulkan_buffer_t* seq_starts,
+                                   int total_tokens, int batch_size, int vocab_size, int num_valid_predictions) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !logits || !targets_u32 || !grad_logits || !loss_rows || !seq_starts) return;
+    HIP_OP(ctx, "cross_entropy_grad_packed", seraph_cross_entropy_grad(FPTR(logits), UPTR(targets_u32), FPTR(grad_logits), FPTR(loss_rows),
+                                                                      UPTR(seq_starts), batch_size, total_tokens, vocab_size,
+                                                                      num_valid_predictions, st->stream));
+}
+
+/* src/vulkan_backend_backward.c:691-800: 512 inputs per output (src/train.c:4906-4913) */
+void vulkan_reduce_sum(vulkan_context_t* ctx, vulkan_buffer_t* in_buf, vulkan_buffer_t* out_buf, size_t count) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !in_buf || !out_buf || count == 0) return;
+    HIP_OP(ctx, "reduce_sum", seraph_reduce_sum(FPTR(in_buf), FPTR(out_buf), count, st->stream));
+}
+
+/* src/vulkan_backend_backward.c:802-929 */
+void vulkan_rmsnorm_backward_batch(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* scale,
+                                   vulkan_buffer_t* grad_output, vulkan_buffer_t* grad_input, vulkan_buffer_t* grad_scale,
+                                   int rows, int cols, float eps) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !input || !scale || !grad_output || !grad_input || !grad_scale) return;
+    size_t need = seraph_rmsnorm_backward_ws_bytes(rows, cols);
+    void* ws = hip_backend_scratch(ctx, need);
+    if (!ws) return;
+    HIP_OP(ctx, "rmsnorm_backward_batch", seraph_rmsnorm_backward(FPTR(input), FPTR(scale), FPTR(grad_output), FPTR(grad_input),
+                                                                  FPTR(grad_scale), rows, cols, eps, ws, st->ws_bytes, st->stream));
+}
+
+/* src/vulkan_backend_backward.c:931-1045 */
+void vulkan_rope_backward(vulkan_context_t* ctx, vulkan_buffer_t* x_in, vulkan_buffer_t* x_out,
+                          int seq_len, int num_heads, int head_dim, float rope_theta) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !x_in || !x_out) return;
+    HIP_OP(ctx, "rope_backward", seraph_rope(FPTR(x_in), FPTR(x_out), NULL, 1, seq_len, num_heads, head_dim, rope_theta, 1, st->stream));
+}
+
+void hip_rope_backward_packed(vulkan_context_t* ctx, vulkan_buffer_t* x_in, vulkan_buffer_t* x_out, vulkan_buffer_t* seq_starts,
+                              int total_tokens, int batch_size, int num_heads, int head_dim, float rope_theta) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !x_in || !x_out || !seq_starts) return;
+    HIP_OP(ctx, "rope_backward_packed", seraph_rope(FPTR(x_in), FPTR(x_out), UPTR(seq_starts), batch_size, total_tokens, num_heads,
+                                                    head_dim, rope_theta, 1, st->stream));
+}
+
+/* src/vulkan_backend_backward.c:1047-1183.  The reference saves neither the attention output
+ * nor the log-sum-exp, so this entry point recomputes both; no sequence-length cap. */
+void vulkan_batch_attention_backward(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulkan_buffer_t* K, vulkan_buffer_t* V,
+                                     vulkan_buffer_t* grad_out, vulkan_buffer_t* grad_Q, vulkan_buffer_t* grad_K,
+                                     vulkan_buffer_t* grad_V, int seq_len, int num_heads, int kv_heads, int head_dim) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !Q || !K || !V || !grad_out || !grad_Q || !grad_K || !grad_V) return;
+    size_t need = seraph_attention_backward_ws_bytes(seq_len, num_heads, kv_heads, head_dim);
+    void* ws = hip_backend_scratch(ctx, need);
+    if (!ws) return;
+    float scale = 1.0f / sqrtf((float)head_dim);          /* :1168 */
+    HIP_OP(ctx, "batch_attention_backward", seraph_attention_backward(FPTR(Q), FPTR(K), FPTR(V), FPTR(grad_out), NULL, NULL,
+                                                                     FPTR(grad_Q), FPTR(grad_K), FPTR(grad_V), NULL, 1, seq_len,
+                                                                     num_heads, kv_heads, head_dim, scale, ws, st->ws_bytes, st->stream));
+}
+
+void hip_batch_attention_backward_packed(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulkan_buffer_t* K, vulkan_buffer_t* V,
+                                         vulkan_buffer_t* attn_out, vulkan_buffer_t* lse, vulkan_buffer_t* grad_out,
+                                         vulkan_buffer_t* grad_Q, vulkan_buffer_t* grad_K, vulkan_buffer_t* grad_V,
+                                         vulkan_buffer_t* seq_starts, int total_tokens, int batch_size,
+                                         int num_heads, int kv_heads, int head_dim) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !Q || !K || !V || !grad_out || !grad_Q || !grad_K || !grad_V || !seq_starts) return;
+    size_t need = seraph_attention_backward_ws_bytes(total_tokens, num_heads, kv_heads, head_dim);
+    void* ws = hip_backend_scratch(ctx, need);
+    if (!ws) return;
+    float scale = 1.0f / sqrtf((float)head_dim);
+    HIP_OP(ctx, "batch_attention_backward_packed",
+           seraph_attention_backward(FPTR(Q), FPTR(K), FPTR(V), FPTR(grad_out), attn_out ? FPTR(attn_out) : NULL, lse ? FPTR(lse) : NULL,
+                                     FPTR(grad_Q), FPTR(grad_K), FPTR(grad_V), UPTR(seq_starts), batch_size, total_tokens,
+                                     num_heads, kv_heads, head_dim, scale, ws, st->ws_bytes, st->stream));
+}
+
+/* src/vulkan_backend_backward.c:1185-1300 */
+void vulkan_embedding_backward(vulkan_context_t* ctx, vulkan_buffer_t* tokens_u32, vulkan_buffer_t* grad_hidden,
+                               vulkan_buffer_t* grad_embed, int seq_len, int hidden_size, int vocab_size) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !tokens_u32 || !grad_hidden || !grad_embed) return;
+    size_t need = seraph_embedding_backward_ws_bytes(seq_len, vocab_size);
+    void* ws = hip_backend_scratch(ctx, need);
+    if (!ws) return;
+    HIP_OP(ctx, "embedding_backward", seraph_embedding_backward(UPTR(tokens_u32), FPTR(grad_hidden), FPTR(grad_embed), seq_len,
+                                                                hidden_size, vocab_size, ws, st->ws_bytes, st->stream));
+}
+
+/* src/vulkan_backend_backward.c:159-297 */
+void vulkan_silu_backward(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* grad_output,
+                          vulkan_buffer_t* grad_input, size_t count) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !input || !grad_output || !grad_input) return;
+    HIP_OP(ctx, "silu_backward", seraph_silu_backward(FPTR(input), FPTR(grad_output), FPTR(grad_input), count, st->stream));
+}
+
+/* src/vulkan_backend_backward.c:300-452 */
+void vulkan_elementwise_mul_backward(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* grad_C,
+                                     vulkan_buffer_t* grad_A, vulkan_buffer_t* grad_B, size_t count) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !A || !B || !grad_C || !grad_A || !grad_B) return;
+    HIP_OP(ctx, "elementwise_mul_backward", seraph_mul_backward(FPTR(A), FPTR(B), FPTR(grad_C), FPTR(grad_A), FPTR(grad_B), count, st->stream));
+}
+
+void hip_swiglu_backward(vulkan_context_t* ctx, vulkan_buffer_t* gate, vulkan_buffer_t* up, vulkan_buffer_t* grad_hidden,
+                         vulkan_buffer_t* grad_gate, vulkan_buffer_t* grad_up, size_t count) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !gate || !up || !grad_hidden || !grad_gate || !grad_up) return;
+    HIP_OP(ctx, "silu_mul_backward", seraph_swiglu_backward(FPTR(gate), FPTR(up), FPTR(grad_hidden), FPTR(grad_gate), FPTR(grad_up), count, st->stream));
+}
+
+void hip_qk_norm_backward(vulkan_context_t* ctx, vulkan_buffer_t* qk_pre, vulkan_buffer_t* grad_out, vulkan_buffer_t* grad_in,
+                          int seq_len, int num_heads, int head_dim, float eps) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !qk_pre || !grad_out || !grad_in) return;
+    HIP_OP(ctx, "qk_norm_backward", seraph_qk_norm_backward(FPTR(qk_pre), FPTR(grad_out), FPTR(grad_in), seq_len, num_heads, head_dim, eps, st->stream));
+}

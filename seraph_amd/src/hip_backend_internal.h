@@ -1,0 +1,51 @@
+/* hip_backend_internal.h - private state shared by hip_backend.c and hip_backend_backward.c */
+#ifndef HIP_BACKEND_INTERNAL_H
+#define HIP_BACKEND_INTERNAL_H
+
+#include <stdio.h>
+
+#include "hip_backend.h"
+#include "seraph_hip.h"
+
+#define HIP_PROF_MAX_OPS 8192
+
+typedef struct {
+    const char* name;
+    void* ev_start;
+    void* ev_stop;
+} hip_prof_op_t;
+
+typedef struct {
+    seraph_stream_t stream;
+    int recording;               /* between vulkan_cmd_begin and vulkan_cmd_end_submit */
+    void* ws;                    /* device scratch shared by the ops that need one */
+    size_t ws_bytes;
+    int errors;
+    /* profiler: one event pair per op of the current step */
+    hip_prof_op_t* prof_ops;
+    int prof_count;
+    int prof_events_made;
+} hip_state_t;
+
+static inline hip_state_t* hip_state(vulkan_context_t* ctx) { return ctx ? (hip_state_t*)ctx->device : NULL; }
+
+/* Grows the shared scratch to at least `bytes`; returns NULL on failure. */
+void* hip_backend_scratch(vulkan_context_t* ctx, size_t bytes);
+void hip_backend_report(vulkan_context_t* ctx, const char* op, int rc);
+void hip_prof_begin(vulkan_context_t* ctx, const char* name);
+void hip_prof_end(vulkan_context_t* ctx);
+
+/* Runs one kernel-library call for op `name`: timing when profiling, error report when it fails. */
+#define HIP_OP(ctx, name, call)                       \
+    do {                                              \
+        hip_prof_begin((ctx), (name));                \
+        int rc_ = (call);                             \
+        hip_prof_end((ctx));                          \
+        if (rc_ != SERAPH_OK) hip_backend_report((ctx), (name), rc_); \
+    } while (0)
+
+#define DPTR(buf) ((buf)->buffer)
+#define FPTR(buf) ((float*)(buf)->buffer)
+#define UPTR(buf) ((uint32_t*)(buf)->buffer)
+
+#endif

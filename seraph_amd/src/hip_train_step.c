@@ -1,0 +1,563 @@
+/*
+ * hip_train_step.c - packed-batch full-weight and LoRA training steps (see hip_train.h).
+ * Plain C over the kernel library's C ABI; one in-order stream, no host round trips
+ * between the token upload and the 4-byte loss download.
+ */
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "hip_train.h"
+#include "seraph_hip.h"
+
+#define CK(call)                                                                         \
+    do {                                                                                 \
+        int rc_ = (call);                                                                \
+        if (rc_ != SERAPH_OK) {                                                          \
+            fprintf(stderr, "ERROR: %s failed (%d): %s\n", #call, rc_, seraph_hip_last_error()); \
+            return -1;                                                                   \
+        }                                                                                \
+    } while (0)
+
+#define OPT_MAX_CLASSES 48
+#define OPT_MAX_EVENTS  32768
+
+typedef struct { int64_t in_norm, q, k, v, o, post_norm, gate, up, down, stride; } layer_layout_t;
+typedef struct { int64_t A[4], B[4], in[4], out[4], stride; } lora_layout_t;
+
+typedef struct {
+    float *layer_in, *xn_attn, *q, *k, *v, *attn_out, *lse, *post_in, *xn_ffn, *gate, *up, *ffn_h;
+} layer_act_t;
+
+struct hip_trainer {
+    hip_model_config_t cfg;
+    hip_optim_config_t opt;
+    int max_tokens, max_batch, lora;
+    int64_t nparams, nlora;
+    int64_t off_embed, off_final_norm, off_layer0;
+    layer_layout_t L;
+    lora_layout_t LL;
+    seraph_stream_t stream;
+    /* arenas */
+    float *P, *G, *M, *V;
+    int own_P, own_G, own_M, own_V;
+    float *LP, *LG, *LM, *LV;
+    /* activations */
+    char* act_arena;
+    size_t act_bytes;
+    layer_act_t* act;
+    float *final_in, *xn_final, *logits, *loss_rows, *red_a, *red_b, *tmp_h, *lora_tmp;
+    float *g_hidden, *g_tmp, *g_xn, *g_ffn, *g_gate, *g_up, *g_attn, *g_q, *g_k, *g_v, *scratch_gs;
+    uint32_t *d_tokens, *d_targets, *d_starts;
+    uint32_t* h_stage;           /* pinned: tokens | targets | starts */
+    void* ws;
+    size_t ws_bytes;
+    size_t device_bytes;
+    /* bookkeeping of src/train.c:5439-5463 */
+    int accumulation_counter, optimizer_step;
+    float last_lr;
+    double attn_pairs;           /* sum over sequences of S(S+1)/2 for the current batch */
+    void* ev[4];
+    float phase_ms[3];
+    /* optional per-op timing: one event pair per kernel-library call, folded per kernel class */
+    int op_timing;
+    hip_op_stat_t op_stats[OPT_MAX_CLASSES];
+    int op_classes;
+    void** op_ev;                /* [2 * OPT_MAX_EVENTS], created on demand */
+    int op_ev_made, op_ev_used;
+    int op_ev_class[OPT_MAX_EVENTS];
+};
+
+static int op_class(hip_trainer_t* t, const char* name) {
+    for (int i = 0; i < t->op_classes; i++)
+        if (t->op_stats[i].name == name || strcmp(t->op_stats[i].name, name) == 0) return i;
+    if (t->op_classes >= OPT_MAX_CLASSES) return -1;
+    memset(&t->op_stats[t->op_classes], 0, sizeof(hip_op_stat_t));
+    t->op_stats[t->op_classes].name = name;
+    return t->op_classes++;
+}
+
+/* Brackets one kernel-library call with events when op timing is on. */
+static int op_begin(hip_trainer_t* t, const char* name, double flops, double bytes) {
+    if (!t->op_timing || t->op_ev_used >= OPT_MAX_EVENTS) return -1;
+    int c = op_class(t, name);
+    if (c < 0) return -1;
+    if (!t->op_ev) t->op_ev = (void**)calloc(2 * OPT_MAX_EVENTS, sizeof(void*));
+    if (!t->op_ev) return -1;
+    int i = t->op_ev_used;
+    if (i >= t->op_ev_made) {
+        if (seraph_hip_event_create(&t->op_ev[2 * i]) != SERAPH_OK || seraph_hip_event_create(&t->op_ev[2 * i + 1]) != SERAPH_OK) return -1;
+        t->op_ev_made = i + 1;
+    }
+    t->op_stats[c].launches++;
+    t->op_stats[c].flops += flops;
+    t->op_stats[c].bytes += bytes;
+    t->op_ev_class[i] = c;
+    seraph_hip_event_record(t->op_ev[2 * i], t->stream);
+    return i;
+}
+
+static void op_end(hip_trainer_t* t, int i) {
+    if (i < 0) return;
+    seraph_hip_event_record(t->op_ev[2 * i + 1], t->stream);
+    t->op_ev_used = i + 1;
+}
+
+static void op_fold(hip_trainer_t* t) {
+    for (int i = 0; i < t->op_ev_used; i++) {
+        float ms = 0.f;
+        if (seraph_hip_event_elapsed_ms(t->op_ev[2 * i], t->op_ev[2 * i + 1], &ms) == SERAPH_OK)
+            t->op_stats[t->op_ev_class[i]].ms += ms;
+    }
+    t->op_ev_used = 0;
+}
+
+#define OP(name, flops, bytes, call)                     \
+    do {                                                 \
+        int oi_ = op_begin(t, (name), (flops), (bytes)); \
+        int rc_ = (call);                                \
+        op_end(t, oi_);                                  \
+        if (rc_ != SERAPH_OK) {                          \
+            fprintf(stderr, "ERROR: %s failed (%d): %s\n", #call, rc_, seraph_hip_last_error()); \
+            return -1;                                   \
+        }                                                \
+    } while (0)
+
+/* GEMM through the kernel library, classed by the kernel instantiation that will run */
+#define GEMM(A_, B_, C_, M_, N_, K_, tA_, tB_, acc_)                                                   \
+    OP(seraph_gemm_kernel_name((M_), (N_), (K_), (tA_), (tB_)), 2.0 * (double)(M_) * (double)(N_) * (double)(K_), 0.0, \
+       seraph_gemm((A_), (B_), (C_), (M_), (N_), (K_), (tA_), (tB_), (acc_), t->stream))
+
+
+/* ------------------------------------------------------------------ layouts */
+static void make_layouts(hip_trainer_t* t) {
+    const hip_model_config_t* c = &t->cfg;
+    int64_t h = c->hidden, qd = (int64_t)c->heads * c->head_dim, kv = (int64_t)c->kv_heads * c->head_dim, f = c->ffn;
+    t->off_embed = 0;
+    t->off_final_norm = (int64_t)c->vocab * h;
+    t->off_layer0 = t->off_final_norm + h;
+    int64_t o = 0;
+    t->L.in_norm = o; o += h;
+    t->L.q = o; o += qd * h;
+    t->L.k = o; o += kv * h;
+    t->L.v = o; o += kv * h;
+    t->L.o = o; o += h * qd;
+    t->L.post_norm = o; o += h;
+    t->L.gate = o; o += f * h;
+    t->L.up = o; o += f * h;
+    t->L.down = o; o += h * f;
+    t->L.stride = o;
+    t->nparams = t->off_layer0 + o * c->layers;
+    int64_t ins[4] = {h, h, h, qd}, outs[4] = {qd, kv, kv, h};
+    o = 0;
+    for (int p = 0; p < 4; p++) {
+        t->LL.in[p] = ins[p]; t->LL.out[p] = outs[p];
+        t->LL.A[p] = t->LL.B[p] = -1;
+        if (c->lora_rank > 0 && ((c->lora_mask >> p) & 1)) {
+            t->LL.A[p] = o; o += (int64_t)c->lora_rank * ins[p];
+            t->LL.B[p] = o; o += outs[p] * (int64_t)c->lora_rank;
+        }
+    }
+    t->LL.stride = o;
+    t->nlora = o * c->layers;
+}
+
+int64_t hip_param_count(const hip_model_config_t* cfg) {
+    hip_trainer_t tmp;
+    memset(&tmp, 0, sizeof(tmp));
+    tmp.cfg = *cfg;
+    make_layouts(&tmp);
+    return tmp.nparams;
+}
+
+int64_t hip_lora_param_count(const hip_model_config_t* cfg) {
+    hip_trainer_t tmp;
+    memset(&tmp, 0, sizeof(tmp));
+    tmp.cfg = *cfg;
+    make_layouts(&tmp);
+    return tmp.nlora;
+}
+
+/* ------------------------------------------------------------------ create / free */
+static size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+static int dev_alloc(hip_trainer_t* t, void** p, size_t bytes) {
+    if (seraph_hip_malloc(p, bytes) != SERAPH_OK) {
+        fprintf(stderr, "ERROR: device allocation of %zu bytes failed: %s\n", bytes, seraph_hip_last_error());
+        return -1;
+    }
+    t->device_bytes += bytes;
+    return 0;
+}
+
+static size_t max_sz(size_t a, size_t b) { return a > b ? a : b; }
+
+hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim_config_t* opt,
+                                  int max_tokens, int max_batch, int device_index,
+                                  float* ext_params, float* ext_grads, float* ext_m, float* ext_v) {
+    if (!cfg || !opt || max_tokens < 2 || max_batch < 1) return NULL;
+    if (cfg->heads % cfg->kv_heads != 0 || cfg->hidden % 4 != 0 || cfg->ffn % 4 != 0 ||
+        !(cfg->head_dim == 32 || cfg->head_dim == 64 || cfg->head_dim == 128)) {
+        fprintf(stderr, "ERROR: unsupported model shape (heads %% kv_heads, hidden/ffn %% 4, head_dim in {32,64,128})\n");
+        return NULL;
+    }
+    if (seraph_hip_init(device_index) != SERAPH_OK) {
+        fprintf(stderr, "ERROR: %s\n", seraph_hip_last_error());
+        return NULL;
+    }
+    hip_trainer_t* t = (hip_trainer_t*)calloc(1, sizeof(*t));
+    if (!t) return NULL;
+    t->cfg = *cfg; t->opt = *opt;
+    t->max_tokens = max_tokens; t->max_batch = max_batch;
+    t->lora = cfg->lora_rank > 0;
+    make_layouts(t);
+    if (seraph_hip_stream_create(&t->stream) != SERAPH_OK) goto fail;
+    for (int i = 0; i < 4; i++) if (seraph_hip_event_create(&t->ev[i]) != SERAPH_OK) goto fail;
+
+    const size_t pbytes = (size_t)t->nparams * sizeof(float);
+    t->P = ext_params;
+    if (!t->P) { if (dev_alloc(t, (void**)&t->P, pbytes)) goto fail; t->own_P = 1; }
+    if (!t->lora) {
+        t->G = ext_grads; t->M = ext_m; t->V = ext_v;
+        if (!t->G) { if (dev_alloc(t, (void**)&t->G, pbytes)) goto fail; t->own_G = 1; }
+        if (!t->M) { if (dev_alloc(t, (void**)&t->M, pbytes)) goto fail; t->own_M = 1; }
+        if (!t->V) { if (dev_alloc(t, (void**)&t->V, pbytes)) goto fail; t->own_V = 1; }
+        if (t->own_G && seraph_fill_u32(t->G, 0, (size_t)t->nparams, t->stream) != SERAPH_OK) goto fail;
+        if (t->own_M && seraph_fill_u32(t->M, 0, (size_t)t->nparams, t->stream) != SERAPH_OK) goto fail;
+        if (t->own_V && seraph_fill_u32(t->V, 0, (size_t)t->nparams, t->stream) != SERAPH_OK) goto fail;
+    } else {
+        const size_t lbytes = (size_t)t->nlora * sizeof(float);
+        if (dev_alloc(t, (void**)&t->LP, lbytes) || dev_alloc(t, (void**)&t->LG, lbytes) ||
+            dev_alloc(t, (void**)&t->LM, lbytes) || dev_alloc(t, (void**)&t->LV, lbytes)) goto fail;
+        float* all[4] = {t->LP, t->LG, t->LM, t->LV};
+        for (int i = 0; i < 4; i++) if (seraph_fill_u32(all[i], 0, (size_t)t->nlora, t->stream) != SERAPH_OK) goto fail;
+    }
+
+    /* activation arena */
+    {
+        const size_t T = (size_t)max_tokens, h = (size_t)cfg->hidden, f = (size_t)cfg->ffn, Vv = (size_t)cfg->vocab;
+        const size_t qd = (size_t)cfg->heads * cfg->head_dim, kv = (size_t)cfg->kv_heads * cfg->head_dim;
+        const size_t r = cfg->lora_rank > 0 ? (size_t)cfg->lora_rank : 1;
+        const size_t per_layer = 4 * up256(T * h * 4) + 2 * up256(T * qd * 4) + 2 * up256(T * kv * 4) +
+                                 up256(T * cfg->heads * 4) + 3 * up256(T * f * 4);
+        const size_t rest = 2 * up256(T * h * 4) + up256(T * Vv * 4) + 3 * up256(T * 4) + up256(T * h * 4) + up256(T * r * 4) +
+                            3 * up256(T * h * 4) + 3 * up256(T * f * 4) + 2 * up256(T * qd * 4) + 2 * up256(T * kv * 4) +
+                            up256(h * 4) + 2 * up256(T * 4) + up256(((size_t)max_batch + 1) * 4);
+        t->act_bytes = per_layer * (size_t)cfg->layers + rest;
+        if (dev_alloc(t, (void**)&t->act_arena, t->act_bytes)) goto fail;
+        t->act = (layer_act_t*)calloc((size_t)cfg->layers, sizeof(layer_act_t));
+        if (!t->act) goto fail;
+        char* p = t->act_arena;
+#define TAKE(dst, bytes) do { (dst) = (void*)p; p += up256(bytes); } while (0)
+        for (int l = 0; l < cfg->layers; l++) {
+            layer_act_t* a = &t->act[l];
+            TAKE(a->layer_in, T * h * 4); TAKE(a->xn_attn, T * h * 4); TAKE(a->post_in, T * h * 4); TAKE(a->xn_ffn, T * h * 4);
+            TAKE(a->q, T * qd * 4); TAKE(a->attn_out, T * qd * 4); TAKE(a->k, T * kv * 4); TAKE(a->v, T * kv * 4);
+            TAKE(a->lse, T * cfg->heads * 4);
+            TAKE(a->gate, T * f * 4); TAKE(a->up, T * f * 4); TAKE(a->ffn_h, T * f * 4);
+        }
+        TAKE(t->final_in, T * h * 4); TAKE(t->xn_final, T * h * 4); TAKE(t->logits, T * Vv * 4);
+        TAKE(t->loss_rows, T * 4); TAKE(t->red_a, T * 4); TAKE(t->red_b, T * 4);
+        TAKE(t->tmp_h, T * h * 4); TAKE(t->lora_tmp, T * r * 4);
+        TAKE(t->g_hidden, T * h * 4); TAKE(t->g_tmp, T * h * 4); TAKE(t->g_xn, T * h * 4);
+        TAKE(t->g_ffn, T * f * 4); TAKE(t->g_gate, T * f * 4); TAKE(t->g_up, T * f * 4);
+        TAKE(t->g_attn, T * qd * 4); TAKE(t->g_q, T * qd * 4); TAKE(t->g_k, T * kv * 4); TAKE(t->g_v, T * kv * 4);
+        TAKE(t->scratch_gs, h * 4);
+        TAKE(t->d_tokens, T * 4); TAKE(t->d_targets, T * 4); TAKE(t->d_starts, ((size_t)max_batch + 1) * 4);
+#undef TAKE
+        if ((size_t)(p - t->act_arena) > t->act_bytes) { fprintf(stderr, "ERROR: activation arena layout overflow\n"); goto fail; }
+    }
+    t->ws_bytes = max_sz(seraph_rmsnorm_backward_ws_bytes(max_tokens, cfg->hidden),
+                         max_sz(seraph_attention_backward_ws_bytes(max_tokens, cfg->heads, cfg->kv_heads, cfg->head_dim),
+                                seraph_embedding_backward_ws_bytes(max_tokens, cfg->vocab)));
+    if (dev_alloc(t, &t->ws, t->ws_bytes)) goto fail;
+    if (seraph_hip_host_alloc((void**)&t->h_stage, ((size_t)2 * max_tokens + max_batch + 1) * 4) != SERAPH_OK) goto fail;
+    if (seraph_hip_stream_sync(t->stream) != SERAPH_OK) goto fail;
+    return t;
+fail:
+    fprintf(stderr, "ERROR: hip_trainer_create failed: %s\n", seraph_hip_last_error());
+    hip_trainer_free(t);
+    return NULL;
+}
+
+void hip_trainer_free(hip_trainer_t* t) {
+    if (!t) return;
+    if (t->stream) seraph_hip_stream_sync(t->stream);
+    if (t->own_P) seraph_hip_free(t->P);
+    if (t->own_G) seraph_hip_free(t->G);
+    if (t->own_M) seraph_hip_free(t->M);
+    if (t->own_V) seraph_hip_free(t->V);
+    seraph_hip_free(t->LP); seraph_hip_free(t->LG); seraph_hip_free(t->LM); seraph_hip_free(t->LV);
+    seraph_hip_free(t->act_arena);
+    seraph_hip_free(t->ws);
+    seraph_hip_host_free(t->h_stage);
+    for (int i = 0; i < 4; i++) seraph_hip_event_destroy(t->ev[i]);
+    if (t->op_ev) {
+        for (int i = 0; i < 2 * t->op_ev_made; i++) seraph_hip_event_destroy(t->op_ev[i]);
+        free(t->op_ev);
+    }
+    seraph_hip_stream_destroy(t->stream);
+    free(t->act);
+    free(t);
+}
+
+static float* arena_of(hip_trainer_t* t, int which, int64_t* count) {
+    float* all[8] = {t->P, t->G, t->M, t->V, t->LP, t->LG, t->LM, t->LV};
+    if (which < 0 || which > 7) return NULL;
+    *count = which < 4 ? t->nparams : t->nlora;
+    return all[which];
+}
+
+int hip_trainer_upload(hip_trainer_t* t, int which, const float* host, int64_t count) {
+    int64_t n = 0;
+    float* d = t ? arena_of(t, which, &n) : NULL;
+    if (!d || !host || count != n) return -1;
+    return seraph_hip_h2d(d, host, (size_t)n * 4, t->stream) == SERAPH_OK ? 0 : -1;
+}
+
+int hip_trainer_download(hip_trainer_t* t, int which, float* host, int64_t count) {
+    int64_t n = 0;
+    float* d = t ? arena_of(t, which, &n) : NULL;
+    if (!d || !host || count != n) return -1;
+    return seraph_hip_d2h(host, d, (size_t)n * 4, t->stream) == SERAPH_OK ? 0 : -1;
+}
+
+void* hip_trainer_device_ptr(hip_trainer_t* t, int which) {
+    int64_t n;
+    return t ? (void*)arena_of(t, which, &n) : NULL;
+}
+
+int hip_trainer_optimizer_step(const hip_trainer_t* t) { return t ? t->optimizer_step : -1; }
+float hip_trainer_last_lr(const hip_trainer_t* t) { return t ? t->last_lr : 0.0f; }
+size_t hip_trainer_device_bytes(const hip_trainer_t* t) { return t ? t->device_bytes : 0; }
+void hip_trainer_last_timing(const hip_trainer_t* t, float ms[3]) {
+    for (int i = 0; i < 3; i++) ms[i] = t ? t->phase_ms[i] : 0.0f;
+}
+
+void hip_trainer_enable_op_timing(hip_trainer_t* t, int on) { if (t) t->op_timing = on ? 1 : 0; }
+void hip_trainer_reset_op_stats(hip_trainer_t* t) { if (t) { t->op_classes = 0; t->op_ev_used = 0; } }
+int hip_trainer_op_stats(const hip_trainer_t* t, hip_op_stat_t* out, int max) {
+    if (!t || !out) return 0;
+    int n = t->op_classes < max ? t->op_classes : max;
+    memcpy(out, t->op_stats, (size_t)n * sizeof(hip_op_stat_t));
+    return n;
+}
+
+/* ------------------------------------------------------------------ the step */
+/* out (+)= ((x A^T) s) B^T, src/train.c:5778-5796 */
+static int lora_forward_add(hip_trainer_t* t, const float* x, float* out, const float* A, const float* B,
+                            int64_t T, int64_t in, int64_t outd) {
+    const int r = t->cfg.lora_rank;
+    const float s = t->cfg.lora_alpha / (float)r;
+    GEMM(x, A, t->lora_tmp, T, r, in, 0, 1, 0);
+    OP("scale", 0.0, 8.0 * (double)(T * r), seraph_scale(t->lora_tmp, (size_t)(T * r), s, t->stream));
+    GEMM(t->lora_tmp, B, out, T, outd, r, 0, 1, 1);
+    return 0;
+}
+
+/* src/train.c:5803-5845 with grad_input == NULL, as every call site passes it */
+static int lora_backward(hip_trainer_t* t, const float* dY, const float* x, const float* A, const float* B,
+                         float* gA, float* gB, int64_t T, int64_t in, int64_t outd) {
+    const int r = t->cfg.lora_rank;
+    const float s = t->cfg.lora_alpha / (float)r;
+    GEMM(x, A, t->lora_tmp, T, r, in, 0, 1, 0);
+    OP("scale", 0.0, 8.0 * (double)(T * r), seraph_scale(t->lora_tmp, (size_t)(T * r), s, t->stream));
+    GEMM(dY, t->lora_tmp, gB, outd, r, T, 1, 0, 1);
+    GEMM(dY, B, t->lora_tmp, T, r, outd, 0, 0, 0);
+    OP("scale", 0.0, 8.0 * (double)(T * r), seraph_scale(t->lora_tmp, (size_t)(T * r), s, t->stream));
+    GEMM(t->lora_tmp, x, gA, r, in, T, 1, 0, 1);
+    return 0;
+}
+
+static int upload_batch(hip_trainer_t* t, const int* tokens, int T, const int* seq_starts, int batch) {
+    uint32_t* tok = t->h_stage;
+    uint32_t* tgt = tok + T;
+    uint32_t* st = tgt + T;
+    for (int b = 0; b <= batch; b++) st[b] = seq_starts ? (uint32_t)seq_starts[b] : (b == 0 ? 0u : (uint32_t)T);
+    if (st[0] != 0 || st[batch] != (uint32_t)T) { fprintf(stderr, "ERROR: seq_starts must run from 0 to total_tokens\n"); return -1; }
+    t->attn_pairs = 0.0;
+    for (int b = 0; b < batch; b++) {
+        if (st[b + 1] > st[b]) t->attn_pairs += 0.5 * (double)(st[b + 1] - st[b]) * (double)(st[b + 1] - st[b] + 1);
+        if (st[b + 1] <= st[b]) { fprintf(stderr, "ERROR: empty or decreasing sequence %d in seq_starts\n", b); return -1; }
+        for (uint32_t i = st[b]; i < st[b + 1]; i++) {                     /* src/train_cuda.c:2029-2043 */
+            tok[i] = tokens[i] < 0 ? 0u : (uint32_t)tokens[i];
+            tgt[i] = (i + 1 < st[b + 1]) ? (tokens[i + 1] < 0 ? 0u : (uint32_t)tokens[i + 1]) : 0u;
+        }
+    }
+    CK(seraph_hip_h2d(t->d_tokens, tok, (size_t)T * 4, t->stream));
+    CK(seraph_hip_h2d(t->d_targets, tgt, (size_t)T * 4, t->stream));
+    CK(seraph_hip_h2d(t->d_starts, st, ((size_t)batch + 1) * 4, t->stream));
+    return 0;
+}
+
+static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, const int* seq_starts, int batch,
+                      int run_optimizer) {
+    if (!t || !tokens || total_tokens < 2 || batch < 1) return -1.0f;
+    if (total_tokens > t->max_tokens || batch > t->max_batch) {
+        fprintf(stderr, "ERROR: batch of %d tokens / %d sequences exceeds the trainer's capacity (%d / %d)\n",
+                total_tokens, batch, t->max_tokens, t->max_batch);
+        return -1.0f;
+    }
+    if (!seq_starts && batch != 1) return -1.0f;
+    const hip_model_config_t* c = &t->cfg;
+    const int lora = t->lora;
+    const int64_t T = total_tokens, h = c->hidden, f = c->ffn, V = c->vocab;
+    const int H = c->heads, KVH = c->kv_heads, D = c->head_dim, NL = c->layers;
+    const int64_t qd = (int64_t)H * D, kv = (int64_t)KVH * D;
+    const float scale = 1.0f / sqrtf((float)D);
+    const float eps = c->rms_eps, theta = c->rope_theta > 0 ? c->rope_theta : 10000.0f;
+    const int num_valid = total_tokens - batch;                         /* src/train_cuda.c:1989-1991 */
+    if (num_valid <= 0) return 0.0f;
+    seraph_stream_t s = t->stream;
+    const float* P = t->P;
+
+    if (upload_batch(t, tokens, total_tokens, seq_starts, batch)) return -1.0f;
+    const uint32_t* starts = t->d_starts;
+
+    if (t->accumulation_counter == 0) {                                  /* src/train.c:4399-4400 */
+        if (lora) OP("fill", 0.0, 4.0 * (double)t->nlora, seraph_fill_u32(t->LG, 0, (size_t)t->nlora, s));
+        else OP("fill", 0.0, 4.0 * (double)t->nparams, seraph_fill_u32(t->G, 0, (size_t)t->nparams, s));
+    }
+    CK(seraph_hip_event_record(t->ev[0], s));
+
+    /* ---------------- forward */
+    OP("embed_lookup", 0.0, 8.0 * (double)(T * h), seraph_embed_lookup(t->d_tokens, P + t->off_embed, t->act[0].layer_in, T, h, V, s));
+    for (int l = 0; l < NL; l++) {
+        const float* W = P + t->off_layer0 + t->L.stride * l;
+        const float* LW = lora ? t->LP + t->LL.stride * l : NULL;
+        layer_act_t* a = &t->act[l];
+        float* next = (l + 1 < NL) ? t->act[l + 1].layer_in : t->final_in;
+        OP("rmsnorm", 0.0, 8.0 * (double)(T * h), seraph_rmsnorm(a->layer_in, W + t->L.in_norm, a->xn_attn, T, h, eps, s));
+        GEMM(a->xn_attn, W + t->L.q, a->q, T, qd, h, 0, 1, 0);
+        if (lora && t->LL.A[0] >= 0 && lora_forward_add(t, a->xn_attn, a->q, LW + t->LL.A[0], LW + t->LL.B[0], T, h, qd)) return -1.0f;
+        GEMM(a->xn_attn, W + t->L.k, a->k, T, kv, h, 0, 1, 0);
+        if (lora && t->LL.A[1] >= 0 && lora_forward_add(t, a->xn_attn, a->k, LW + t->LL.A[1], LW + t->LL.B[1], T, h, kv)) return -1.0f;
+        GEMM(a->xn_attn, W + t->L.v, a->v, T, kv, h, 0, 1, 0);
+        if (lora && t->LL.A[2] >= 0 && lora_forward_add(t, a->xn_attn, a->v, LW + t->LL.A[2], LW + t->LL.B[2], T, h, kv)) return -1.0f;
+        OP("rope", 0.0, 8.0 * (double)(T * qd), seraph_rope(a->q, a->q, starts, batch, T, H, D, theta, 0, s));
+        OP("rope", 0.0, 8.0 * (double)(T * kv), seraph_rope(a->k, a->k, starts, batch, T, KVH, D, theta, 0, s));
+        OP("attention_forward", 4.0 * D * t->attn_pairs * H, 0.0, seraph_attention_forward(a->q, a->k, a->v, a->attn_out, a->lse, starts, batch, T, H, KVH, D, scale, s));
+        GEMM(a->attn_out, W + t->L.o, t->tmp_h, T, h, qd, 0, 1, 0);
+        if (lora && t->LL.A[3] >= 0 && lora_forward_add(t, a->attn_out, t->tmp_h, LW + t->LL.A[3], LW + t->LL.B[3], T, qd, h)) return -1.0f;
+        OP("add", 0.0, 12.0 * (double)(T * h), seraph_add(a->layer_in, t->tmp_h, a->post_in, (size_t)(T * h), s));
+        OP("rmsnorm", 0.0, 8.0 * (double)(T * h), seraph_rmsnorm(a->post_in, W + t->L.post_norm, a->xn_ffn, T, h, eps, s));
+        GEMM(a->xn_ffn, W + t->L.gate, a->gate, T, f, h, 0, 1, 0);
+        GEMM(a->xn_ffn, W + t->L.up, a->up, T, f, h, 0, 1, 0);
+        OP("swiglu", 0.0, 12.0 * (double)(T * f), seraph_swiglu(a->gate, a->up, a->ffn_h, (size_t)(T * f), s));
+        GEMM(a->ffn_h, W + t->L.down, t->tmp_h, T, h, f, 0, 1, 0);
+        OP("add", 0.0, 12.0 * (double)(T * h), seraph_add(a->post_in, t->tmp_h, next, (size_t)(T * h), s));
+    }
+    OP("rmsnorm", 0.0, 8.0 * (double)(T * h), seraph_rmsnorm(t->final_in, P + t->off_final_norm, t->xn_final, T, h, eps, s));
+    GEMM(t->xn_final, P + t->off_embed, t->logits, T, V, h, 0, 1, 0);      /* tied head, src/train.c:4869-4872 */
+
+    /* ---------------- loss: gradient written over the logits */
+    OP("cross_entropy_grad", 0.0, 8.0 * (double)T * (double)V + 8.0 * (double)T, seraph_cross_entropy_grad(t->logits, t->d_targets, t->logits, t->loss_rows, starts, batch, T, V, num_valid, s));
+    float* red_in = t->loss_rows;
+    float* red_out = t->red_a;
+    for (size_t n = (size_t)T; n > 1; n = (n + 511) / 512) {                              /* src/train.c:4902-4913 */
+        CK(seraph_reduce_sum(red_in, red_out, n, s));
+        red_in = red_out;
+        red_out = (red_out == t->red_a) ? t->red_b : t->red_a;
+    }
+    CK(seraph_hip_event_record(t->ev[1], s));
+
+    /* ---------------- backward */
+    float* glog = t->logits;
+    GEMM(glog, P + t->off_embed, t->g_hidden, T, h, V, 0, 0, 0);            /* LM head dgrad */
+    if (!lora) GEMM(glog, t->xn_final, t->G + t->off_embed, V, h, T, 1, 0, 1); /* LM head wgrad */
+    OP("rmsnorm_backward", 0.0, 12.0 * (double)(T * h), seraph_rmsnorm_backward(t->final_in, P + t->off_final_norm, t->g_hidden, t->g_tmp,
+                               lora ? t->scratch_gs : t->G + t->off_final_norm, T, h, eps, t->ws, t->ws_bytes, s));
+    { float* sw = t->g_hidden; t->g_hidden = t->g_tmp; t->g_tmp = sw; }                   /* grad_hidden = grad_tmp (copy, src/train.c:5089) */
+
+    for (int l = NL - 1; l >= 0; l--) {
+        const float* W = P + t->off_layer0 + t->L.stride * l;
+        float* GW = lora ? NULL : t->G + t->off_layer0 + t->L.stride * l;
+        const float* LW = lora ? t->LP + t->LL.stride * l : NULL;
+        float* LGW = lora ? t->LG + t->LL.stride * l : NULL;
+        layer_act_t* a = &t->act[l];
+
+        /* FFN */
+        if (!lora) GEMM(t->g_hidden, a->ffn_h, GW + t->L.down, h, f, T, 1, 0, 1);
+        GEMM(t->g_hidden, W + t->L.down, t->g_ffn, T, f, h, 0, 0, 0);
+        OP("swiglu_backward", 0.0, 20.0 * (double)(T * f), seraph_swiglu_backward(a->gate, a->up, t->g_ffn, t->g_gate, t->g_up, (size_t)(T * f), s));
+        if (!lora) {
+            GEMM(t->g_gate, a->xn_ffn, GW + t->L.gate, f, h, T, 1, 0, 1);
+            GEMM(t->g_up, a->xn_ffn, GW + t->L.up, f, h, T, 1, 0, 1);
+        }
+        GEMM(t->g_gate, W + t->L.gate, t->g_xn, T, h, f, 0, 0, 0);
+        GEMM(t->g_up, W + t->L.up, t->g_xn, T, h, f, 0, 0, 1);
+        OP("rmsnorm_backward", 0.0, 12.0 * (double)(T * h), seraph_rmsnorm_backward(a->post_in, W + t->L.post_norm, t->g_xn, t->g_tmp,
+                                   lora ? t->scratch_gs : GW + t->L.post_norm, T, h, eps, t->ws, t->ws_bytes, s));
+        OP("add", 0.0, 12.0 * (double)(T * h), seraph_add(t->g_tmp, t->g_hidden, t->g_hidden, (size_t)(T * h), s));
+
+        /* attention */
+        if (!lora) GEMM(t->g_hidden, a->attn_out, GW + t->L.o, h, qd, T, 1, 0, 1);
+        GEMM(t->g_hidden, W + t->L.o, t->g_attn, T, qd, h, 0, 0, 0);
+        if (lora && t->LL.A[3] >= 0 &&
+            lora_backward(t, t->g_hidden, a->attn_out, LW + t->LL.A[3], LW + t->LL.B[3], LGW + t->LL.A[3], LGW + t->LL.B[3], T, qd, h)) return -1.0f;
+        OP("fill", 0.0, 4.0 * (double)(T * kv), seraph_fill_u32(t->g_k, 0, (size_t)(T * kv), s));                               /* src/train.c:5221-5222 */
+        OP("fill", 0.0, 4.0 * (double)(T * kv), seraph_fill_u32(t->g_v, 0, (size_t)(T * kv), s));
+        OP("attention_backward", 10.0 * D * t->attn_pairs * H, 0.0, seraph_attention_backward(a->q, a->k, a->v, t->g_attn, a->attn_out, a->lse, t->g_q, t->g_k, t->g_v,
+                                     starts, batch, T, H, KVH, D, scale, t->ws, t->ws_bytes, s));
+        OP("rope", 0.0, 8.0 * (double)(T * qd), seraph_rope(t->g_q, t->g_q, starts, batch, T, H, D, theta, 1, s));
+        OP("rope", 0.0, 8.0 * (double)(T * kv), seraph_rope(t->g_k, t->g_k, starts, batch, T, KVH, D, theta, 1, s));
+        if (!lora) {
+            GEMM(t->g_q, a->xn_attn, GW + t->L.q, qd, h, T, 1, 0, 1);
+            GEMM(t->g_k, a->xn_attn, GW + t->L.k, kv, h, T, 1, 0, 1);
+            GEMM(t->g_v, a->xn_attn, GW + t->L.v, kv, h, T, 1, 0, 1);
+        } else {
+            float* gs[3] = {t->g_q, t->g_k, t->g_v};
+            int64_t outs[3] = {qd, kv, kv};
+            for (int p = 0; p < 3; p++)
+                if (t->LL.A[p] >= 0 &&
+                    lora_backward(t, gs[p], a->xn_attn, LW + t->LL.A[p], LW + t->LL.B[p], LGW + t->LL.A[p], LGW + t->LL.B[p], T, h, outs[p])) return -1.0f;
+        }
+        GEMM(t->g_q, W + t->L.q, t->g_xn, T, h, qd, 0, 0, 0);
+        GEMM(t->g_k, W + t->L.k, t->g_xn, T, h, kv, 0, 0, 1);
+        GEMM(t->g_v, W + t->L.v, t->g_xn, T, h, kv, 0, 0, 1);
+        OP("rmsnorm_backward", 0.0, 12.0 * (double)(T * h), seraph_rmsnorm_backward(a->layer_in, W + t->L.in_norm, t->g_xn, t->g_tmp,
+                                   lora ? t->scratch_gs : GW + t->L.in_norm, T, h, eps, t->ws, t->ws_bytes, s));
+        OP("add", 0.0, 12.0 * (double)(T * h), seraph_add(t->g_tmp, t->g_hidden, t->g_hidden, (size_t)(T * h), s));
+    }
+    if (!lora) OP("embedding_backward", 0.0, 12.0 * (double)(T * h), seraph_embedding_backward(t->d_tokens, t->g_hidden, t->G + t->off_embed, T, h, V, t->ws, t->ws_bytes, s));
+    CK(seraph_hip_event_record(t->ev[2], s));
+
+    /* ---------------- optimizer (src/train.c:5439-5463, LoRA :6617-6640) */
+    t->accumulation_counter++;
+    int accum = t->opt.gradient_accumulation_steps < 1 ? 1 : t->opt.gradient_accumulation_steps;
+    if (t->accumulation_counter >= accum) {
+        if (run_optimizer) {
+            t->optimizer_step++;
+            float lr = t->opt.learning_rate;
+            float warm = (float)t->opt.warmup_steps;
+            if ((float)t->optimizer_step < warm) lr = t->opt.learning_rate * ((float)t->optimizer_step / warm);
+            lr = lr / (float)accum;
+            t->last_lr = lr;
+            if (lora) OP("adamw", 0.0, 28.0 * (double)t->nlora, seraph_adamw(t->LP, t->LG, t->LM, t->LV, (size_t)t->nlora, lr, t->opt.beta1, t->opt.beta2,
+                                      t->opt.weight_decay, t->opt.eps, t->optimizer_step, t->opt.clip, s));
+            else OP("adamw", 0.0, 28.0 * (double)t->nparams, seraph_adamw(t->P, t->G, t->M, t->V, (size_t)t->nparams, lr, t->opt.beta1, t->opt.beta2,
+                                 t->opt.weight_decay, t->opt.eps, t->optimizer_step, t->opt.clip, s));
+        }
+        t->accumulation_counter = 0;
+    }
+    CK(seraph_hip_event_record(t->ev[3], s));
+
+    float loss_sum = 0.0f;
+    CK(seraph_hip_d2h(&loss_sum, red_in, sizeof(float), s));               /* waits for the whole step */
+    for (int i = 0; i < 3; i++) seraph_hip_event_elapsed_ms(t->ev[i], t->ev[i + 1], &t->phase_ms[i]);
+    op_fold(t);
+    return loss_sum / (float)num_valid;
+}
+
+float hip_train_step_full_batch(hip_trainer_t* t, const int* tokens_packed, int total_tokens,
+                                const int* seq_starts, int batch_size, int run_optimizer) {
+    if (!t || t->lora) { fprintf(stderr, "ERROR: trainer is not in full-weight mode\n"); return -1.0f; }
+    return run_step(t, tokens_packed, total_tokens, seq_starts, batch_size, run_optimizer);
+}
+
+float hip_train_step_lora_batch(hip_trainer_t* t, const int* tokens_packed, int total_tokens,
+                                const int* seq_starts, int batch_size, int run_optimizer) {
+    if (!t || !t->lora) { fprintf(stderr, "ERROR: trainer is not in LoRA mode\n"); return -1.0f; }
+    return run_step(t, tokens_packed, total_tokens, seq_starts, batch_size, run_optimizer);
+}

@@ -1,0 +1,151 @@
+"""The vulkan_* compatible backend (the API src/train.c links against) driven the way the
+reference's step drives it: context, buffers, a recorded batch of ops, one submit, a
+download - every result checked against the CPU oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+class Buf(C.Structure):
+    _fields_ = [("buffer", C.c_void_p), ("memory", C.c_void_p), ("size", C.c_size_t), ("mapped", C.c_void_p)]
+
+
+@pytest.fixture(scope="module")
+def vk():
+    from seraph_amd._lib import backend
+    lib = backend()
+    lib.vulkan_init_ex.restype = C.c_void_p
+    lib.vulkan_buffer_create.restype = C.POINTER(Buf)
+    lib.vulkan_buffer_create.argtypes = [C.c_void_p, C.c_size_t]
+    ctx = lib.vulkan_init_ex(0, -1)
+    assert ctx
+    yield lib, C.c_void_p(ctx)
+    lib.vulkan_free(C.c_void_p(ctx))
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def up(vk, a):
+    lib, ctx = vk
+    a = np.ascontiguousarray(a)
+    b = lib.vulkan_buffer_create(ctx, a.nbytes)
+    assert b and b.contents.size == a.nbytes and not b.contents.mapped
+    lib.vulkan_buffer_upload_bytes(ctx, b, a.ctypes.data_as(C.c_void_p), C.c_size_t(a.nbytes))
+    return b
+
+
+def down(vk, b, shape, dtype=np.float32):
+    lib, ctx = vk
+    out = np.empty(shape, dtype)
+    lib.vulkan_buffer_download_bytes(ctx, b, out.ctypes.data_as(C.c_void_p), C.c_size_t(out.nbytes))
+    return out
+
+
+def close(got, ref, rtol=1e-4, atol=1e-5):
+    got, ref = got.astype(np.float64), np.asarray(ref, np.float64)
+    assert (np.abs(got - ref) <= atol + rtol * np.abs(ref)).all(), np.abs(got - ref).max()
+
+
+def test_buffers_and_fill_range(vk):
+    lib, ctx = vk
+    x = rng(0).standard_normal(1024).astype(np.float32)            # tests/test_vulkan.c: 4 KB round trip
+    b = up(vk, x)
+    assert (down(vk, b, 1024) == x).all()
+    lib.vulkan_fill_buffer_range(ctx, b, C.c_size_t(18), C.c_uint32(0), C.c_size_t(23))   # aligned down: bytes 16..35
+    y = down(vk, b, 1024)
+    assert (y[4:9] == 0).all() and (y[:4] == x[:4]).all() and (y[9:] == x[9:]).all()
+    lib.vulkan_fill_buffer(ctx, b, C.c_uint32(0x3f800000), C.c_size_t(1 << 20))          # clamped to the buffer
+    assert (down(vk, b, 1024) == 1.0).all()
+    lib.vulkan_buffer_free(ctx, b)
+    lib.vulkan_silu(ctx, None, None, C.c_size_t(5))                 # NULL buffers are ignored, not fatal
+    assert lib.hip_backend_error_count(ctx) == 0
+
+
+def test_recorded_backward_slice(vk, orc):
+    """One attention block's backward ops in the reference's order (src/train.c:5205-5351),
+    recorded between cmd_begin and cmd_end_submit."""
+    lib, ctx = vk
+    r = rng(1)
+    T, H, KVH, D, h = 96, 4, 2, 32, 64
+    qd, kv = H * D, KVH * D
+    q, k, v = (r.standard_normal((T, w)).astype(np.float32) * 0.4 for w in (qd, kv, kv))
+    g_hidden = (1e-2 * r.standard_normal((T, h))).astype(np.float32)
+    w_o = (0.05 * r.standard_normal((h, qd))).astype(np.float32)
+    w_q = (0.05 * r.standard_normal((qd, h))).astype(np.float32)
+    xn = r.standard_normal((T, h)).astype(np.float32)
+    layer_in = r.standard_normal((T, h)).astype(np.float32)
+    w_norm = (1 + 0.02 * r.standard_normal(h)).astype(np.float32)
+    g_wq0 = (1e-3 * r.standard_normal((qd, h))).astype(np.float32)
+
+    B = {n: up(vk, a) for n, a in dict(q=q, k=k, v=v, g_hidden=g_hidden, w_o=w_o, w_q=w_q, xn=xn, layer_in=layer_in,
+                                       w_norm=w_norm, g_wq=g_wq0).items()}
+    for n, shape in dict(g_attn=(T, qd), g_q=(T, qd), g_k=(T, kv), g_v=(T, kv), g_xn=(T, h), g_tmp=(T, h), g_norm=(h,)).items():
+        B[n] = up(vk, np.full(shape, 7.0, np.float32))              # stale contents the ops must overwrite or be told to zero
+
+    assert lib.vulkan_cmd_begin(ctx) == 1
+    lib.vulkan_matmul(ctx, B["g_hidden"], B["w_o"], B["g_attn"], T, qd, h)
+    lib.vulkan_fill_buffer(ctx, B["g_k"], C.c_uint32(0), C.c_size_t(T * kv * 4))
+    lib.vulkan_fill_buffer(ctx, B["g_v"], C.c_uint32(0), C.c_size_t(T * kv * 4))
+    lib.vulkan_fill_buffer(ctx, B["g_norm"], C.c_uint32(0), C.c_size_t(h * 4))
+    lib.vulkan_batch_attention_backward(ctx, B["q"], B["k"], B["v"], B["g_attn"], B["g_q"], B["g_k"], B["g_v"], T, H, KVH, D)
+    lib.vulkan_rope_backward(ctx, B["g_q"], B["g_q"], T, H, D, C.c_float(10000.0))
+    lib.vulkan_matmul_transpose(ctx, B["g_q"], B["xn"], B["g_wq"], qd, h, T, 1, 0, 1)
+    lib.vulkan_matmul(ctx, B["g_q"], B["w_q"], B["g_xn"], T, h, qd)
+    lib.vulkan_rmsnorm_backward_batch(ctx, B["layer_in"], B["w_norm"], B["g_xn"], B["g_tmp"], B["g_norm"], T, h, C.c_float(1e-5))
+    lib.vulkan_add(ctx, B["g_tmp"], B["g_hidden"], B["g_hidden"], C.c_size_t(T * h))
+    assert lib.vulkan_cmd_end_submit(ctx) == 1
+    assert lib.vulkan_cmd_end_submit(ctx) == 0                      # nothing recording any more
+
+    g_attn = orc.matmul(g_hidden, w_o, T, qd, h)
+    dq, dk, dv = orc.attention_backward(q, k, v, g_attn, H, KVH, D)
+    dq = orc.rope(dq, H, D, 10000.0, backward=True)
+    close(down(vk, B["g_k"], (T, kv)), dk); close(down(vk, B["g_v"], (T, kv)), dv)
+    close(down(vk, B["g_q"], (T, qd)), dq)
+    close(down(vk, B["g_wq"], (qd, h)), orc.matmul(dq, xn, qd, h, T, 1, 0, g_wq0))
+    g_xn = orc.matmul(dq, w_q, T, h, qd)
+    dx, gs = orc.rmsnorm_backward_batch(layer_in, w_norm, g_xn, 1e-5)
+    close(down(vk, B["g_norm"], (h,)), gs)
+    close(down(vk, B["g_hidden"], (T, h)), dx + g_hidden)
+    for b in B.values():
+        lib.vulkan_buffer_free(ctx, b)
+    assert lib.hip_backend_error_count(ctx) == 0
+
+
+def test_loss_chain_and_adamw(vk, orc):
+    """cross_entropy_grad + the 512-wide reduce_sum ping-pong (src/train.c:4887-4913), then
+    AdamW with the host-side bias corrections (src/vulkan_backend.c:2151-2152)."""
+    lib, ctx = vk
+    r = rng(2)
+    T, V = 1200, 1000
+    x = (2 * r.standard_normal((T, V))).astype(np.float32)
+    t = r.integers(0, V, T).astype(np.uint32)
+    bx, bt = up(vk, x), up(vk, t)
+    bg, bl = up(vk, np.zeros((T, V), np.float32)), up(vk, np.zeros(T, np.float32))
+    ra, rb = up(vk, np.zeros(T, np.float32)), up(vk, np.zeros(T, np.float32))
+    lib.vulkan_cmd_begin(ctx)
+    lib.vulkan_cross_entropy_grad(ctx, bx, bt, bg, bl, T - 1, V, T - 1)
+    n, rin, rout = T - 1, bl, ra
+    while n > 1:
+        lib.vulkan_reduce_sum(ctx, rin, rout, C.c_size_t(n))
+        n = (n + 511) // 512
+        rin, rout = rout, (rb if rout is ra else ra)
+    lib.vulkan_cmd_end_submit(ctx)
+    rg, rl = orc.cross_entropy_grad(x[:T - 1], t[:T - 1], valid_rows=T - 1)
+    close(down(vk, bg, (T, V))[:T - 1], rg, atol=1e-7)
+    close(down(vk, rin, (1,)), [rl.astype(np.float64).sum()], rtol=1e-5, atol=1e-3)
+
+    n = 5000
+    w = r.standard_normal(n).astype(np.float32)
+    g = (1e-3 * r.standard_normal(n)).astype(np.float32)
+    z = np.zeros(n, np.float32)
+    bw, bgr, bm, bv = up(vk, w), up(vk, g), up(vk, z), up(vk, z)
+    f = C.c_float
+    lib.vulkan_adamw_update(ctx, bw, bgr, bm, bv, f(3.14e-4), f(0.9), f(0.999), f(0.01), f(1e-8), 3, C.c_size_t(n))
+    rw, rm, rv = orc.adamw(w, g, z, z, 3.14e-4, 0.9, 0.999, 0.01, 1e-8, 3)
+    close(down(vk, bw, n), rw, atol=1e-7); close(down(vk, bm, n), rm, atol=1e-9); close(down(vk, bv, n), rv, atol=1e-12)
+    assert lib.hip_backend_error_count(ctx) == 0
