@@ -27,6 +27,7 @@
 // search over the batch+1 offsets); a score (i, j) is kept when start[i] <= j <= i.  Tiles are anchored on the global token
 // axis at multiples of 32/128, so ragged sequence lengths need no padding.
 #include <limits.h>
+#include <mutex>
 
 #include "common.hpp"
 
@@ -43,15 +44,93 @@ __device__ __forceinline__ v16f mfma(float a, float b, v16f c) { return __builti
 // row index inside a 32x32 accumulator block held by register v of a lane in half-wave h
 __device__ __forceinline__ int acc_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3); }
 
-// ---------------------------------------------------------------- sequence bounds of a token
-__device__ __forceinline__ int seq_start_of(const uint32_t* __restrict__ ss, int batch, int64_t t) {
-    return ss ? (int)ss[find_seq(ss, batch, t)] : 0;
+// The products that contract over the accumulator's row index take their other operand from a
+// tile row in LDS, one value per (lane, 32-wide block of head_dim).  Lane r of block db is given
+// feature d = DB*r + db (DB = head_dim/32) instead of db*32 + r, so the DB values a lane needs sit
+// next to each other and arrive with one 4/8/16-byte LDS read that feeds DB MFMAs; results are
+// written back with the same mapping, which also makes the final global accesses DB floats wide.
+template <int DB> struct DVec { float v[DB]; };
+template <int DB>
+__device__ __forceinline__ DVec<DB> lds_dvec(const float* row, int r) {
+    DVec<DB> o;
+    if (DB == 4) { const float4 t = *reinterpret_cast<const float4*>(row + 4 * r); o.v[0] = t.x; o.v[1] = t.y; o.v[2 % DB] = t.z; o.v[3 % DB] = t.w; }
+    else if (DB == 2) { const float2 t = *reinterpret_cast<const float2*>(row + 2 * r); o.v[0] = t.x; o.v[1 % DB] = t.y; }
+    else { o.v[0] = row[r]; }
+    return o;
 }
-__device__ __forceinline__ int seq_end_of(const uint32_t* __restrict__ ss, int batch, int64_t t, int64_t T) {
-    if (!ss) return (int)T;
-    const int64_t e = (int64_t)ss[find_seq(ss, batch, t) + 1];
-    return (int)(e < T ? e : T);
+
+// ---------------------------------------------------------------- packed-sequence offsets
+// Every workgroup copies the batch+1 prefix offsets into LDS once (up to kMaxSeqLds of
+// them; larger batches are searched in global memory) and binary-searches them there:
+// a lookup costs a few LDS round trips instead of a chain of dependent global loads.
+constexpr int kMaxSeqLds = 1024;
+
+struct SeqTable {
+    const uint32_t* g;     // global offsets (NULL = one sequence of T tokens)
+    const uint32_t* s;     // LDS copy or NULL
+    int batch;
+    int T;
+    __device__ __forceinline__ int find(int t) const {
+        const uint32_t* p = s ? s : g;
+        int lo = 0, hi = batch;
+        while (lo < hi) {
+            int mid = (lo + hi) >> 1;
+            if ((int)p[mid + 1] <= t) lo = mid + 1; else hi = mid;
+        }
+        return lo;
+    }
+    __device__ __forceinline__ int start_of(int t) const { return g ? (int)(s ? s : g)[find(t)] : 0; }
+    __device__ __forceinline__ int end_of(int t) const {
+        if (!g) return T;
+        int e = (int)(s ? s : g)[find(t) + 1];
+        return e < T ? e : T;
+    }
+};
+
+// Call from all lanes of the workgroup, before any lookup; contains a barrier.
+__device__ __forceinline__ SeqTable load_seq_table(const uint32_t* __restrict__ seq_starts, int batch, int T,
+                                                   uint32_t* __restrict__ lds) {
+    SeqTable st;
+    st.g = seq_starts; st.s = nullptr; st.batch = batch; st.T = T;
+    if (seq_starts && batch + 1 <= kMaxSeqLds) {
+        for (int i = threadIdx.x; i <= batch; i += kAttnThreads) lds[i] = seq_starts[i];
+        st.s = lds;
+    }
+    __syncthreads();
+    return st;
 }
+
+// ---------------------------------------------------------------- dynamic tile queue
+// Causal attention tiles differ in cost by up to two orders of magnitude, and the hardware
+// deals workgroups to CUs in a fixed rotation, so a one-tile-per-workgroup launch leaves half of
+// the machine idle behind the CUs that drew the long tiles.  The kernels are therefore
+// persistent: a resident set of workgroups pulls tile indices, longest first, from a device
+// counter until it runs dry.  Every workgroup makes exactly one failing pull and then leaves, so
+// the grid always drains; the last one out rewinds the counter pair for the next launch.
+// Counters come from a fixed pool in device memory (zero at module load), one pair per launch in
+// rotation, so launches on different streams do not share a pair.
+constexpr int kQueueSlots = 1024;
+static __device__ unsigned int g_tile_queues[2 * kQueueSlots];
+
+struct TileQueue {
+    unsigned int* q;        // q[0] next item, q[1] workgroups finished
+    int* slot;              // one int of LDS
+    int total;
+    __device__ __forceinline__ int next() const {
+        if (threadIdx.x == 0) *slot = (int)atomicAdd(&q[0], 1u);
+        __syncthreads();
+        const int item = *slot;
+        __syncthreads();
+        return item < total ? item : -1;
+    }
+    __device__ __forceinline__ void leave() const {
+        if (threadIdx.x == 0 && atomicAdd(&q[1], 1u) == gridDim.x - 1) {
+            q[0] = 0u;
+            q[1] = 0u;
+            __threadfence();
+        }
+    }
+};
 
 // ---------------------------------------------------------------- tile staging (32 rows x D)
 template <int D>
@@ -81,20 +160,27 @@ struct Tile32 {
 // ---------------------------------------------------------------- forward
 // grid (query tiles of 128, heads); wave w owns queries i0+32w .. +31; key/value tiles of 32.
 template <int D>
-__global__ __launch_bounds__(kAttnThreads) void attn_fwd_kernel(const float* __restrict__ Q, const float* __restrict__ K,
+__global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_fwd_kernel(const float* __restrict__ Q, const float* __restrict__ K,
                                                                 const float* __restrict__ V, float* __restrict__ O,
                                                                 float* __restrict__ LSE, const uint32_t* __restrict__ seq_starts, int batch,
-                                                                int64_t T, int H, int KVH, float scale_log2e) {
+                                                                int64_t T, int H, int KVH, float scale_log2e,
+                                                                unsigned int* __restrict__ queue) {
     constexpr int LD = D + 4, DB = D / 32;
     __shared__ __attribute__((aligned(16))) float sK[2][32 * LD];
     __shared__ __attribute__((aligned(16))) float sV[2][32 * LD];
-    const int head = blockIdx.y, kvh = head / (H / KVH);
-    const int qt = gridDim.x - 1 - blockIdx.x;                 // long rows first
-    const int64_t i0 = (int64_t)qt * 128;
+    __shared__ uint32_t sSeq[kMaxSeqLds];
+    __shared__ int sItem;
+    const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
+    const int nqt = (int)((T + 127) / 128);
+    const TileQueue tq_{queue, &sItem, nqt * H};
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
+    for (int item = tq_.next(); item >= 0; item = tq_.next()) {
+    const int head = item % H, kvh = head / (H / KVH);
+    const int qt = nqt - 1 - item / H;                         // long rows first
+    const int64_t i0 = (int64_t)qt * 128;
     const int64_t iw0 = i0 + 32 * w, i_lane = iw0 + r;
     const bool row_ok = i_lane < T;
-    const int ss_lane = row_ok ? seq_start_of(seq_starts, batch, i_lane) : INT_MAX;
+    const int ss_lane = row_ok ? seqs.start_of((int)i_lane) : INT_MAX;
     const int64_t qw = (int64_t)H * D, kw = (int64_t)KVH * D;
 
     float4 qf[D / 8];
@@ -103,7 +189,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_fwd_kernel(const float* __r
         qf[s8] = row_ok ? *reinterpret_cast<const float4*>(Q + i_lane * qw + head * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
 
     const int64_t i_last = (i0 + 127 < T - 1) ? i0 + 127 : T - 1;
-    const int64_t jbeg = (seq_start_of(seq_starts, batch, i0) / 32) * 32;
+    const int64_t jbeg = (seqs.start_of((int)i0) / 32) * 32;
     const int ntiles = (int)((i_last + 1 - jbeg + 31) / 32);
 
     float m = -INFINITY, l = 0.0f;
@@ -131,39 +217,57 @@ __global__ __launch_bounds__(kAttnThreads) void attn_fwd_kernel(const float* __r
             v16f s;
 #pragma unroll
             for (int v = 0; v < 16; v++) s[v] = 0.0f;
+            // LDS operands are fetched one step ahead of the MFMAs that consume them
+            float4 kb[2];
+            kb[0] = *reinterpret_cast<const float4*>(&sK[cur][r * LD + 4 * h]);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
 #pragma unroll
             for (int s8 = 0; s8 < D / 8; s8++) {
-                const float4 a = *reinterpret_cast<const float4*>(&sK[cur][r * LD + s8 * 8 + 4 * h]);
+                if (s8 + 1 < D / 8) kb[(s8 + 1) & 1] = *reinterpret_cast<const float4*>(&sK[cur][r * LD + (s8 + 1) * 8 + 4 * h]);
+                const float4 a = kb[s8 & 1];
                 s = mfma(a.x, qf[s8].x, s); s = mfma(a.y, qf[s8].y, s);
                 s = mfma(a.z, qf[s8].z, s); s = mfma(a.w, qf[s8].w, s);
+                if (s8 + 1 < D / 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
             }
             float mloc = -INFINITY;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int64_t j = j0 + acc_row(v, h);
-                const bool valid = (j >= ss_lane) && (j <= i_lane);
+                const int j = (int)j0 + acc_row(v, h);
+                const bool valid = (j >= ss_lane) && (j <= (int)i_lane);
                 s[v] = valid ? s[v] * scale_log2e : -INFINITY;
                 mloc = fmaxf(mloc, s[v]);
             }
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+            // Lazy rescaling: the running maximum is only advanced (and O, l rescaled) when some
+            // query of the wave has outgrown it by more than 2^8; until then probabilities are formed
+            // against the slightly stale maximum, which is exact after the final division by l.
             const float mnew = fmaxf(m, mloc);
-            const float msafe = mnew == -INFINITY ? 0.0f : mnew;
-            const float alpha = fast_exp2(m - msafe);
+            if (__any(mnew > m + 8.0f)) {
+                const float alpha = fast_exp2(m - (mnew == -INFINITY ? 0.0f : mnew));
+                l *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; db++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) o[db][v] *= alpha;
+                m = mnew;
+            }
+            const float msafe = m == -INFINITY ? 0.0f : m;
             float lsum = 0.0f;
 #pragma unroll
             for (int v = 0; v < 16; v++) { s[v] = fast_exp2(s[v] - msafe); lsum += s[v]; }
             lsum += __shfl_xor(lsum, 32, 64);
-            l = l * alpha + lsum;
-            m = mnew;
-#pragma unroll
-            for (int db = 0; db < DB; db++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) o[db][v] *= alpha;
+            l += lsum;
+            DVec<DB> vb[2];
+            vb[0] = lds_dvec<DB>(&sV[cur][acc_row(0, h) * LD], r);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int jl = acc_row(v, h);
+                if (v + 1 < 16) vb[(v + 1) & 1] = lds_dvec<DB>(&sV[cur][acc_row(v + 1, h) * LD], r);
 #pragma unroll
-                for (int db = 0; db < DB; db++) o[db] = mfma(sV[cur][jl * LD + db * 32 + r], s[v], o[db]);
+                for (int db = 0; db < DB; db++) o[db] = mfma(vb[v & 1].v[db], s[v], o[db]);
+                if (v + 1 < 16) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, DB, 0);
             }
         }
         if (t + 1 < ntiles) {
@@ -175,15 +279,22 @@ __global__ __launch_bounds__(kAttnThreads) void attn_fwd_kernel(const float* __r
 
     if (row_ok) {
         const float inv = 1.0f / l;
+        // accumulator row a of block db is feature DB*a + db: registers 4g..4g+3 of all blocks are
+        // 4*DB consecutive features starting at DB*(8g + 4h)
 #pragma unroll
-        for (int db = 0; db < DB; db++)
+        for (int g = 0; g < 4; g++) {
+            float* dst = O + i_lane * qw + head * D + DB * (8 * g + 4 * h);
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                float4 out = make_float4(o[db][4 * g] * inv, o[db][4 * g + 1] * inv, o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
-                *reinterpret_cast<float4*>(O + i_lane * qw + head * D + db * 32 + 8 * g + 4 * h) = out;
+            for (int e = 0; e < 4; e++) {
+                if (DB == 4) *reinterpret_cast<float4*>(dst + 4 * e) = make_float4(o[0][4 * g + e] * inv, o[1 % DB][4 * g + e] * inv, o[2 % DB][4 * g + e] * inv, o[3 % DB][4 * g + e] * inv);
+                else if (DB == 2) *reinterpret_cast<float2*>(dst + 2 * e) = make_float2(o[0][4 * g + e] * inv, o[1 % DB][4 * g + e] * inv);
+                else dst[e] = o[0][4 * g + e] * inv;
             }
+        }
         if (LSE && h == 0) LSE[i_lane * H + head] = (m + __log2f(l)) * kLn2;
     }
+    }   // tile queue
+    tq_.leave();
 }
 
 // ---------------------------------------------------------------- delta = rowsum(dO * O)
@@ -209,30 +320,51 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const float* __restrict
 // ---------------------------------------------------------------- backward: dK, dV
 // grid (key tiles of 128, kv heads); wave w owns keys j0+32w .. +31 for every query head of the group.
 template <int D>
-__global__ __launch_bounds__(kAttnThreads) void attn_bwd_dkv_kernel(const float* __restrict__ Q, const float* __restrict__ K,
+__global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_kernel(const float* __restrict__ Q, const float* __restrict__ K,
                                                                     const float* __restrict__ V, const float* __restrict__ dO,
                                                                     const float* __restrict__ LSE, const float* __restrict__ DELTA,
                                                                     float* __restrict__ dK, float* __restrict__ dV,
                                                                     const uint32_t* __restrict__ seq_starts, int batch,
-                                                                    int64_t T, int H, int KVH, float scale, float scale_log2e) {
+                                                                    int64_t T, int H, int KVH, float scale, float scale_log2e,
+                                                                    unsigned int* __restrict__ queue) {
     constexpr int LD = D + 4, DB = D / 32;
     __shared__ __attribute__((aligned(16))) float sQ[2][32 * LD];
     __shared__ __attribute__((aligned(16))) float sG[2][32 * LD];     // dO
     __shared__ __attribute__((aligned(16))) float sLse[2][32];
     __shared__ __attribute__((aligned(16))) float sDel[2][32];
     __shared__ __attribute__((aligned(16))) int sSS[2][32];
-    const int kvh = blockIdx.y, G = H / KVH;
-    const int64_t j0 = (int64_t)blockIdx.x * 128;
+    __shared__ uint32_t sSeq[kMaxSeqLds];
+    __shared__ int sItem;
+    const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
+    const int G = H / KVH;
+    const TileQueue tq_{queue, &sItem, (int)((T + 127) / 128) * KVH};
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
+    for (int item = tq_.next(); item >= 0; item = tq_.next()) {
+    const int kvh = item % KVH;
+    const int64_t j0 = (int64_t)(item / KVH) * 128;            // early keys of a sequence are the long ones
     const int64_t jw0 = j0 + 32 * w, j_lane = jw0 + r;
     const bool col_ok = j_lane < T;
     const int64_t qw = (int64_t)H * D, kw = (int64_t)KVH * D;
 
-    float4 kf[D / 8], vf[D / 8];
+    // This wave's 32 keys as B operands (lane = key, k = d).  K always lives in registers; V
+    // does too for head_dim <= 64, but at 128 the two fragments plus the dK/dV accumulators
+    // exceed the register file, so V for the workgroup's 128 keys is parked in LDS instead.
+    constexpr bool kVinLds = D > 64;
+    __shared__ __attribute__((aligned(16))) float sVt[kVinLds ? 128 * LD : 4];
+    float4 kf[D / 8], vf[kVinLds ? 1 : D / 8];
 #pragma unroll
     for (int s8 = 0; s8 < D / 8; s8++) {
         kf[s8] = col_ok ? *reinterpret_cast<const float4*>(K + j_lane * kw + kvh * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
-        vf[s8] = col_ok ? *reinterpret_cast<const float4*>(V + j_lane * kw + kvh * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (!kVinLds)
+            vf[s8] = col_ok ? *reinterpret_cast<const float4*>(V + j_lane * kw + kvh * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if (kVinLds) {
+        Tile32<D> tvv;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            tvv.gload(V, j0 + 32 * q, T, kw, kvh * D);
+            tvv.sstore(sVt + q * 32 * LD);
+        }
     }
     v16f dk[DB], dv[DB];
 #pragma unroll
@@ -241,7 +373,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_bwd_dkv_kernel(const float*
         for (int v = 0; v < 16; v++) { dk[db][v] = 0.0f; dv[db][v] = 0.0f; }
 
     const int64_t j_last = (j0 + 127 < T - 1) ? j0 + 127 : T - 1;
-    const int64_t i_end = seq_end_of(seq_starts, batch, j_last, T);                         // queries of the last key's sequence
+    const int64_t i_end = seqs.end_of((int)j_last);                         // queries of the last key's sequence
     const int nq = (int)((i_end - j0 + 31) / 32);
     const int iters = nq * G;
 
@@ -254,7 +386,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_bwd_dkv_kernel(const float*
         if (threadIdx.x < 32) {
             st_lse = i < T ? LSE[i * H + head] * kLog2e : 0.f;
             st_del = i < T ? DELTA[i * H + head] : 0.f;
-            st_ss = i < T ? seq_start_of(seq_starts, batch, i) : INT_MAX;
+            st_ss = i < T ? seqs.start_of((int)i) : INT_MAX;
         }
     };
     auto stats_store = [&](int buf) {
@@ -283,10 +415,11 @@ __global__ __launch_bounds__(kAttnThreads) void attn_bwd_dkv_kernel(const float*
             for (int s8 = 0; s8 < D / 8; s8++) {
                 const float4 a = *reinterpret_cast<const float4*>(&sQ[cur][r * LD + s8 * 8 + 4 * h]);
                 const float4 b = *reinterpret_cast<const float4*>(&sG[cur][r * LD + s8 * 8 + 4 * h]);
-                s = mfma(a.x, kf[s8].x, s); dp = mfma(b.x, vf[s8].x, dp);
-                s = mfma(a.y, kf[s8].y, s); dp = mfma(b.y, vf[s8].y, dp);
-                s = mfma(a.z, kf[s8].z, s); dp = mfma(b.z, vf[s8].z, dp);
-                s = mfma(a.w, kf[s8].w, s); dp = mfma(b.w, vf[s8].w, dp);
+                const float4 vv = kVinLds ? *reinterpret_cast<const float4*>(&sVt[(32 * w + r) * LD + s8 * 8 + 4 * h]) : vf[kVinLds ? 0 : s8];
+                s = mfma(a.x, kf[s8].x, s); dp = mfma(b.x, vv.x, dp);
+                s = mfma(a.y, kf[s8].y, s); dp = mfma(b.y, vv.y, dp);
+                s = mfma(a.z, kf[s8].z, s); dp = mfma(b.z, vv.z, dp);
+                s = mfma(a.w, kf[s8].w, s); dp = mfma(b.w, vv.w, dp);
             }
 #pragma unroll
             for (int g = 0; g < 4; g++) {
@@ -297,8 +430,8 @@ __global__ __launch_bounds__(kAttnThreads) void attn_bwd_dkv_kernel(const float*
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const int v = 4 * g + e;
-                    const int64_t i = i0 + 8 * g + 4 * h + e;
-                    const bool valid = (j_lane <= i) && (j_lane >= ss_p[e]);       // ss = INT_MAX for i >= T
+                    const int i = (int)i0 + 8 * g + 4 * h + e;
+                    const bool valid = ((int)j_lane <= i) && ((int)j_lane >= ss_p[e]);     // ss = INT_MAX for i >= T
                     const float p = valid ? fast_exp2(s[v] * scale_log2e - lse_p[e]) : 0.0f;
                     s[v] = p;
                     dp[v] = p * (dp[v] - del_p[e]);
@@ -307,10 +440,12 @@ __global__ __launch_bounds__(kAttnThreads) void attn_bwd_dkv_kernel(const float*
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int il = acc_row(v, h);
+                const DVec<DB> go = lds_dvec<DB>(&sG[cur][il * LD], r);
+                const DVec<DB> qq = lds_dvec<DB>(&sQ[cur][il * LD], r);
 #pragma unroll
                 for (int db = 0; db < DB; db++) {
-                    dv[db] = mfma(s[v], sG[cur][il * LD + db * 32 + r], dv[db]);
-                    dk[db] = mfma(dp[v], sQ[cur][il * LD + db * 32 + r], dk[db]);
+                    dv[db] = mfma(s[v], go.v[db], dv[db]);
+                    dk[db] = mfma(dp[v], qq.v[db], dk[db]);
                 }
             }
         }
@@ -319,36 +454,56 @@ __global__ __launch_bounds__(kAttnThreads) void attn_bwd_dkv_kernel(const float*
     }
 
 #pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int64_t j = jw0 + acc_row(v, h);
-            if (j < T) {
-                const int64_t off = j * kw + kvh * D + db * 32 + r;
-                dK[off] += dk[db][v] * scale;
-                dV[off] += dv[db][v];
+    for (int v = 0; v < 16; v++) {
+        const int64_t j = jw0 + acc_row(v, h);
+        if (j < T) {
+            float* pk = dK + j * kw + kvh * D + DB * r;        // lane r owns features DB*r .. DB*r+DB-1
+            float* pv = dV + j * kw + kvh * D + DB * r;
+            if (DB == 4) {
+                float4 a = *reinterpret_cast<float4*>(pk), b = *reinterpret_cast<float4*>(pv);
+                a.x += dk[0][v] * scale; a.y += dk[1 % DB][v] * scale; a.z += dk[2 % DB][v] * scale; a.w += dk[3 % DB][v] * scale;
+                b.x += dv[0][v]; b.y += dv[1 % DB][v]; b.z += dv[2 % DB][v]; b.w += dv[3 % DB][v];
+                *reinterpret_cast<float4*>(pk) = a; *reinterpret_cast<float4*>(pv) = b;
+            } else if (DB == 2) {
+                float2 a = *reinterpret_cast<float2*>(pk), b = *reinterpret_cast<float2*>(pv);
+                a.x += dk[0][v] * scale; a.y += dk[1 % DB][v] * scale;
+                b.x += dv[0][v]; b.y += dv[1 % DB][v];
+                *reinterpret_cast<float2*>(pk) = a; *reinterpret_cast<float2*>(pv) = b;
+            } else {
+                pk[0] += dk[0][v] * scale;
+                pv[0] += dv[0][v];
             }
         }
+    }
+    }   // tile queue
+    tq_.leave();
 }
 
 // ---------------------------------------------------------------- backward: dQ
 // grid (query tiles of 128, heads); wave w owns queries i0+32w .. +31; key/value tiles of 32.
 template <int D>
-__global__ __launch_bounds__(kAttnThreads) void attn_bwd_dq_kernel(const float* __restrict__ Q, const float* __restrict__ K,
+__global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dq_kernel(const float* __restrict__ Q, const float* __restrict__ K,
                                                                    const float* __restrict__ V, const float* __restrict__ dO,
                                                                    const float* __restrict__ LSE, const float* __restrict__ DELTA,
                                                                    float* __restrict__ dQ, const uint32_t* __restrict__ seq_starts, int batch,
-                                                                   int64_t T, int H, int KVH, float scale, float scale_log2e) {
+                                                                   int64_t T, int H, int KVH, float scale, float scale_log2e,
+                                                                   unsigned int* __restrict__ queue) {
     constexpr int LD = D + 4, DB = D / 32;
     __shared__ __attribute__((aligned(16))) float sK[2][32 * LD];
     __shared__ __attribute__((aligned(16))) float sV[2][32 * LD];
-    const int head = blockIdx.y, kvh = head / (H / KVH);
-    const int qt = gridDim.x - 1 - blockIdx.x;
-    const int64_t i0 = (int64_t)qt * 128;
+    __shared__ uint32_t sSeq[kMaxSeqLds];
+    __shared__ int sItem;
+    const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
+    const int nqt = (int)((T + 127) / 128);
+    const TileQueue tq_{queue, &sItem, nqt * H};
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
+    for (int item = tq_.next(); item >= 0; item = tq_.next()) {
+    const int head = item % H, kvh = head / (H / KVH);
+    const int qt = nqt - 1 - item / H;
+    const int64_t i0 = (int64_t)qt * 128;
     const int64_t iw0 = i0 + 32 * w, i_lane = iw0 + r;
     const bool row_ok = i_lane < T;
-    const int ss_lane = row_ok ? seq_start_of(seq_starts, batch, i_lane) : INT_MAX;
+    const int ss_lane = row_ok ? seqs.start_of((int)i_lane) : INT_MAX;
     const float lse_i = row_ok ? LSE[i_lane * H + head] * kLog2e : 0.0f;
     const float del_i = row_ok ? DELTA[i_lane * H + head] : 0.0f;
     const int64_t qw = (int64_t)H * D, kw = (int64_t)KVH * D;
@@ -366,7 +521,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_bwd_dq_kernel(const float* 
         for (int v = 0; v < 16; v++) dq[db][v] = 0.0f;
 
     const int64_t i_last = (i0 + 127 < T - 1) ? i0 + 127 : T - 1;
-    const int64_t jbeg = (seq_start_of(seq_starts, batch, i0) / 32) * 32;
+    const int64_t jbeg = (seqs.start_of((int)i0) / 32) * 32;
     const int ntiles = (int)((i_last + 1 - jbeg + 31) / 32);
 
     Tile32<D> tk, tv;
@@ -398,16 +553,16 @@ __global__ __launch_bounds__(kAttnThreads) void attn_bwd_dq_kernel(const float* 
             }
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int64_t j = j0 + acc_row(v, h);
-                const bool valid = (j >= ss_lane) && (j <= i_lane);
+                const int j = (int)j0 + acc_row(v, h);
+                const bool valid = (j >= ss_lane) && (j <= (int)i_lane);
                 const float p = valid ? fast_exp2(s[v] * scale_log2e - lse_i) : 0.0f;
                 dp[v] = p * (dp[v] - del_i);
             }
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int jl = acc_row(v, h);
+                const DVec<DB> kk = lds_dvec<DB>(&sK[cur][acc_row(v, h) * LD], r);
 #pragma unroll
-                for (int db = 0; db < DB; db++) dq[db] = mfma(dp[v], sK[cur][jl * LD + db * 32 + r], dq[db]);
+                for (int db = 0; db < DB; db++) dq[db] = mfma(dp[v], kk.v[db], dq[db]);
             }
         }
         if (t + 1 < ntiles) {
@@ -418,12 +573,17 @@ __global__ __launch_bounds__(kAttnThreads) void attn_bwd_dq_kernel(const float* 
     }
 
 #pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int64_t i = iw0 + acc_row(v, h);
-            if (i < T) dQ[i * qw + head * D + db * 32 + r] = dq[db][v] * scale;
+    for (int v = 0; v < 16; v++) {
+        const int64_t i = iw0 + acc_row(v, h);
+        if (i < T) {
+            float* pq = dQ + i * qw + head * D + DB * r;
+            if (DB == 4) *reinterpret_cast<float4*>(pq) = make_float4(dq[0][v] * scale, dq[1 % DB][v] * scale, dq[2 % DB][v] * scale, dq[3 % DB][v] * scale);
+            else if (DB == 2) *reinterpret_cast<float2*>(pq) = make_float2(dq[0][v] * scale, dq[1 % DB][v] * scale);
+            else pq[0] = dq[0][v] * scale;
         }
+    }
+    }   // tile queue
+    tq_.leave();
 }
 
 // ---------------------------------------------------------------- host side
@@ -447,11 +607,34 @@ static int check_attn_shape(const char* who, int64_t T, int H, int KVH, int D) {
     return SERAPH_OK;
 }
 
+// One counter pair per launch, in rotation over the pool.
+static int acquire_tile_queue(unsigned int** out) {
+    static std::mutex mu;
+    static unsigned int* base[64] = {nullptr};
+    static unsigned next_slot = 0;
+    int dev = 0;
+    SERAPH_HIP_CHECK(hipGetDevice(&dev));
+    SERAPH_REQUIRE(dev >= 0 && dev < 64, "device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lk(mu);
+    if (!base[dev]) SERAPH_HIP_CHECK(hipGetSymbolAddress((void**)&base[dev], HIP_SYMBOL(g_tile_queues)));
+    *out = base[dev] + 2 * (next_slot++ % kQueueSlots);
+    return SERAPH_OK;
+}
+
+// Resident workgroups for a persistent launch: as many as fit per CU, never more than there are tiles.
+static unsigned persistent_grid(int64_t items, int D) {
+    int64_t cap = (int64_t)num_compute_units() * (D <= 64 ? 2 : 1);
+    return (unsigned)(items < cap ? items : cap);
+}
+
 template <int D>
 static int run_forward(const float* Q, const float* K, const float* V, float* O, float* lse, const uint32_t* seq_starts, int batch,
                        int64_t T, int H, int KVH, float scale, hipStream_t st) {
-    dim3 grid((unsigned)ceil_div(T, 128), (unsigned)H);
-    hipLaunchKernelGGL(attn_fwd_kernel<D>, grid, dim3(kAttnThreads), 0, st, Q, K, V, O, lse, seq_starts, batch, T, H, KVH, scale * kLog2e);
+    unsigned int* queue = nullptr;
+    int rc = acquire_tile_queue(&queue);
+    if (rc != SERAPH_OK) return rc;
+    dim3 grid(persistent_grid(ceil_div(T, 128) * H, D));
+    hipLaunchKernelGGL(attn_fwd_kernel<D>, grid, dim3(kAttnThreads), 0, st, Q, K, V, O, lse, seq_starts, batch, T, H, KVH, scale * kLog2e, queue);
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }
@@ -462,12 +645,16 @@ static int run_backward(const float* Q, const float* K, const float* V, const fl
                         int64_t T, int H, int KVH, float scale, hipStream_t st) {
     hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)ceil_div(T, 4)), dim3(256), 0, st, dO, O, delta, T, H);
     SERAPH_LAUNCH_CHECK();
-    dim3 gkv((unsigned)ceil_div(T, 128), (unsigned)KVH), gq((unsigned)ceil_div(T, 128), (unsigned)H);
+    unsigned int *qkv = nullptr, *qq = nullptr;
+    int rc = acquire_tile_queue(&qkv);
+    if (rc == SERAPH_OK) rc = acquire_tile_queue(&qq);
+    if (rc != SERAPH_OK) return rc;
+    dim3 gkv(persistent_grid(ceil_div(T, 128) * KVH, D)), gq(persistent_grid(ceil_div(T, 128) * H, D));
     hipLaunchKernelGGL(attn_bwd_dkv_kernel<D>, gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dK, dV, seq_starts, batch,
-                       T, H, KVH, scale, scale * kLog2e);
+                       T, H, KVH, scale, scale * kLog2e, qkv);
     SERAPH_LAUNCH_CHECK();
     hipLaunchKernelGGL(attn_bwd_dq_kernel<D>, gq, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dQ, seq_starts, batch,
-                       T, H, KVH, scale, scale * kLog2e);
+                       T, H, KVH, scale, scale * kLog2e, qq);
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }
