@@ -38,6 +38,8 @@ struct EmbWs {
     uint32_t* nuniq;    // [1]
     uint32_t* perm;     // [T]          positions grouped by token, arbitrary order inside a group
     uint32_t* sorted;   // [T]          the same, ascending inside each group
+    uint32_t* csum;     // [chunks]     per-chunk count totals, then bases
+    uint32_t* cnz;      // [chunks]     per-chunk distinct-token totals, then bases
 };
 
 static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -51,7 +53,10 @@ static size_t emb_ws_layout(int64_t T, int64_t vocab, char* base, EmbWs* w) {
     uint32_t* nuniq = take(1);
     uint32_t* perm = take((size_t)T);
     uint32_t* sorted = take((size_t)T);
-    if (w) { w->cnt = cnt; w->off = off; w->uniq = uniq; w->nuniq = nuniq; w->perm = perm; w->sorted = sorted; }
+    const size_t chunks = (size_t)((vocab + 4095) / 4096);
+    uint32_t* csum = take(chunks);
+    uint32_t* cnz = take(chunks);
+    if (w) { w->csum = csum; w->cnz = cnz; w->cnt = cnt; w->off = off; w->uniq = uniq; w->nuniq = nuniq; w->perm = perm; w->sorted = sorted; }
     return o;
 }
 
@@ -61,33 +66,87 @@ __global__ __launch_bounds__(256) void emb_count_kernel(const uint32_t* __restri
     if (p < T && (int64_t)tokens[p] < vocab) atomicAdd(&cnt[tokens[p]], 1u);     // integer: order-independent
 }
 
-// One workgroup scans the whole vocabulary: off = exclusive scan(cnt), uniq = tokens with
-// cnt > 0, and cnt is cleared so the fill kernel can reuse it as a cursor.
-__global__ __launch_bounds__(1024) void emb_scan_kernel(uint32_t* cnt, uint32_t* off, uint32_t* uniq,
-                                                        uint32_t* nuniq, int64_t vocab) {
-    __shared__ uint32_t s_sum[1024], s_nz[1024];
+// Exclusive scan of the per-token counts over the vocabulary in three small launches:
+// per-chunk totals (4096 tokens per workgroup, coalesced 16-byte loads), a serial scan of the
+// few chunk totals, then a rescan of every chunk from its base.  The last pass writes
+// off = exclusive scan(cnt) and uniq = tokens with cnt > 0 in ascending order, and clears cnt
+// so the fill kernel can reuse it as a cursor.
+constexpr int kScanBlock = 1024;
+constexpr int kScanChunk = 4 * kScanBlock;
+
+__device__ __forceinline__ uint4 load_cnt4(const uint32_t* cnt, int64_t v0, int64_t vocab) {
+    uint4 c = make_uint4(0, 0, 0, 0);
+    if (v0 + 3 < vocab && ((v0 & 3) == 0)) return *reinterpret_cast<const uint4*>(cnt + v0);
+    if (v0 < vocab) c.x = cnt[v0];
+    if (v0 + 1 < vocab) c.y = cnt[v0 + 1];
+    if (v0 + 2 < vocab) c.z = cnt[v0 + 2];
+    if (v0 + 3 < vocab) c.w = cnt[v0 + 3];
+    return c;
+}
+
+__global__ __launch_bounds__(kScanBlock) void emb_chunk_sums_kernel(const uint32_t* __restrict__ cnt, int64_t vocab,
+                                                                    uint32_t* __restrict__ csum, uint32_t* __restrict__ cnz) {
+    __shared__ uint32_t s_sum[kScanBlock / 64], s_nz[kScanBlock / 64];
+    const int64_t v0 = (int64_t)blockIdx.x * kScanChunk + 4 * threadIdx.x;
+    const uint4 c = load_cnt4(cnt, v0, vocab);
+    uint32_t sum = c.x + c.y + c.z + c.w;
+    uint32_t nz = (c.x ? 1u : 0u) + (c.y ? 1u : 0u) + (c.z ? 1u : 0u) + (c.w ? 1u : 0u);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { sum += __shfl_xor(sum, o, 64); nz += __shfl_xor(nz, o, 64); }
+    if ((threadIdx.x & 63) == 0) { s_sum[threadIdx.x >> 6] = sum; s_nz[threadIdx.x >> 6] = nz; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t a = 0, b = 0;
+        for (int w = 0; w < kScanBlock / 64; w++) { a += s_sum[w]; b += s_nz[w]; }
+        csum[blockIdx.x] = a;
+        cnz[blockIdx.x] = b;
+    }
+}
+
+// chunk totals -> exclusive chunk bases (in place); also off[vocab] and the number of distinct tokens
+__global__ void emb_chunk_scan_kernel(uint32_t* csum, uint32_t* cnz, int nchunks, uint32_t* off, uint32_t* nuniq, int64_t vocab) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    uint32_t a = 0, b = 0;
+    for (int i = 0; i < nchunks; i++) {
+        uint32_t x = csum[i], y = cnz[i];
+        csum[i] = a; cnz[i] = b;
+        a += x; b += y;
+    }
+    off[vocab] = a;
+    *nuniq = b;
+}
+
+__global__ __launch_bounds__(kScanBlock) void emb_chunk_write_kernel(uint32_t* __restrict__ cnt, int64_t vocab,
+                                                                     const uint32_t* __restrict__ csum,
+                                                                     const uint32_t* __restrict__ cnz,
+                                                                     uint32_t* __restrict__ off, uint32_t* __restrict__ uniq) {
+    __shared__ uint32_t s_sum[kScanBlock], s_nz[kScanBlock];
     const int tid = threadIdx.x;
-    const int64_t per = (vocab + 1023) / 1024;
-    const int64_t lo = tid * per, hi = (lo + per < vocab) ? lo + per : vocab;
-    uint32_t sum = 0, nz = 0;
-    for (int64_t v = lo; v < hi; v++) { uint32_t c = cnt[v]; sum += c; nz += c ? 1u : 0u; }
+    const int64_t v0 = (int64_t)blockIdx.x * kScanChunk + 4 * tid;
+    const uint4 c = load_cnt4(cnt, v0, vocab);
+    const uint32_t sum = c.x + c.y + c.z + c.w;
+    const uint32_t nz = (c.x ? 1u : 0u) + (c.y ? 1u : 0u) + (c.z ? 1u : 0u) + (c.w ? 1u : 0u);
     s_sum[tid] = sum; s_nz[tid] = nz;
     __syncthreads();
-    for (int d = 1; d < 1024; d <<= 1) {                       // Hillis-Steele inclusive scan
+    for (int d = 1; d < kScanBlock; d <<= 1) {                 // Hillis-Steele inclusive scan
         uint32_t a = tid >= d ? s_sum[tid - d] : 0u, b = tid >= d ? s_nz[tid - d] : 0u;
         __syncthreads();
         s_sum[tid] += a; s_nz[tid] += b;
         __syncthreads();
     }
-    uint32_t run = s_sum[tid] - sum, urun = s_nz[tid] - nz;    // exclusive prefixes of this lane's chunk
-    for (int64_t v = lo; v < hi; v++) {
-        uint32_t c = cnt[v];
-        off[v] = run;
-        if (c) uniq[urun++] = (uint32_t)v;
-        run += c;
-        cnt[v] = 0;
+    uint32_t run = csum[blockIdx.x] + s_sum[tid] - sum;         // exclusive prefix of this lane's four tokens
+    uint32_t urun = cnz[blockIdx.x] + s_nz[tid] - nz;
+    const uint32_t cs[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int64_t v = v0 + e;
+        if (v < vocab) {
+            off[v] = run;
+            if (cs[e]) uniq[urun++] = (uint32_t)v;
+            run += cs[e];
+            cnt[v] = 0;
+        }
     }
-    if (tid == 1023) { off[vocab] = s_sum[1023]; *nuniq = s_nz[1023]; }
 }
 
 __global__ __launch_bounds__(256) void emb_fill_kernel(const uint32_t* __restrict__ tokens, uint32_t* cnt,
@@ -184,7 +243,12 @@ int seraph_embedding_backward(const uint32_t* tokens, const float* dH, float* gr
     const dim3 tgrid((unsigned)ceil_div(T, 256));
     hipLaunchKernelGGL(emb_count_kernel, tgrid, dim3(256), 0, st, tokens, w.cnt, T, vocab);
     SERAPH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(emb_scan_kernel, dim3(1), dim3(1024), 0, st, w.cnt, w.off, w.uniq, w.nuniq, vocab);
+    const int nchunks = (int)ceil_div(vocab, kScanChunk);
+    hipLaunchKernelGGL(emb_chunk_sums_kernel, dim3(nchunks), dim3(kScanBlock), 0, st, w.cnt, vocab, w.csum, w.cnz);
+    SERAPH_LAUNCH_CHECK();
+    hipLaunchKernelGGL(emb_chunk_scan_kernel, dim3(1), dim3(64), 0, st, w.csum, w.cnz, nchunks, w.off, w.nuniq, vocab);
+    SERAPH_LAUNCH_CHECK();
+    hipLaunchKernelGGL(emb_chunk_write_kernel, dim3(nchunks), dim3(kScanBlock), 0, st, w.cnt, vocab, w.csum, w.cnz, w.off, w.uniq);
     SERAPH_LAUNCH_CHECK();
     hipLaunchKernelGGL(emb_fill_kernel, tgrid, dim3(256), 0, st, tokens, w.cnt, w.off, w.perm, T, vocab);
     SERAPH_LAUNCH_CHECK();

@@ -142,36 +142,44 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_f32_mfma_kernel(const float
         }
         const float* sa = lds_a[cur];
         const float* sb = lds_b[cur];
-#pragma unroll
-        for (int slab = 0; slab < kBK / 8; slab++) {
-            float fa[TM][4], fb[TN][4];
+        // Operand fragments are read from LDS one 8-deep slab ahead of the MFMAs that use them.
+        float fa[2][TM][4], fb[2][TN][4];
+        auto read_slab = [&](int slab, int buf) {
 #pragma unroll
             for (int i = 0; i < TM; i++) {
                 if (A_KC) {
                     const float4 t = *reinterpret_cast<const float4*>(sa + (wm0 + 32 * i + r) * (kBK + kPadK) + slab * 8 + 4 * h);
-                    fa[i][0] = t.x; fa[i][1] = t.y; fa[i][2] = t.z; fa[i][3] = t.w;
+                    fa[buf][i][0] = t.x; fa[buf][i][1] = t.y; fa[buf][i][2] = t.z; fa[buf][i][3] = t.w;
                 } else {
 #pragma unroll
-                    for (int s = 0; s < 4; s++) fa[i][s] = sa[(slab * 8 + 4 * h + s) * (BM + kPadM) + wm0 + 32 * i + r];
+                    for (int q = 0; q < 4; q++) fa[buf][i][q] = sa[(slab * 8 + 4 * h + q) * (BM + kPadM) + wm0 + 32 * i + r];
                 }
             }
 #pragma unroll
             for (int j = 0; j < TN; j++) {
                 if (B_KC) {
                     const float4 t = *reinterpret_cast<const float4*>(sb + (wn0 + 32 * j + r) * (kBK + kPadK) + slab * 8 + 4 * h);
-                    fb[j][0] = t.x; fb[j][1] = t.y; fb[j][2] = t.z; fb[j][3] = t.w;
+                    fb[buf][j][0] = t.x; fb[buf][j][1] = t.y; fb[buf][j][2] = t.z; fb[buf][j][3] = t.w;
                 } else {
 #pragma unroll
-                    for (int s = 0; s < 4; s++) fb[j][s] = sb[(slab * 8 + 4 * h + s) * (BN + kPadM) + wn0 + 32 * j + r];
+                    for (int q = 0; q < 4; q++) fb[buf][j][q] = sb[(slab * 8 + 4 * h + q) * (BN + kPadM) + wn0 + 32 * j + r];
                 }
             }
+        };
+        read_slab(0, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
 #pragma unroll
-            for (int s = 0; s < 4; s++)
+        for (int slab = 0; slab < kBK / 8; slab++) {
+            if (slab + 1 < kBK / 8) read_slab(slab + 1, (slab + 1) & 1);
+#pragma unroll
+            for (int q = 0; q < 4; q++)
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
                     for (int j = 0; j < TN; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[slab & 1][i][q], fb[slab & 1][j][q], acc[i][j], 0, 0, 0);
+            if (slab + 1 < kBK / 8) __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 4 * TM * TN, 0);
         }
         if (kt + 1 < nk) {
             la.store(lds_a[cur ^ 1]);

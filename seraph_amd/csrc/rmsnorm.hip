@@ -1,12 +1,14 @@
 // rmsnorm.hip - RMSNorm forward, batched RMSNorm backward with FP64 intermediates,
 // and the gain-less all-heads qk_norm with its derivative.
 //
-// One wavefront owns one row: the row (and, going backward, dy) lives in registers as
-// float4 slots, the two row sums are wave reductions (no LDS, no barrier), and each
-// byte of x / dy / dx crosses HBM exactly once.  The column reduction for grad_scale is
-// deterministic: lanes keep per-column partial sums over the rows their wave visits,
-// the block's four waves are combined through LDS, each block writes one partial row
-// to scratch, and a second small kernel adds the partial rows in a fixed order.
+// A row (and, going backward, dy) lives in registers as float4 slots while its two sums are
+// reduced, so each byte of x / dy / dx crosses HBM exactly once.  Short rows (<= 512) are
+// owned by one wavefront (wave reductions only, no LDS, no barrier); longer rows by one
+// workgroup, two float4 per lane at 2048 columns, which keeps the register footprint small
+// enough for four or more waves per SIMD to overlap the FP64 arithmetic with the loads.
+// The column reduction for grad_scale is deterministic: a lane keeps per-column partial sums
+// over the rows it visits, each workgroup writes one partial row to scratch, and a second
+// small kernel adds the partial rows in a fixed order.
 #include "common.hpp"
 
 namespace seraph {
@@ -165,6 +167,76 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const float* __rest
     }
 }
 
+// Rows of up to 8192 columns: one workgroup per row, VPL float4 per lane.  The four waves
+// exchange their two partial sums through a double-buffered LDS slot, one barrier per row.
+template <int VPL>
+__global__ __launch_bounds__(kBlock) void rmsnorm_bwd_block_kernel(const float* __restrict__ x,
+                                                                   const float* __restrict__ scale,
+                                                                   const float* __restrict__ dy,
+                                                                   float* __restrict__ dx,
+                                                                   float* __restrict__ partial,   // [gridDim.x, cols]
+                                                                   int64_t rows, int cols, float eps) {
+    __shared__ double red[2][kWavesPerBlock][2];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int n4 = cols >> 2;
+    float4 sc[VPL], gs[VPL];
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+        int i4 = threadIdx.x + kBlock * k;
+        sc[k] = i4 < n4 ? reinterpret_cast<const float4*>(scale)[i4] : make_float4(0, 0, 0, 0);
+        gs[k] = make_float4(0, 0, 0, 0);
+    }
+    int it = 0;
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x, it ^= 1) {
+        const float4* xr = reinterpret_cast<const float4*>(x + row * cols);
+        const float4* gr = reinterpret_cast<const float4*>(dy + row * cols);
+        float4 xv[VPL], gv[VPL];
+#pragma unroll
+        for (int k = 0; k < VPL; k++) {
+            int i4 = threadIdx.x + kBlock * k;
+            xv[k] = i4 < n4 ? xr[i4] : make_float4(0, 0, 0, 0);
+            gv[k] = i4 < n4 ? gr[i4] : make_float4(0, 0, 0, 0);
+        }
+        double ssq = 0.0, cp = 0.0;
+#pragma unroll
+        for (int k = 0; k < VPL; k++) {
+            const float* xs = &xv[k].x; const float* g = &gv[k].x; const float* s = &sc[k].x;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                double xd = (double)xs[e];
+                ssq += xd * xd;
+                cp += (double)g[e] * (double)s[e] * xd;
+            }
+        }
+        ssq = wave_sum(ssq);
+        cp = wave_sum(cp);
+        if (lane == 0) { red[it][wv][0] = ssq; red[it][wv][1] = cp; }
+        __syncthreads();
+        ssq = (red[it][0][0] + red[it][1][0]) + (red[it][2][0] + red[it][3][0]);
+        cp = (red[it][0][1] + red[it][1][1]) + (red[it][2][1] + red[it][3][1]);
+        RowStats st = row_stats(ssq, cp, cols, eps);
+        float4* dr = reinterpret_cast<float4*>(dx + row * cols);
+#pragma unroll
+        for (int k = 0; k < VPL; k++) {
+            int i4 = threadIdx.x + kBlock * k;
+            const float* xs = &xv[k].x; const float* g = &gv[k].x; const float* s = &sc[k].x;
+            float o[4]; float* acc = &gs[k].x;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                double xd = (double)xs[e], gd = (double)g[e];
+                acc[e] += (float)(gd * xd * st.inv);                                 // :90
+                o[e] = (float)(gd * (double)s[e] * st.inv - xd * st.k);              // :98
+            }
+            if (i4 < n4) dr[i4] = make_float4(o[0], o[1], o[2], o[3]);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+        int i4 = threadIdx.x + kBlock * k;
+        if (i4 < n4) reinterpret_cast<float4*>(partial + (size_t)blockIdx.x * cols)[i4] = gs[k];
+    }
+}
+
 // Generic shape: one wave per row, scalar accesses, per-wave partial rows in scratch.
 __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_generic_kernel(const float* __restrict__ x,
                                                                      const float* __restrict__ scale,
@@ -196,14 +268,31 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_generic_kernel(const float
     }
 }
 
-// grad_scale[c] += sum over partial rows, fixed order, double accumulator
-__global__ __launch_bounds__(kBlock) void colsum_add_kernel(const float* __restrict__ partial, int nparts,
-                                                            int64_t cols, float* __restrict__ grad_scale) {
-    int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (c >= cols) return;
+// grad_scale[c] += sum over partial rows in a fixed order.  64 columns x 16 row groups per
+// workgroup: group g adds rows g, g+16, ... in double, the 16 group sums are combined in order.
+__global__ __launch_bounds__(1024) void colsum_add_kernel(const float* __restrict__ partial, int nparts,
+                                                           int64_t cols, float* __restrict__ grad_scale) {
+    __shared__ double part[16][64];
+    const int cx = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const int64_t c = (int64_t)blockIdx.x * 64 + cx;
     double s = 0.0;
-    for (int p = 0; p < nparts; p++) s += (double)partial[(size_t)p * cols + c];
-    grad_scale[c] = (float)((double)grad_scale[c] + s);
+    if (c < cols) {
+        int p = g;
+        for (; p + 48 < nparts; p += 64) {
+            float a0 = partial[(size_t)p * cols + c], a1 = partial[(size_t)(p + 16) * cols + c];
+            float a2 = partial[(size_t)(p + 32) * cols + c], a3 = partial[(size_t)(p + 48) * cols + c];
+            s += (double)a0; s += (double)a1; s += (double)a2; s += (double)a3;
+        }
+        for (; p < nparts; p += 16) s += (double)partial[(size_t)p * cols + c];
+    }
+    part[g][cx] = s;
+    __syncthreads();
+    if (g == 0 && c < cols) {
+        double t = 0.0;
+#pragma unroll
+        for (int k = 0; k < 16; k++) t += part[k][cx];
+        grad_scale[c] = (float)((double)grad_scale[c] + t);
+    }
 }
 
 // ---------------------------------------------------------------- qk_norm
@@ -256,11 +345,25 @@ static int pick_vpl(int64_t cols) {
     return 0;
 }
 
+// wave-per-row kernels (short or odd rows): workgroups in the grid
 static int bwd_grid(int64_t rows) {
     int64_t want = ceil_div(rows, kWavesPerBlock * 2);          // at least two rows per wave
-    int64_t cap = (int64_t)num_compute_units() * 3;
+    int64_t cap = (int64_t)num_compute_units() * 4;
     if (want < 1) want = 1;
     return (int)(want < cap ? want : cap);
+}
+
+// block-per-row kernel: float4 slots per lane, or 0 when the shape does not qualify
+static int pick_block_vpl(int64_t cols) {
+    if (cols % 4 != 0 || cols <= 512) return 0;
+    int64_t n4 = cols / 4;
+    for (int v = 1; v <= 8; v *= 2) if (n4 <= kBlock * v) return v;
+    return 0;
+}
+
+static int bwd_block_grid(int64_t rows) {
+    int64_t cap = (int64_t)num_compute_units() * 4;
+    return (int)(rows < cap ? rows : cap);
 }
 
 }  // namespace seraph
@@ -297,7 +400,9 @@ int seraph_rmsnorm(const float* x, const float* scale, float* y, int64_t rows, i
 size_t seraph_rmsnorm_backward_ws_bytes(int64_t rows, int64_t cols) {
     if (rows <= 0 || cols <= 0) return 0;
     // the generic path needs one partial row per wave, the register path one per block
-    return (size_t)bwd_grid(rows) * kWavesPerBlock * (size_t)cols * sizeof(float);
+    size_t parts = (size_t)bwd_grid(rows) * kWavesPerBlock;
+    if ((size_t)bwd_block_grid(rows) > parts) parts = (size_t)bwd_block_grid(rows);
+    return parts * (size_t)cols * sizeof(float);
 }
 
 int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy, float* dx, float* grad_scale,
@@ -310,28 +415,38 @@ int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy,
         return SERAPH_ERR_WORKSPACE;
     }
     hipStream_t st = as_stream(s);
-    int grid = bwd_grid(rows);
     float* partial = (float*)ws;
-    int vpl = (aligned16(x) && aligned16(scale) && aligned16(dy) && aligned16(dx) && aligned16(ws)) ? pick_vpl(cols) : 0;
-    size_t lds = (size_t)kWavesPerBlock * cols * sizeof(float);
+    const bool aligned = aligned16(x) && aligned16(scale) && aligned16(dy) && aligned16(dx) && aligned16(ws);
+    const int bvpl = aligned ? pick_block_vpl(cols) : 0;
+    const int wvpl = (aligned && !bvpl && cols <= 512) ? pick_vpl(cols) : 0;
     int nparts;
-#define BWD(V) hipLaunchKernelGGL(rmsnorm_bwd_kernel<V>, dim3(grid), dim3(kBlock), lds, st, x, scale, dy, dx, partial, rows, (int)cols, eps)
-    switch (vpl) {
-        case 1: BWD(1); nparts = grid; break;
-        case 2: BWD(2); nparts = grid; break;
-        case 4: BWD(4); nparts = grid; break;
-        case 8: BWD(8); nparts = grid; break;
-        case 16: BWD(16); nparts = grid; break;
-        default: {
-            nparts = grid * kWavesPerBlock;
-            int rc = seraph_fill_u32(partial, 0u, (size_t)nparts * cols, s);
-            if (rc != SERAPH_OK) return rc;
-            hipLaunchKernelGGL(rmsnorm_bwd_generic_kernel, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, dx, partial, rows, cols, eps);
+    if (bvpl) {
+        const int grid = bwd_block_grid(rows);
+        nparts = grid;
+#define BBWD(V) hipLaunchKernelGGL(rmsnorm_bwd_block_kernel<V>, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, dx, partial, rows, (int)cols, eps)
+        switch (bvpl) {
+            case 1: BBWD(1); break;
+            case 2: BBWD(2); break;
+            case 4: BBWD(4); break;
+            default: BBWD(8); break;
         }
-    }
+#undef BBWD
+    } else if (wvpl) {
+        const int grid = bwd_grid(rows);
+        nparts = grid;
+        const size_t lds = (size_t)kWavesPerBlock * cols * sizeof(float);
+#define BWD(V) hipLaunchKernelGGL(rmsnorm_bwd_kernel<V>, dim3(grid), dim3(kBlock), lds, st, x, scale, dy, dx, partial, rows, (int)cols, eps)
+        if (wvpl == 1) BWD(1); else BWD(2);
 #undef BWD
+    } else {
+        const int grid = bwd_grid(rows);
+        nparts = grid * kWavesPerBlock;
+        int rc = seraph_fill_u32(partial, 0u, (size_t)nparts * cols, s);
+        if (rc != SERAPH_OK) return rc;
+        hipLaunchKernelGGL(rmsnorm_bwd_generic_kernel, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, dx, partial, rows, cols, eps);
+    }
     SERAPH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(colsum_add_kernel, dim3((unsigned)ceil_div(cols, kBlock)), dim3(kBlock), 0, st,
+    hipLaunchKernelGGL(colsum_add_kernel, dim3((unsigned)ceil_div(cols, 64)), dim3(1024), 0, st,
                        partial, nparts, cols, grad_scale);
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
