@@ -14,6 +14,7 @@
 namespace seraph {
 
 constexpr float kNegBig = -3.4e38f;      // the shader's initial maximum
+constexpr size_t kLastLevelCacheBytes = 256u << 20;   // MI355X Infinity Cache
 
 struct MaxSum { float m, s; };
 
@@ -223,7 +224,20 @@ extern "C" int seraph_cross_entropy_grad(const float* logits, const uint32_t* ta
         else SMALL(32);
 #undef SMALL
     } else if (vec) {
-        hipLaunchKernelGGL((ce_stream_kernel<1024, true>), grid, dim3(1024), 0, st, logits, targets, grad, loss_rows,
+        // Rows in flight are re-read by the second sweep: keep their total under the last-level cache.
+        // Two 1024-lane workgroups fit a CU; when that many long rows would overflow the cache, an
+        // LDS reservation of more than half a CU's LDS holds residency to one workgroup per CU.
+        const size_t in_flight = (size_t)num_compute_units() * 2 * (size_t)cols * sizeof(float);
+        const size_t lds_pad = in_flight > kLastLevelCacheBytes * 3 / 4 ? 84 * 1024 : 0;
+        if (lds_pad) {
+            static bool attr_set = false;
+            if (!attr_set) {
+                SERAPH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&ce_stream_kernel<1024, true>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_pad));
+                attr_set = true;
+            }
+        }
+        hipLaunchKernelGGL((ce_stream_kernel<1024, true>), grid, dim3(1024), lds_pad, st, logits, targets, grad, loss_rows,
                            seq_starts, batch, cols, scale);
     } else {
         hipLaunchKernelGGL((ce_stream_kernel<256, false>), grid, dim3(256), 0, st, logits, targets, grad, loss_rows,

@@ -8,11 +8,12 @@
 
 namespace seraph {
 
-constexpr int kBlock = 256;
+constexpr int kBlock = 256;           // nan check, 512-wide reduce
+constexpr int kStreamBlock = 512;     // streaming kernels
 constexpr int kUnroll = 4;      // independent float4 accesses in flight per lane and stream
 
 static inline int stream_grid(size_t n4) {
-    int64_t want = ceil_div((int64_t)n4, (int64_t)kBlock * kUnroll);
+    int64_t want = ceil_div((int64_t)n4, (int64_t)kStreamBlock * kUnroll);
     int64_t cap = (int64_t)num_compute_units() * 16;
     if (want < 1) want = 1;
     return (int)(want < cap ? want : cap);
@@ -21,9 +22,9 @@ static inline int stream_grid(size_t n4) {
 // F provides:  void vec(size_t i4) const   - one float4 slot
 //              void one(size_t i)  const   - one scalar element
 template <typename F>
-__global__ __launch_bounds__(kBlock) void stream_kernel(F f, size_t n4, size_t n, int vec_ok) {
-    const size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    const size_t stride = (size_t)gridDim.x * kBlock;
+__global__ __launch_bounds__(kStreamBlock) void stream_kernel(F f, size_t n4, size_t n, int vec_ok) {
+    const size_t tid = (size_t)blockIdx.x * kStreamBlock + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * kStreamBlock;
     if (vec_ok) {
         size_t i = tid;
         for (; i + (kUnroll - 1) * stride < n4; i += kUnroll * stride) {
@@ -42,7 +43,7 @@ static int launch_stream(F f, size_t n, bool vec_ok, hipStream_t st) {
     if (n == 0) return SERAPH_OK;
     size_t n4 = vec_ok ? n / 4 : 0;
     int grid = stream_grid(vec_ok ? n4 : n / 4 + 1);
-    hipLaunchKernelGGL(stream_kernel<F>, dim3(grid), dim3(kBlock), 0, st, f, n4, n, vec_ok ? 1 : 0);
+    hipLaunchKernelGGL(stream_kernel<F>, dim3(grid), dim3(kStreamBlock), 0, st, f, n4, n, vec_ok ? 1 : 0);
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }
