@@ -1,0 +1,63 @@
+"""The reference's own step driver (train_step -> train_step_gpu_full, src/train.c:6808/:4365),
+compiled unmodified from the Seraph tree and linked against this repository's vulkan_* backend
+(oracle/_ref/ref_step_hip, built by `make -C oracle ref` where the tree is present), must agree
+with the CPU oracle's step: same loss, same gradients, same weights after its AdamW schedule.
+
+What this pins: the oracle's op ORDER, scaling factors, target shift, warm-up schedule and
+optimizer constants against the reference's real driver code, and the backend's whole vulkan_*
+surface under the call pattern the reference actually uses (command recording, buffer reuse,
+fill ranges, accumulate flags).  The binary is skipped when it was not built."""
+import os
+import subprocess
+import numpy as np
+import pytest
+
+from tests.test_gpu_step import init_params, tensor_slices, check_tensors
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+BIN = os.path.join(HERE, "..", "oracle", "_ref", "ref_step_hip")
+
+CASES = [
+    dict(hidden=64, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=96, vocab=101, T=48, steps=2),
+    dict(hidden=128, layers=1, heads=2, kv_heads=1, head_dim=64, ffn=160, vocab=211, T=130, steps=3),
+]
+
+
+@pytest.mark.skipif(not os.path.exists(BIN), reason="oracle/_ref/ref_step_hip not built (needs the Seraph tree)")
+@pytest.mark.parametrize("case", CASES)
+def test_reference_driver_matches_oracle(orc, case, tmp_path):
+    case = dict(case)
+    T, steps = case.pop("T"), case.pop("steps")
+    lr0, theta = 2e-3, 10000.0
+    ocfg = orc.make_config(**case, rms_eps=1e-5, rope_theta=theta)
+    p = init_params(orc, ocfg, 11)
+    tok = np.random.default_rng(12).integers(0, case["vocab"], steps * T).astype(np.int32)
+
+    fin, fout = tmp_path / "in.bin", tmp_path / "out.bin"
+    with open(fin, "wb") as f:
+        np.array([case["hidden"], case["layers"], case["heads"], case["kv_heads"], case["head_dim"], case["ffn"],
+                  case["vocab"], steps, T], np.int32).tofile(f)
+        np.array([lr0, theta], np.float32).tofile(f)
+        p.tofile(f)
+        tok.tofile(f)
+    print(f"running {BIN} case={case} T={T} steps={steps}", flush=True)
+    r = subprocess.run([BIN, str(fin), str(fout)], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    out = np.fromfile(fout, np.float32)
+    n = p.size
+    assert out.size == steps + 2 * n
+    loss, g, w = out[:steps], out[steps:steps + n], out[steps + n:]
+
+    # oracle: the same steps with the reference's schedule (src/train.c:5449-5466)
+    rw, rm, rv = p.copy(), np.zeros_like(p), np.zeros_like(p)
+    starts = np.array([0, T], np.int32)
+    for s in range(steps):
+        ref_loss, ref_g = orc.step_full(ocfg, rw, tok[s * T:(s + 1) * T], starts)
+        assert abs(loss[s] - ref_loss) < 1e-5 * max(1.0, abs(ref_loss)), (s, loss[s], ref_loss)
+        lr = orc.lr_schedule(lr0, s + 1, 1)
+        rw, rm, rv = orc.adamw(rw, ref_g, rm, rv, lr, 0.9, 0.999, 0.01, 1e-8, s + 1)
+    sl = tensor_slices(ocfg)
+    check_tensors(g, ref_g, sl, "reference-driver grad")
+    check_tensors(w, rw, sl, "reference-driver weight")
