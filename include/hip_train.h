@@ -19,7 +19,7 @@
  *
  * Arena layout (floats): embed[V,h], final_norm[h], then per layer
  *   in_norm[h], q[q,h], k[kv,h], v[kv,h], o[h,q], post_norm[h], gate[f,h], up[f,h], down[h,f].
- * LoRA arena: per layer, for each of q,k,v,o selected by lora_mask (bit 0..3): A[r,in], B[out,r].
+ * LoRA arena: per layer, for each of q,k,v,o,gate,up,down selected by lora_mask (bit 0..6): A[r,in], B[out,r].
  */
 #ifndef HIP_TRAIN_H
 #define HIP_TRAIN_H
@@ -37,7 +37,7 @@ typedef struct {
     float   rope_theta;
     int32_t lora_rank;      /* 0 = full-weight training */
     float   lora_alpha;
-    int32_t lora_mask;      /* bit0 q, bit1 k, bit2 v, bit3 o */
+    int32_t lora_mask;      /* bit0 q, 1 k, 2 v, 3 o, 4 gate, 5 up, 6 down (src/lora.c:372-396) */
 } hip_model_config_t;
 
 typedef struct {

@@ -12,17 +12,21 @@
  * oracle's step against the reference's own driver.
  *
  * usage: ref_step_hip <in.bin> <out.bin>
- *   in : int32 hidden, layers, heads, kv_heads, head_dim, ffn, vocab, steps, T
- *        float32 lr, rope_theta
+ *   in : int32 hidden, layers, heads, kv_heads, head_dim, ffn, vocab, steps, T, lora_rank, lora_mask
+ *        float32 lr, rope_theta, lora_alpha
  *        float32 params[...] in this build's arena order
+ *        float32 lora[...]   (lora_rank > 0) per layer, per selected adapter q k v o gate up down: A[r,in], B[out,r]
  *        int32 tokens[steps * T]
- *   out: float32 loss[steps], float32 grads[...] (last step), float32 weights[...] (after last step)
+ *   out (full): float32 loss[steps], grads[...] (last step), weights[...] (after last step)
+ *   out (LoRA): float32 loss[steps], lora weights[...], adam m[...], adam v[...]  (after last step; pulled
+ *               back through the reference's own save_checkpoint -> lora_gpu_download_to_cpu, src/train.c:7760-7767)
  */
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 
 #include "model_config.h"
+#include "lora.h"
 #include "train.h"
 #include "vulkan_backend.h"
 
@@ -34,10 +38,10 @@ int main(int argc, char** argv) {
     if (argc != 3) { fprintf(stderr, "usage: %s in.bin out.bin\n", argv[0]); return 2; }
     FILE* f = fopen(argv[1], "rb");
     if (!f) { perror("in.bin"); return 2; }
-    int hdr[9]; float fl[2];
+    int hdr[11]; float fl[3];
     if (rd(hdr, sizeof(hdr), f) || rd(fl, sizeof(fl), f)) return 2;
     const int hidden = hdr[0], layers = hdr[1], heads = hdr[2], kvh = hdr[3], hd = hdr[4], ffn = hdr[5], vocab = hdr[6];
-    const int steps = hdr[7], T = hdr[8];
+    const int steps = hdr[7], T = hdr[8], rank = hdr[9], mask = hdr[10];
 
     model_config_t cfg;
     memset(&cfg, 0, sizeof(cfg));
@@ -48,14 +52,14 @@ int main(int argc, char** argv) {
     train_state_t st;
     memset(&st, 0, sizeof(st));
     st.config = &cfg;
-    st.use_full_training = 1;
-    st.full_weights = trainable_weights_alloc(&cfg);
+    st.use_full_training = rank == 0;
+    trainable_weights_t* w = trainable_weights_alloc(&cfg);   /* in LoRA mode only a host staging area */
+    if (rank == 0) st.full_weights = w;
     st.learning_rate = fl[0];
     st.gradient_accumulation_steps = 1;
-    if (!st.full_weights) return 3;
+    if (!w) return 3;
 
     /* this build's arena order: embed, final_norm, per layer in_norm q k v o post_norm gate up down */
-    trainable_weights_t* w = st.full_weights;
     int nslots = 2 + 9 * layers, k = 0;
     slot_t* slots = calloc((size_t)nslots, sizeof(slot_t));
     slots[k++].t = &w->embed_tokens; slots[k++].t = &w->final_norm;
@@ -69,6 +73,29 @@ int main(int argc, char** argv) {
     for (int i = 0; i < nslots; i++) {
         if (rd(slots[i].t->weight, slots[i].t->size * sizeof(float), f)) { fprintf(stderr, "short params\n"); return 2; }
         total += slots[i].t->size;
+    }
+    /* LoRA adapters (src/lora.c:342-397 creates q and v; the others are added the same way) */
+    lora_adapter_t*** kinds[7];
+    size_t nlora = 0;
+    if (rank > 0) {
+        lora_model_t* lm = lora_model_create_from_config(&cfg, rank, fl[2]);
+        const int qd = heads * hd, kvd = kvh * hd;
+        const int ins[7] = {hidden, hidden, hidden, qd, hidden, hidden, ffn};
+        const int outs[7] = {qd, kvd, kvd, hidden, ffn, ffn, hidden};
+        kinds[0] = &lm->q_adapters; kinds[1] = &lm->k_adapters; kinds[2] = &lm->v_adapters; kinds[3] = &lm->o_adapters;
+        kinds[4] = &lm->gate_adapters; kinds[5] = &lm->up_adapters; kinds[6] = &lm->down_adapters;
+        lm->apply_to_q = mask & 1; lm->apply_to_k = (mask >> 1) & 1; lm->apply_to_v = (mask >> 2) & 1;
+        lm->apply_to_o = (mask >> 3) & 1; lm->apply_to_ffn = (mask >> 4) != 0;
+        for (int l = 0; l < layers; l++)
+            for (int p = 0; p < 7; p++) {
+                lora_adapter_t** slot = &(*kinds[p])[l];
+                if (!((mask >> p) & 1)) { if (*slot) { lora_adapter_free(*slot); *slot = NULL; } continue; }
+                if (!*slot) *slot = lora_adapter_create(ins[p], outs[p], rank, fl[2]);
+                size_t na = (size_t)rank * ins[p], nb = (size_t)outs[p] * rank;
+                if (rd((*slot)->A, na * sizeof(float), f) || rd((*slot)->B, nb * sizeof(float), f)) { fprintf(stderr, "short lora\n"); return 2; }
+                nlora += na + nb;
+            }
+        st.lora = lm;
     }
     int* tokens = malloc((size_t)steps * T * sizeof(int));
     if (rd(tokens, (size_t)steps * T * sizeof(int), f)) { fprintf(stderr, "short tokens\n"); return 2; }
@@ -84,8 +111,47 @@ int main(int argc, char** argv) {
     ctx->max_buffer_size = st.max_tensor_size;
     ctx->max_fwd_buffer_size = st.max_tensor_size;
 
+    if (rank > 0) {
+        /* frozen base weights: what ensure_lora_gpu_base_weights (src/train.c:2039-2151) leaves in the context,
+         * minus the BF16 checkpoint it reads them from -- FP32 values go up as they are */
+        ctx->gpu_weights_num_layers = layers; ctx->gpu_weights_hidden_size = hidden;
+        ctx->gpu_weights_intermediate_size = ffn; ctx->gpu_weights_vocab_size = vocab;
+        ctx->gpu_weights_q_dim = heads * hd; ctx->gpu_weights_kv_dim = kvh * hd;
+        void*** arrs[9] = {(void***)&ctx->gpu_w_in_norm, (void***)&ctx->gpu_w_q, (void***)&ctx->gpu_w_k, (void***)&ctx->gpu_w_v,
+                           (void***)&ctx->gpu_w_o, (void***)&ctx->gpu_w_post_norm, (void***)&ctx->gpu_w_gate,
+                           (void***)&ctx->gpu_w_up, (void***)&ctx->gpu_w_down};
+        for (int i = 0; i < 9; i++) *arrs[i] = calloc((size_t)layers, sizeof(void*));
+        for (int i = 0; i < nslots; i++) {
+            vulkan_buffer_t* b = vulkan_buffer_create(ctx, slots[i].t->size * sizeof(float));
+            vulkan_buffer_upload(ctx, b, slots[i].t->weight, slots[i].t->size);
+            if (i == 0) ctx->gpu_w_embed = b;
+            else if (i == 1) ctx->gpu_w_final_norm = b;
+            else (*arrs[(i - 2) % 9])[(i - 2) / 9] = b;
+        }
+    }
+
     float* loss = malloc((size_t)steps * sizeof(float));
     for (int s = 0; s < steps; s++) loss[s] = train_step(&st, tokens + (size_t)s * T, T);
+
+    if (rank > 0) {
+        if (save_checkpoint(&st, argv[2]) != 0) return 5;      /* pulls A, B, m, v back into st.lora */
+        FILE* o = fopen(argv[2], "wb");
+        if (!o) { perror("out.bin"); return 2; }
+        fwrite(loss, sizeof(float), (size_t)steps, o);
+        for (int pass = 0; pass < 3; pass++)
+            for (int l = 0; l < layers; l++)
+                for (int p = 0; p < 7; p++) {
+                    lora_adapter_t* a = (*kinds[p])[l];
+                    if (!a) continue;
+                    size_t na = (size_t)a->rank * a->in_dim, nb = (size_t)a->out_dim * a->rank;
+                    fwrite(pass == 0 ? a->A : pass == 1 ? a->m_A : a->v_A, sizeof(float), na, o);
+                    fwrite(pass == 0 ? a->B : pass == 1 ? a->m_B : a->v_B, sizeof(float), nb, o);
+                }
+        fclose(o);
+        printf("ref_step_hip: LoRA %d steps of %d tokens, %zu adapter parameters, optimizer_step=%d, last loss %.6f\n",
+               steps, T, nlora, st.optimizer_step, loss[steps - 1]);
+        return 0;
+    }
 
     /* device buffers the reference step keeps in its context (include/vulkan_backend.h:258-311) */
     k = 0;

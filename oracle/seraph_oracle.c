@@ -516,15 +516,16 @@ int64_t orc_param_count(const orc_config_t* c) {
 }
 
 /* per-layer LoRA block: for each selected projection, A[r,in] then B[out,r] */
-typedef struct { int64_t A[4], B[4], in[4], out[4], stride; } lora_layout_t;
+typedef struct { int64_t A[7], B[7], in[7], out[7], stride; } lora_layout_t;
 
 static lora_layout_t make_lora_layout(const orc_config_t* c) {
     lora_layout_t L;
     int64_t h = c->hidden, qd = (int64_t)c->heads * c->head_dim, kv = (int64_t)c->kv_heads * c->head_dim;
-    int64_t ins[4]  = { h, h, h, qd };
-    int64_t outs[4] = { qd, kv, kv, h };
+    int64_t f = c->ffn;
+    int64_t ins[7]  = { h, h, h, qd, h, h, f };      /* q k v o gate up down: src/lora.c:372-396 */
+    int64_t outs[7] = { qd, kv, kv, h, f, f, h };
     int64_t o = 0;
-    for (int p = 0; p < 4; p++) {
+    for (int p = 0; p < 7; p++) {
         L.in[p] = ins[p]; L.out[p] = outs[p];
         L.A[p] = L.B[p] = -1;
         if (c->lora_rank > 0 && (c->lora_mask >> p) & 1) {
@@ -635,10 +636,13 @@ static float step_impl(const orc_config_t* c, const float* P, float* G,
         orc_rmsnorm(hidden, W + L.rel.post_norm, xn_ffn[l], T, h, eps);
         gate[l] = fnew(T * f); up[l] = fnew(T * f); silu_out[l] = fnew(T * f); ffn_h[l] = fnew(T * f);
         orc_matmul(xn_ffn[l], W + L.rel.gate, gate[l], T, f, h, 0, 1, 0);
+        if (lora && LL.A[4] >= 0) lora_forward_add(xn_ffn[l], gate[l], LW + LL.A[4], LW + LL.B[4], ltmp, T, h, f, r, ls);
         orc_matmul(xn_ffn[l], W + L.rel.up, up[l], T, f, h, 0, 1, 0);
+        if (lora && LL.A[5] >= 0) lora_forward_add(xn_ffn[l], up[l], LW + LL.A[5], LW + LL.B[5], ltmp, T, h, f, r, ls);
         orc_silu(gate[l], silu_out[l], T * f);
         for (int64_t i = 0; i < T * f; i++) ffn_h[l][i] = silu_out[l][i] * up[l][i];
         orc_matmul(ffn_h[l], W + L.rel.down, tmp_h, T, h, f, 0, 1, 0);
+        if (lora && LL.A[6] >= 0) lora_forward_add(ffn_h[l], tmp_h, LW + LL.A[6], LW + LL.B[6], ltmp, T, f, h, r, ls);
         add_into(hidden, hidden, tmp_h, T * h);
     }
     float* final_in = fnew(T * h); memcpy(final_in, hidden, (size_t)(T * h) * 4);
@@ -678,8 +682,14 @@ static float step_impl(const orc_config_t* c, const float* P, float* G,
 
         if (!lora) orc_matmul(g_hidden, ffn_h[l], GW + L.rel.down, h, f, T, 1, 0, 1);
         orc_matmul(g_hidden, W + L.rel.down, g_ffn, T, f, h, 0, 0, 0);
+        if (lora && LL.A[6] >= 0)                                            /* src/train.c:6422-6429 */
+            lora_backward(g_hidden, ffn_h[l], LW + LL.A[6], LW + LL.B[6], LGW + LL.A[6], LGW + LL.B[6], ltmp, T, f, h, r, ls);
         orc_mul_backward(silu_out[l], up[l], g_ffn, g_gate, g_up, T * f);
         orc_silu_backward(gate[l], g_gate, g_gate, T * f);
+        if (lora && LL.A[4] >= 0)                                            /* src/train.c:6446-6461 */
+            lora_backward(g_gate, xn_ffn[l], LW + LL.A[4], LW + LL.B[4], LGW + LL.A[4], LGW + LL.B[4], ltmp, T, h, f, r, ls);
+        if (lora && LL.A[5] >= 0)
+            lora_backward(g_up, xn_ffn[l], LW + LL.A[5], LW + LL.B[5], LGW + LL.A[5], LGW + LL.B[5], ltmp, T, h, f, r, ls);
         if (!lora) {
             orc_matmul(g_gate, xn_ffn[l], GW + L.rel.gate, f, h, T, 1, 0, 1);
             orc_matmul(g_up, xn_ffn[l], GW + L.rel.up, f, h, T, 1, 0, 1);

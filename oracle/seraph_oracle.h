@@ -154,7 +154,7 @@ typedef struct {
     /* LoRA (rank 0 = full-weight training) */
     int32_t lora_rank;
     float   lora_alpha;
-    int32_t lora_mask;    /* bit0 q, bit1 k, bit2 v, bit3 o */
+    int32_t lora_mask;    /* bit0 q, 1 k, 2 v, 3 o, 4 gate, 5 up, 6 down */
 } orc_config_t;
 
 /* Element offsets of every tensor inside one flat parameter vector:
@@ -162,7 +162,7 @@ typedef struct {
  *   in_norm[h], q[q,h], k[kv,h], v[kv,h], o[h,q], post_norm[h],
  *   gate[f,h], up[f,h], down[h,f].                                       */
 int64_t orc_param_count(const orc_config_t* c);
-/* LoRA vector: per layer, for each of q,k,v,o selected by lora_mask in that
+/* LoRA vector: per layer, for each of q,k,v,o,gate,up,down selected by lora_mask in that
  * order: A[r,in] then B[out,r]. */
 int64_t orc_lora_param_count(const orc_config_t* c);
 

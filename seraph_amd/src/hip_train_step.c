@@ -24,7 +24,7 @@
 #define OPT_MAX_EVENTS  32768
 
 typedef struct { int64_t in_norm, q, k, v, o, post_norm, gate, up, down, stride; } layer_layout_t;
-typedef struct { int64_t A[4], B[4], in[4], out[4], stride; } lora_layout_t;
+typedef struct { int64_t A[7], B[7], in[7], out[7], stride; } lora_layout_t;   /* q k v o gate up down */
 
 typedef struct {
     float *layer_in, *xn_attn, *q, *k, *v, *attn_out, *lse, *post_in, *xn_ffn, *gate, *up, *ffn_h;
@@ -149,9 +149,9 @@ static void make_layouts(hip_trainer_t* t) {
     t->L.down = o; o += h * f;
     t->L.stride = o;
     t->nparams = t->off_layer0 + o * c->layers;
-    int64_t ins[4] = {h, h, h, qd}, outs[4] = {qd, kv, kv, h};
+    int64_t ins[7] = {h, h, h, qd, h, h, f}, outs[7] = {qd, kv, kv, h, f, f, h};   /* src/lora.c:372-396 */
     o = 0;
-    for (int p = 0; p < 4; p++) {
+    for (int p = 0; p < 7; p++) {
         t->LL.in[p] = ins[p]; t->LL.out[p] = outs[p];
         t->LL.A[p] = t->LL.B[p] = -1;
         if (c->lora_rank > 0 && ((c->lora_mask >> p) & 1)) {
@@ -443,9 +443,12 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         OP("add", 0.0, 12.0 * (double)(T * h), seraph_add(a->layer_in, t->tmp_h, a->post_in, (size_t)(T * h), s));
         OP("rmsnorm", 0.0, 8.0 * (double)(T * h), seraph_rmsnorm(a->post_in, W + t->L.post_norm, a->xn_ffn, T, h, eps, s));
         GEMM(a->xn_ffn, W + t->L.gate, a->gate, T, f, h, 0, 1, 0);
+        if (lora && t->LL.A[4] >= 0 && lora_forward_add(t, a->xn_ffn, a->gate, LW + t->LL.A[4], LW + t->LL.B[4], T, h, f)) return -1.0f;
         GEMM(a->xn_ffn, W + t->L.up, a->up, T, f, h, 0, 1, 0);
+        if (lora && t->LL.A[5] >= 0 && lora_forward_add(t, a->xn_ffn, a->up, LW + t->LL.A[5], LW + t->LL.B[5], T, h, f)) return -1.0f;
         OP("swiglu", 0.0, 12.0 * (double)(T * f), seraph_swiglu(a->gate, a->up, a->ffn_h, (size_t)(T * f), s));
         GEMM(a->ffn_h, W + t->L.down, t->tmp_h, T, h, f, 0, 1, 0);
+        if (lora && t->LL.A[6] >= 0 && lora_forward_add(t, a->ffn_h, t->tmp_h, LW + t->LL.A[6], LW + t->LL.B[6], T, f, h)) return -1.0f;
         OP("add", 0.0, 12.0 * (double)(T * h), seraph_add(a->post_in, t->tmp_h, next, (size_t)(T * h), s));
     }
     OP("rmsnorm", 0.0, 8.0 * (double)(T * h), seraph_rmsnorm(t->final_in, P + t->off_final_norm, t->xn_final, T, h, eps, s));
@@ -480,7 +483,13 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         /* FFN */
         if (!lora) GEMM(t->g_hidden, a->ffn_h, GW + t->L.down, h, f, T, 1, 0, 1);
         GEMM(t->g_hidden, W + t->L.down, t->g_ffn, T, f, h, 0, 0, 0);
+        if (lora && t->LL.A[6] >= 0 &&                                       /* src/train.c:6422-6429 */
+            lora_backward(t, t->g_hidden, a->ffn_h, LW + t->LL.A[6], LW + t->LL.B[6], LGW + t->LL.A[6], LGW + t->LL.B[6], T, f, h)) return -1.0f;
         OP("swiglu_backward", 0.0, 20.0 * (double)(T * f), seraph_swiglu_backward(a->gate, a->up, t->g_ffn, t->g_gate, t->g_up, (size_t)(T * f), s));
+        if (lora && t->LL.A[4] >= 0 &&                                       /* src/train.c:6446-6461 */
+            lora_backward(t, t->g_gate, a->xn_ffn, LW + t->LL.A[4], LW + t->LL.B[4], LGW + t->LL.A[4], LGW + t->LL.B[4], T, h, f)) return -1.0f;
+        if (lora && t->LL.A[5] >= 0 &&
+            lora_backward(t, t->g_up, a->xn_ffn, LW + t->LL.A[5], LW + t->LL.B[5], LGW + t->LL.A[5], LGW + t->LL.B[5], T, h, f)) return -1.0f;
         if (!lora) {
             GEMM(t->g_gate, a->xn_ffn, GW + t->L.gate, f, h, T, 1, 0, 1);
             GEMM(t->g_up, a->xn_ffn, GW + t->L.up, f, h, T, 1, 0, 1);

@@ -33,12 +33,13 @@ def split_params(cfg, flat):
 def split_lora(cfg, flat):
     h = cfg.hidden
     qd, kv, r = cfg.heads * cfg.head_dim, cfg.kv_heads * cfg.head_dim, cfg.lora_rank
-    ins, outs = [h, h, h, qd], [qd, kv, kv, h]
+    f = cfg.ffn
+    ins, outs = [h, h, h, qd, h, h, f], [qd, kv, kv, h, f, f, h]
     o = 0
     layers = []
     for _ in range(cfg.layers):
         d = {}
-        for p, name in enumerate("qkvo"):
+        for p, name in enumerate(("q", "k", "v", "o", "gate", "up", "down")):
             if (cfg.lora_mask >> p) & 1:
                 A = flat[o:o + r * ins[p]].view(r, ins[p]); o += r * ins[p]
                 B = flat[o:o + outs[p] * r].view(outs[p], r); o += outs[p] * r
@@ -107,8 +108,8 @@ def loss_fn(cfg, P, tokens, seq_starts, lora=None, drop_adapter_dgrad=True):
         a = attention(q, k, v, seq_id, H, KVH, D)
         x = x + proj(a, W["o"], ad.get("o"))
         xn = rmsnorm(x, W["post_norm"], cfg.rms_eps)
-        g, u = xn @ W["gate"].T, xn @ W["up"].T
-        x = x + (torch.nn.functional.silu(g) * u) @ W["down"].T
+        g, u = proj(xn, W["gate"], ad.get("gate")), proj(xn, W["up"], ad.get("up"))
+        x = x + proj(torch.nn.functional.silu(g) * u, W["down"], ad.get("down"))
     logits = rmsnorm(x, P["final_norm"], cfg.rms_eps) @ P["embed"].T
     valid = np.ones(T, bool)
     valid[starts[1:] - 1] = False

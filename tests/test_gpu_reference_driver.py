@@ -25,7 +25,26 @@ CASES = [
 ]
 
 
-@pytest.mark.skipif(not os.path.exists(BIN), reason="oracle/_ref/ref_step_hip not built (needs the Seraph tree)")
+needs_bin = pytest.mark.skipif(not os.path.exists(BIN), reason="oracle/_ref/ref_step_hip not built (needs the Seraph tree)")
+
+
+def run_driver(tmp_path, case, steps, T, lr0, theta, p, tok, rank=0, mask=0, alpha=0.0, lora=None):
+    fin, fout = tmp_path / "in.bin", tmp_path / "out.bin"
+    with open(fin, "wb") as f:
+        np.array([case["hidden"], case["layers"], case["heads"], case["kv_heads"], case["head_dim"], case["ffn"],
+                  case["vocab"], steps, T, rank, mask], np.int32).tofile(f)
+        np.array([lr0, theta, alpha], np.float32).tofile(f)
+        p.tofile(f)
+        if lora is not None:
+            lora.tofile(f)
+        tok.tofile(f)
+    print(f"running {BIN} case={case} T={T} steps={steps} rank={rank} mask={mask:#b}", flush=True)
+    r = subprocess.run([BIN, str(fin), str(fout)], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    return np.fromfile(fout, np.float32)
+
+
+@needs_bin
 @pytest.mark.parametrize("case", CASES)
 def test_reference_driver_matches_oracle(orc, case, tmp_path):
     case = dict(case)
@@ -34,18 +53,7 @@ def test_reference_driver_matches_oracle(orc, case, tmp_path):
     ocfg = orc.make_config(**case, rms_eps=1e-5, rope_theta=theta)
     p = init_params(orc, ocfg, 11)
     tok = np.random.default_rng(12).integers(0, case["vocab"], steps * T).astype(np.int32)
-
-    fin, fout = tmp_path / "in.bin", tmp_path / "out.bin"
-    with open(fin, "wb") as f:
-        np.array([case["hidden"], case["layers"], case["heads"], case["kv_heads"], case["head_dim"], case["ffn"],
-                  case["vocab"], steps, T], np.int32).tofile(f)
-        np.array([lr0, theta], np.float32).tofile(f)
-        p.tofile(f)
-        tok.tofile(f)
-    print(f"running {BIN} case={case} T={T} steps={steps}", flush=True)
-    r = subprocess.run([BIN, str(fin), str(fout)], capture_output=True, text=True, timeout=100)
-    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
-    out = np.fromfile(fout, np.float32)
+    out = run_driver(tmp_path, case, steps, T, lr0, theta, p, tok)
     n = p.size
     assert out.size == steps + 2 * n
     loss, g, w = out[:steps], out[steps:steps + n], out[steps + n:]
@@ -61,3 +69,34 @@ def test_reference_driver_matches_oracle(orc, case, tmp_path):
     sl = tensor_slices(ocfg)
     check_tensors(g, ref_g, sl, "reference-driver grad")
     check_tensors(w, rw, sl, "reference-driver weight")
+
+
+@needs_bin
+@pytest.mark.parametrize("mask", [0b0000101, 0b0001111, 0b1111111])
+def test_reference_lora_driver_matches_oracle(orc, mask, tmp_path):
+    """train_step_gpu_lora (src/train.c:5846-6719) over this backend: adapters, Adam moments and loss
+    after three steps against the oracle's LoRA step + AdamW.  The first moment after step 1 is
+    0.1 * gradient, so the moments pin the gradients themselves; from step 2 on B != 0, which is
+    where the reference's dropped adapter input-gradient term (grad_input = NULL) matters."""
+    case = dict(hidden=64, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=96, vocab=101)
+    T, steps, rank, alpha, lr0, theta = 57, 3, 8, 16.0, 5e-2, 10000.0
+    ocfg = orc.make_config(**case, rms_eps=1e-5, rope_theta=theta, lora_rank=rank, lora_alpha=alpha, lora_mask=mask)
+    p = init_params(orc, ocfg, 21)
+    r = np.random.default_rng(22)
+    n = orc.lora_param_count(ocfg)
+    lo = (0.05 * r.standard_normal(n)).astype(np.float32)
+    tok = r.integers(0, case["vocab"], steps * T).astype(np.int32)
+    out = run_driver(tmp_path, case, steps, T, lr0, theta, p, tok, rank, mask, alpha, lo)
+    assert out.size == steps + 3 * n
+    loss, w, m, v = out[:steps], out[steps:steps + n], out[steps + n:steps + 2 * n], out[steps + 2 * n:]
+
+    rw, rm, rv = lo.copy(), np.zeros_like(lo), np.zeros_like(lo)
+    starts = np.array([0, T], np.int32)
+    for s in range(steps):
+        ref_loss, ref_g = orc.step_lora(ocfg, p, rw, tok[s * T:(s + 1) * T], starts)
+        assert abs(loss[s] - ref_loss) < 1e-5 * max(1.0, abs(ref_loss)), (s, loss[s], ref_loss)
+        rw, rm, rv = orc.adamw(rw, ref_g, rm, rv, orc.lr_schedule(lr0, s + 1, 1), 0.9, 0.999, 0.01, 1e-8, s + 1)
+    for name, got, ref in (("adapter", w, rw), ("adam m", m, rm), ("adam v", v, rv)):
+        bad = np.abs(got.astype(np.float64) - ref) > 1e-5 + 1e-4 * np.abs(ref)
+        assert not bad.any(), f"{name}: {bad.sum()}/{bad.size} outside tolerance, max {np.abs(got - ref).max():.3e}"
+    assert np.abs(w - lo).max() > 1e-5            # the adapters did move

@@ -130,10 +130,11 @@ def test_full_step_gradient_accumulation(tr, orc):
     t.close()
 
 
+@pytest.mark.parametrize("mask", [0b0001111, 0b1111111, 0b1010101])
 @pytest.mark.parametrize("b_zero", [True, False])
-def test_lora_step(tr, orc, b_zero):
+def test_lora_step(tr, orc, b_zero, mask):
     case = dict(hidden=64, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=96, vocab=101, lora_rank=16,
-                lora_alpha=32.0, lora_mask=0b1111)
+                lora_alpha=32.0, lora_mask=mask)
     starts = np.array([0, 41, 90], np.int32)
     ocfg = orc.make_config(**case)
     cfg = tr.model_config(**case)
@@ -142,10 +143,12 @@ def test_lora_step(tr, orc, b_zero):
     r = rng(7)
     lo = (0.05 * r.standard_normal(orc.lora_param_count(ocfg))).astype(np.float32)
     if b_zero:                                         # the reference's initial state: B = 0 (src/lora.c:76-78)
-        h, qd, kv, rk = 64, 128, 64, 16
+        h, qd, kv, f, rk = 64, 128, 64, 96, 16
         o = 0
         for _ in range(2):
-            for i, oo in ((h, qd), (h, kv), (h, kv), (qd, h)):
+            for bit, (i, oo) in enumerate(((h, qd), (h, kv), (h, kv), (qd, h), (h, f), (h, f), (f, h))):
+                if not (mask >> bit) & 1:
+                    continue
                 o += rk * i
                 lo[o:o + oo * rk] = 0
                 o += oo * rk

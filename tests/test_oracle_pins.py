@@ -362,9 +362,10 @@ def test_step_full_single_sequence_equals_unpacked(orc):
     assert l1 == l2 and (g1 == g2).all()
 
 
+@pytest.mark.parametrize("mask", [0b0001111, 0b1111111, 0b1010101])
 @pytest.mark.parametrize("b_zero", [True, False])
-def test_step_lora_vs_autograd(orc, b_zero):
-    cfg = _tiny_cfg(orc, lora_rank=4, lora_alpha=8.0, lora_mask=0b1111)
+def test_step_lora_vs_autograd(orc, b_zero, mask):
+    cfg = _tiny_cfg(orc, lora_rank=4, lora_alpha=8.0, lora_mask=mask)
     p = _init(orc, cfg, 104)
     r = rng(105)
     lo = (0.05 * r.standard_normal(orc.lora_param_count(cfg))).astype(np.float32)
