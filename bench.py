@@ -3,12 +3,18 @@
 training step on ONE MI355X, with the dominant kernel's roofline fraction measured live and
 the CPU oracle timed beside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c1] [--pmc-calibration]
 
 Workloads (BASELINE.json configs): c5 = Qwen3-1.7B-shape full-weight FP32 training,
 4 x 4096 tokens (default); c4 = the same model, LoRA r16 on q/k/v/o, 1 x 2048; c1 = the
 33M Seraph-native model, 8 x 256.  Synthetic data: uniform token ids, N(0, 0.02) weights,
 norm gains 1, fixed seeds.  Prints ONE JSON line.
+
+--pmc-calibration launches the library's in-place scale kernel three times over 1 GiB before
+the steps (reads 1 GiB, writes 1 GiB per launch): under `rocprofv3 --pmc FETCH_SIZE` /
+`--pmc WRITE_SIZE` its counter readings give the factor that turns the counter into bytes.
+roofline.traffic is read from profiles/train_step_<workload>_hbm_traffic.txt when that file
+holds a line `traffic_bytes_per_launch | <kernel> | N` (taken from such counter runs), else null.
 """
 import argparse
 import json
@@ -84,6 +90,20 @@ def cpu_baseline(w, budget_tokens=192):
                         f"{head:.2f}s + {per_layer:.2f}s per layer scaled to {w['layers']} layers"))
 
 
+def measured_traffic(kernel, workload):
+    """HBM bytes per launch of `kernel` from the committed counter summary, or None."""
+    path = os.path.join(ROOT, "profiles", f"train_step_{workload}_hbm_traffic.txt")
+    try:
+        with open(path) as f:
+            for line in f:
+                part = [x.strip() for x in line.split("|")]
+                if len(part) == 3 and part[0] == "traffic_bytes_per_launch" and part[1] == kernel:
+                    return float(part[2])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -91,6 +111,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
@@ -130,6 +151,14 @@ def main():
                 lo[o:o + oo * r] = 0
                 o += oo * r
         t.upload(tr.LORA_PARAMS, lo)
+
+    if args.pmc_calibration:
+        from seraph_amd import ops
+        cal = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        for _ in range(3):
+            ops.scale_(cal, 1.0)
+        torch.cuda.synchronize()
+        del cal
 
     rng = np.random.default_rng(99)
     starts = np.arange(0, T + 1, w["seq"], dtype=np.int32)
@@ -173,6 +202,8 @@ def main():
         roofline = dict(bound="hbm", kernel=dom["name"], achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
                         frac=round(achieved / PEAK_HBM_GBS, 4), traffic=None, launches=dom["launches"],
                         avg_launch_ms=round(dom["ms"] / dom["launches"], 4), bytes_per_launch=dom["bytes"] / dom["launches"])
+
+    roofline["traffic"] = measured_traffic(dom["name"], args.workload)
 
     out = {
         "metric": "train tok/s (fwd+bwd+AdamW)", "value": round(args.steps * T / elapsed, 2), "unit": "tok/s",
