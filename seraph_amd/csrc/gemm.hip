@@ -21,6 +21,7 @@
 // Accumulator layout of the 32x32x2 instruction: lane l, register v holds
 //   row 8*(v/4) + 4*(l/32) + v%4, column l%32.
 #include "common.hpp"
+#include <type_traits>
 
 namespace seraph {
 
@@ -205,6 +206,234 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_f32_mfma_kernel(const float
         }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Pipelined kernel for the aligned case (K a multiple of 32, 16-byte aligned rows): the same
+// tiling, LDS layout and fragment mapping as above, with everything that is not a matrix
+// instruction, an LDS access or a global load moved out of the K loop.
+//   * Global addresses are a uniform tile pointer (scalar registers, advanced once per stage)
+//     plus a per-lane 32-bit offset fixed before the loop.  Rows past the edge of the operand
+//     are clamped to the last valid row: they feed only output rows/columns that are never
+//     stored, so no per-element predicate is needed.
+//   * A stage is four 8-deep slabs.  The fragments of slab s+1 are read from LDS while the 16
+//     matrix instructions of slab s issue; the next stage's tile is written to the other LDS
+//     buffer after slab 2, and the barrier plus the first fragment read of the next stage sit
+//     in front of slab 3's matrix instructions, which do not depend on them.
+// A wave-uniform pointer moved into scalar registers, so that loads through it take the
+// scalar-base + 32-bit lane offset form and need no per-lane address arithmetic.
+template <typename T>
+__device__ __forceinline__ T* scalar_ptr(T* p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<T*>(((uint64_t)hi << 32) | lo);
+}
+
+template <int TILE, bool KC>
+struct FastLoader {
+    static constexpr int kSlots = TILE * kBK / 4 / kGemmThreads;
+    uint32_t off[kSlots];                                  // byte offsets
+    float4 r[2][kSlots];                                   // two tiles in flight
+
+    // offsets relative to the tile origin (KC: P + mn0*ld + k0, else P + k0*ld + mn0)
+    __device__ __forceinline__ void init(int64_t ld, int64_t mn0, int64_t mn_total) {
+#pragma unroll
+        for (int u = 0; u < kSlots; u++) {
+            const int f = threadIdx.x + kGemmThreads * u;
+            if (KC) {
+                int64_t row = mn0 + f / (kBK / 4);
+                if (row > mn_total - 1) row = mn_total - 1;
+                off[u] = (uint32_t)(4 * ((row - mn0) * ld + 4 * (f % (kBK / 4))));
+            } else {
+                int64_t mn = mn0 + 4 * (f % (TILE / 4));
+                if (mn > mn_total - 4) mn = mn_total - 4;
+                off[u] = (uint32_t)(4 * ((int64_t)(f / (TILE / 4)) * ld + (mn - mn0)));
+            }
+        }
+    }
+    template <int SET>
+    __device__ __forceinline__ void load(const float* __restrict__ tile) {
+        // buffer load: scalar descriptor (base = tile origin) + 32-bit lane offset, no address arithmetic
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(tile), 0, 0x7fffffff, 0x00020000);
+#pragma unroll
+        for (int u = 0; u < kSlots; u++)
+            r[SET][u] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off[u], 0, 0));
+    }
+    template <int SET>
+    __device__ __forceinline__ void store(float* __restrict__ lds) const {
+#pragma unroll
+        for (int u = 0; u < kSlots; u++) {
+            const int f = threadIdx.x + kGemmThreads * u;
+            int o;
+            if (KC) o = (f / (kBK / 4)) * (kBK + kPadK) + 4 * (f % (kBK / 4));
+            else    o = (f / (TILE / 4)) * (TILE + kPadM) + 4 * (f % (TILE / 4));
+            *reinterpret_cast<float4*>(lds + o) = r[SET][u];
+        }
+    }
+};
+
+template <int TM, int TN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_kernel(const float* __restrict__ A,
+                                                                               const float* __restrict__ B,
+                                                                               float* __restrict__ C,
+                                                                               int64_t M, int64_t N, int64_t K,
+                                                                               int accumulate, int nbm, int nbn) {
+    constexpr int BM = 64 * TM, BN = 64 * TN;
+    constexpr int A_FLOATS = lds_floats<BM, A_KC>(), B_FLOATS = lds_floats<BN, B_KC>();
+    __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
+    __shared__ __attribute__((aligned(16))) float lds_b[2][B_FLOATS];
+
+    const int total = nbm * nbn;
+    const int pid = xcd_regroup(blockIdx.x, total);
+    const int width = kGroupM * nbn;
+    const int group = pid / width;
+    const int first_m = group * kGroupM;
+    const int gsize = (nbm - first_m) < kGroupM ? (nbm - first_m) : kGroupM;
+    const int pm = first_m + (pid % width) % gsize;
+    const int pn = (pid % width) / gsize;
+    const int64_t m0 = (int64_t)pm * BM, n0 = (int64_t)pn * BN;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int wm0 = (wave >> 1) * (32 * TM), wn0 = (wave & 1) * (32 * TN);
+    const int64_t lda = A_KC ? K : M, ldb = B_KC ? K : N;
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    FastLoader<BM, A_KC> la;
+    FastLoader<BN, B_KC> lb;
+    la.init(lda, m0, M);
+    lb.init(ldb, n0, N);
+    const float* ta = A_KC ? A + m0 * lda : A + m0;          // tile origin at k = 0 (uniform)
+    const float* tb = B_KC ? B + n0 * ldb : B + n0;
+    const int64_t step_a = A_KC ? kBK : kBK * lda, step_b = B_KC ? kBK : kBK * ldb;
+    const int nk = (int)(K / kBK);
+
+    // per-lane LDS fragment addresses (floats) inside one buffer
+    const int fa_off = A_KC ? (wm0 + r) * (kBK + kPadK) + 4 * h : (4 * h) * (BM + kPadM) + wm0 + r;
+    const int fb_off = B_KC ? (wn0 + r) * (kBK + kPadK) + 4 * h : (4 * h) * (BN + kPadM) + wn0 + r;
+
+    float fa[2][TM][4], fb[2][TN][4];
+    auto read_slab = [&](const float* sa, const float* sb, int slab, int buf) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            if (A_KC) {
+                const float4 t = *reinterpret_cast<const float4*>(sa + fa_off + 32 * i * (kBK + kPadK) + slab * 8);
+                fa[buf][i][0] = t.x; fa[buf][i][1] = t.y; fa[buf][i][2] = t.z; fa[buf][i][3] = t.w;
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; q++) fa[buf][i][q] = sa[fa_off + (slab * 8 + q) * (BM + kPadM) + 32 * i];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            if (B_KC) {
+                const float4 t = *reinterpret_cast<const float4*>(sb + fb_off + 32 * j * (kBK + kPadK) + slab * 8);
+                fb[buf][j][0] = t.x; fb[buf][j][1] = t.y; fb[buf][j][2] = t.z; fb[buf][j][3] = t.w;
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; q++) fb[buf][j][q] = sb[fb_off + (slab * 8 + q) * (BN + kPadM) + 32 * j];
+            }
+        }
+    };
+    auto mfma_slab = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[buf][i][q], fb[buf][j][q], acc[i][j], 0, 0, 0);
+    };
+    constexpr int kMfmaPerSlab = 4 * TM * TN;
+
+    // Tile t travels global -> register set (t & 1) -> LDS buffer (t & 1).  Stage kt issues the
+    // loads of tile kt+2 and, after slab 2, moves tile kt+1 (loaded during stage kt-1) into LDS,
+    // so a load has more than a whole stage of matrix work to complete.  The loop body has no
+    // branches: past the end of K the last tile is simply loaded and staged again (never used),
+    // which keeps the compiler's wait counts exact (a conditional load would force every wait to
+    // assume the load had not been issued).
+    la.template load<0>(ta);
+    lb.template load<0>(tb);
+    if (nk > 1) { ta += step_a; tb += step_b; }
+    la.template load<1>(ta);
+    lb.template load<1>(tb);
+    if (nk > 2) { ta += step_a; tb += step_b; }
+    la.template store<0>(lds_a[0]);
+    lb.template store<0>(lds_b[0]);
+    __syncthreads();
+    read_slab(lds_a[0], lds_b[0], 0, 0);
+
+    auto stage = [&](auto parity, int kt) {
+        constexpr int CUR = decltype(parity)::value;
+        const float* sa = lds_a[CUR];
+        const float* sb = lds_b[CUR];
+        la.template load<CUR>(ta);
+        lb.template load<CUR>(tb);
+        const bool adv = kt + 3 < nk;
+        ta += adv ? step_a : 0;
+        tb += adv ? step_b : 0;
+        __builtin_amdgcn_sched_group_barrier(0x020, 2 * FastLoader<BM, A_KC>::kSlots, 0);     // VMEM reads first
+        read_slab(sa, sb, 1, 1);
+        mfma_slab(0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerSlab, 0);
+        read_slab(sa, sb, 2, 0);
+        mfma_slab(1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerSlab, 0);
+        read_slab(sa, sb, 3, 1);
+        mfma_slab(0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerSlab, 0);
+        la.template store<CUR ^ 1>(lds_a[CUR ^ 1]);
+        lb.template store<CUR ^ 1>(lds_b[CUR ^ 1]);
+        __syncthreads();
+        read_slab(lds_a[CUR ^ 1], lds_b[CUR ^ 1], 0, 0);
+        mfma_slab(1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerSlab, 0);
+    };
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+        stage(std::integral_constant<int, 0>{}, kt);
+        stage(std::integral_constant<int, 1>{}, kt + 1);
+    }
+    if (kt < nk) stage(std::integral_constant<int, 0>{}, kt);
+
+    // ---- epilogue: uniform tile pointer + 32-bit lane offsets; predicates only on edge tiles
+    float* ct = scalar_ptr(C + m0 * N + n0);
+    const bool full = (m0 + BM <= M) && (n0 + BN <= N);
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int col = wn0 + 32 * j + r;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = wm0 + 32 * i + 8 * (v >> 2) + 4 * h + (v & 3);
+                const uint32_t o = 4u * ((uint32_t)row * (uint32_t)N + (uint32_t)col);
+                if (full || (m0 + row < M && n0 + col < N)) {
+                    float* dst = reinterpret_cast<float*>(reinterpret_cast<char*>(ct) + o);
+                    *dst = accumulate ? *dst + acc[i][j][v] : acc[i][j][v];
+                }
+            }
+        }
+}
+
+// The pipelined kernel needs whole K stages, and every per-lane offset inside a tile panel
+// (up to 128 rows of a k-contiguous operand, 32 rows of the other kind, 128 rows of C) in 32 bits.
+static bool pipelined_ok(int64_t M, int64_t N, int64_t K, int tA, int tB) {
+    const int64_t lda = tA ? M : K, ldb = tB ? K : N;
+    const int64_t lim = (int64_t)1 << 31;
+    return K >= kBK && K % kBK == 0 && M >= 4 && N >= 4 && 4 * 129 * lda < lim && 4 * 129 * ldb < lim && 4 * 129 * N < lim;
+}
+
 template <int TM, int TN>
 static int launch_gemm(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
                        int tA, int tB, int accumulate, bool vec, hipStream_t st) {
@@ -213,8 +442,15 @@ static int launch_gemm(const float* A, const float* B, float* C, int64_t M, int6
     const dim3 grid((unsigned)(nbm * nbn)), block(kGemmThreads);
 #define GO(AKC, BKC, V) \
     hipLaunchKernelGGL((gemm_f32_mfma_kernel<TM, TN, AKC, BKC, V>), grid, block, 0, st, A, B, C, M, N, K, accumulate, (int)nbm, (int)nbn)
+#define GOFAST(AKC, BKC) \
+    hipLaunchKernelGGL((gemm_f32_mfma_pipelined_kernel<TM, TN, AKC, BKC>), grid, block, 0, st, A, B, C, M, N, K, accumulate, (int)nbm, (int)nbn)
     // A is k-contiguous unless transposed; B is k-contiguous when transposed.
-    if (vec) {
+    if (vec && pipelined_ok(M, N, K, tA, tB)) {
+        if (!tA && !tB) GOFAST(true, false);
+        else if (!tA && tB) GOFAST(true, true);
+        else if (tA && !tB) GOFAST(false, false);
+        else GOFAST(false, true);
+    } else if (vec) {
         if (!tA && !tB) GO(true, false, true);
         else if (!tA && tB) GO(true, true, true);
         else if (tA && !tB) GO(false, false, true);
@@ -226,6 +462,7 @@ static int launch_gemm(const float* A, const float* B, float* C, int64_t M, int6
         else GO(false, true, false);
     }
 #undef GO
+#undef GOFAST
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }
@@ -240,13 +477,20 @@ static bool use_big_tiles(int64_t M, int64_t N) {
 }
 
 extern "C" const char* seraph_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int transpose_A, int transpose_B) {
-    (void)K;
-    static const char* names[2][4] = {
+    // names for 16-byte aligned operands (the case the training step always has)
+    static const char* generic[2][4] = {
         {"seraph::gemm_f32_mfma_kernel<1, 1, true, false, true>", "seraph::gemm_f32_mfma_kernel<1, 1, true, true, true>",
          "seraph::gemm_f32_mfma_kernel<1, 1, false, false, true>", "seraph::gemm_f32_mfma_kernel<1, 1, false, true, true>"},
         {"seraph::gemm_f32_mfma_kernel<2, 2, true, false, true>", "seraph::gemm_f32_mfma_kernel<2, 2, true, true, true>",
          "seraph::gemm_f32_mfma_kernel<2, 2, false, false, true>", "seraph::gemm_f32_mfma_kernel<2, 2, false, true, true>"}};
-    return names[use_big_tiles(M, N) ? 1 : 0][(transpose_A ? 2 : 0) + (transpose_B ? 1 : 0)];
+    static const char* pipelined[2][4] = {
+        {"seraph::gemm_f32_mfma_pipelined_kernel<1, 1, true, false>", "seraph::gemm_f32_mfma_pipelined_kernel<1, 1, true, true>",
+         "seraph::gemm_f32_mfma_pipelined_kernel<1, 1, false, false>", "seraph::gemm_f32_mfma_pipelined_kernel<1, 1, false, true>"},
+        {"seraph::gemm_f32_mfma_pipelined_kernel<2, 2, true, false>", "seraph::gemm_f32_mfma_pipelined_kernel<2, 2, true, true>",
+         "seraph::gemm_f32_mfma_pipelined_kernel<2, 2, false, false>", "seraph::gemm_f32_mfma_pipelined_kernel<2, 2, false, true>"}};
+    const int64_t lda = transpose_A ? M : K, ldb = transpose_B ? K : N;
+    const bool fast = lda % 4 == 0 && ldb % 4 == 0 && pipelined_ok(M, N, K, transpose_A, transpose_B);
+    return (fast ? pipelined : generic)[use_big_tiles(M, N) ? 1 : 0][(transpose_A ? 2 : 0) + (transpose_B ? 1 : 0)];
 }
 
 extern "C" int seraph_gemm(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
