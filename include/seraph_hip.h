@@ -127,6 +127,21 @@ int seraph_attention_backward(const float* Q, const float* K, const float* V, co
                               int heads, int kv_heads, int head_dim, float scale,
                               void* ws, size_t ws_bytes, seraph_stream_t s);
 
+/* The same backward with a bound on the length of any packed sequence.  When the scratch holds
+ * seraph_attention_backward_ws_bytes_banded(...) bytes, the dK/dV pass leaves dS behind in a band of
+ * 32x32 tiles (heads x ceil(T/32) x (ceil(max_seq_len/32)+1) x 4 KiB) and dQ is one product over it:
+ * 5 matrix products instead of 7.  With the smaller scratch of seraph_attention_backward_ws_bytes the
+ * call is identical to seraph_attention_backward.  max_seq_len <= 0 means T.  A sequence longer than
+ * max_seq_len is a caller error (its far-off-diagonal contributions to dQ would be dropped).
+ * Same reference ops as seraph_attention_backward. */
+size_t seraph_attention_backward_ws_bytes_banded(int64_t T, int heads, int kv_heads, int head_dim, int64_t max_seq_len);
+int seraph_attention_backward_banded(const float* Q, const float* K, const float* V, const float* dO,
+                                     const float* attn_out, const float* lse,
+                                     float* dQ, float* dK, float* dV,
+                                     const uint32_t* seq_starts, int batch, int64_t T,
+                                     int heads, int kv_heads, int head_dim, float scale, int64_t max_seq_len,
+                                     void* ws, size_t ws_bytes, seraph_stream_t s);
+
 /* ---------------------------------------------------------------- norm / position */
 /* vulkan_rmsnorm, include/vulkan_backend.h:499-503 (shaders/rmsnorm.comp) */
 int seraph_rmsnorm(const float* x, const float* scale, float* y, int64_t rows, int64_t cols, float eps,

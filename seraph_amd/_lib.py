@@ -23,8 +23,8 @@ def kernels():
             raise SeraphError(f"{KERNEL_LIB} is not built; run `python -m seraph_amd.build` (needs hipcc)")
         lib = C.CDLL(KERNEL_LIB, mode=C.RTLD_GLOBAL)
         lib.seraph_hip_last_error.restype = C.c_char_p
-        for name in ("seraph_attention_backward_ws_bytes", "seraph_rmsnorm_backward_ws_bytes",
-                     "seraph_embedding_backward_ws_bytes"):
+        for name in ("seraph_attention_backward_ws_bytes", "seraph_attention_backward_ws_bytes_banded",
+                     "seraph_rmsnorm_backward_ws_bytes", "seraph_embedding_backward_ws_bytes"):
             getattr(lib, name).restype = C.c_size_t
         _kernels = lib
     return _kernels

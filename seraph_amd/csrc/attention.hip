@@ -27,6 +27,8 @@
 // search over the batch+1 offsets); a score (i, j) is kept when start[i] <= j <= i.  Tiles are anchored on the global token
 // axis at multiples of 32/128, so ragged sequence lengths need no padding.
 #include <limits.h>
+#include <type_traits>
+#include <algorithm>
 #include <mutex>
 
 #include "common.hpp"
@@ -326,7 +328,8 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
                                                                     float* __restrict__ dK, float* __restrict__ dV,
                                                                     const uint32_t* __restrict__ seq_starts, int batch,
                                                                     int64_t T, int H, int KVH, float scale, float scale_log2e,
-                                                                    unsigned int* __restrict__ queue) {
+                                                                    unsigned int* __restrict__ queue,
+                                                                    float* __restrict__ DS, int ds_slots) {
     constexpr int LD = D + 4, DB = D / 32;
     __shared__ __attribute__((aligned(16))) float sQ[2][32 * LD];
     __shared__ __attribute__((aligned(16))) float sG[2][32 * LD];     // dO
@@ -435,6 +438,16 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
                     const float p = valid ? fast_exp2(s[v] * scale_log2e - lse_p[e]) : 0.0f;
                     s[v] = p;
                     dp[v] = p * (dp[v] - del_p[e]);
+                }
+            }
+            if (DS) {
+                // dS tile (32 queries x 32 keys, row-major) for the dQ pass: band slot = query tile - key tile
+                const int qt = (int)(i0 >> 5), slot = qt - (int)(jw0 >> 5);
+                if (slot < ds_slots) {
+                    const int head = kvh * G + it / nq;
+                    float* tile = DS + ((((int64_t)head * ((T + 31) >> 5) + qt) * ds_slots + slot) << 10);
+#pragma unroll
+                    for (int v = 0; v < 16; v++) tile[acc_row(v, h) * 32 + r] = dp[v];
                 }
             }
 #pragma unroll
@@ -586,8 +599,118 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dq_k
     tq_.leave();
 }
 
+// ---------------------------------------------------------------- backward: dQ from stored dS
+// The dK/dV kernel can leave dS = P (dP - delta) behind, one 32x32 row-major tile per (head,
+// query tile, key tile) in a band of ds_slots key tiles below the diagonal.  dQ = scale dS K is
+// then a single product per tile and the backward executes 5 products instead of 7.
+// grid: persistent over (128-query tiles, heads); wave w owns queries i0+32w .. +31.
+template <int D>
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const float* __restrict__ K, const float* __restrict__ DS,
+                                                                         float* __restrict__ dQ, const uint32_t* __restrict__ seq_starts,
+                                                                         int batch, int64_t T, int H, int KVH, float scale, int ds_slots,
+                                                                         unsigned int* __restrict__ queue) {
+    constexpr int LD = D + 4, DB = D / 32;
+    __shared__ __attribute__((aligned(16))) float sK[2][32 * LD];
+    __shared__ uint32_t sSeq[kMaxSeqLds];
+    __shared__ int sItem;
+    const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
+    const int nqt = (int)((T + 127) / 128);
+    const int64_t nqt32 = (T + 31) >> 5;
+    const TileQueue tq_{queue, &sItem, nqt * H};
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
+    for (int item = tq_.next(); item >= 0; item = tq_.next()) {
+    const int head = item % H, kvh = head / (H / KVH);
+    const int qt128 = nqt - 1 - item / H;
+    const int64_t i0 = (int64_t)qt128 * 128;
+    const int64_t iw0 = i0 + 32 * w;
+    const int64_t qw = (int64_t)H * D, kw = (int64_t)KVH * D;
+    const int64_t i_last = (i0 + 127 < T - 1) ? i0 + 127 : T - 1;
+    const int64_t jbeg = (seqs.start_of((int)i0) / 32) * 32;
+    const int ntiles = (int)((i_last + 1 - jbeg + 31) / 32);
+    // this wave's own range of key tiles (relative to jbeg): from the tile holding the start of its
+    // first query's sequence up to its diagonal tile; empty when the wave lies past the end
+    const bool wave_ok = iw0 < T;
+    const int qt = (int)(iw0 >> 5);
+    int tb = 0, te = -1;
+    if (wave_ok) {
+        tb = (int)(((int64_t)(seqs.start_of((int)iw0) / 32) * 32 - jbeg) / 32);
+        te = (int)((iw0 - jbeg) / 32);
+    }
+    const float* band = DS + ((((int64_t)head * nqt32 + (wave_ok ? qt : 0)) * ds_slots) << 10);   // slot 0 = diagonal tile
+    const int kt0 = (int)(jbeg >> 5);
+
+    v16f dq[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) dq[db][v] = 0.0f;
+
+    float4 dsf[2][4];
+    auto ds_load = [&](int t, int buf) {                       // buf is a literal at every call site
+        // a tile outside the wave's range is replaced by one inside it (loaded, never used)
+        int tc = t < tb ? tb : t;
+        tc = tc > te ? te : tc;
+        const int slot = wave_ok ? qt - (kt0 + tc) : 0;
+        const float* tile = band + ((int64_t)slot << 10) + r * 32 + 4 * h;
+#pragma unroll
+        for (int s8 = 0; s8 < 4; s8++) dsf[buf][s8] = *reinterpret_cast<const float4*>(tile + 8 * s8);
+    };
+
+    Tile32<D> tk;
+    tk.gload(K, jbeg, T, kw, kvh * D);
+    ds_load(0, 0);
+    tk.sstore(sK[0]);
+    __syncthreads();
+
+    auto body = [&](auto parity, int t) {
+        constexpr int CUR = decltype(parity)::value;          // register and LDS buffers by compile-time parity
+        if (t + 1 < ntiles) tk.gload(K, jbeg + 32 * (int64_t)(t + 1), T, kw, kvh * D);
+        ds_load(t + 1 < ntiles ? t + 1 : t, CUR ^ 1);
+        if (t >= tb && t <= te) {
+#pragma unroll
+            for (int s8 = 0; s8 < 4; s8++) {
+                const float e[4] = {dsf[CUR][s8].x, dsf[CUR][s8].y, dsf[CUR][s8].z, dsf[CUR][s8].w};
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const DVec<DB> kk = lds_dvec<DB>(&sK[CUR][(8 * s8 + 4 * h + q) * LD], r);
+#pragma unroll
+                    for (int db = 0; db < DB; db++) dq[db] = mfma(e[q], kk.v[db], dq[db]);
+                }
+            }
+        }
+        if (t + 1 < ntiles) tk.sstore(sK[CUR ^ 1]);
+        __syncthreads();
+    };
+    int t = 0;
+    for (; t + 1 < ntiles; t += 2) {
+        body(std::integral_constant<int, 0>{}, t);
+        body(std::integral_constant<int, 1>{}, t + 1);
+    }
+    if (t < ntiles) body(std::integral_constant<int, 0>{}, t);
+
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const int64_t i = iw0 + acc_row(v, h);
+        if (i < T) {
+            float* pq = dQ + i * qw + head * D + DB * r;
+            if (DB == 4) *reinterpret_cast<float4*>(pq) = make_float4(dq[0][v] * scale, dq[1 % DB][v] * scale, dq[2 % DB][v] * scale, dq[3 % DB][v] * scale);
+            else if (DB == 2) *reinterpret_cast<float2*>(pq) = make_float2(dq[0][v] * scale, dq[1 % DB][v] * scale);
+            else pq[0] = dq[0][v] * scale;
+        }
+    }
+    }   // tile queue
+    tq_.leave();
+}
+
 // ---------------------------------------------------------------- host side
-struct AttnWs { float* lse; float* delta; float* out; };
+struct AttnWs { float* lse; float* delta; float* out; float* ds; };
+
+// Band of dS tiles: for every head and 32-query tile, the key tiles from the diagonal down to the
+// tile that holds the start of the longest sequence allowed.
+static int ds_slot_count(int64_t max_seq_len) { return (int)((max_seq_len + 31) / 32) + 1; }
+static size_t ds_band_bytes(int64_t T, int H, int64_t max_seq_len) {
+    return (size_t)H * (size_t)((T + 31) / 32) * (size_t)ds_slot_count(max_seq_len) * 4096;
+}
 
 static size_t a256(size_t x) { return (x + 255) & ~(size_t)255; }
 
@@ -596,7 +719,7 @@ static size_t attn_ws_layout(int64_t T, int H, int D, char* base, AttnWs* w) {
     auto take = [&](size_t bytes) { char* p = base ? base + o : nullptr; o += a256(bytes); return p; };
     char* c = take((size_t)T * H * 4); char* d = take((size_t)T * H * 4);
     char* e = take((size_t)T * H * D * 4);
-    if (w) { w->lse = (float*)c; w->delta = (float*)d; w->out = (float*)e; }
+    if (w) { w->lse = (float*)c; w->delta = (float*)d; w->out = (float*)e; w->ds = base ? (float*)(base + o) : nullptr; }
     return o;
 }
 
@@ -642,7 +765,7 @@ static int run_forward(const float* Q, const float* K, const float* V, float* O,
 template <int D>
 static int run_backward(const float* Q, const float* K, const float* V, const float* dO, const float* O, const float* lse,
                         float* delta, float* dQ, float* dK, float* dV, const uint32_t* seq_starts, int batch,
-                        int64_t T, int H, int KVH, float scale, hipStream_t st) {
+                        int64_t T, int H, int KVH, float scale, float* ds, int ds_slots, hipStream_t st) {
     hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)ceil_div(T, 4)), dim3(256), 0, st, dO, O, delta, T, H);
     SERAPH_LAUNCH_CHECK();
     unsigned int *qkv = nullptr, *qq = nullptr;
@@ -651,10 +774,15 @@ static int run_backward(const float* Q, const float* K, const float* V, const fl
     if (rc != SERAPH_OK) return rc;
     dim3 gkv(persistent_grid(ceil_div(T, 128) * KVH, D)), gq(persistent_grid(ceil_div(T, 128) * H, D));
     hipLaunchKernelGGL(attn_bwd_dkv_kernel<D>, gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dK, dV, seq_starts, batch,
-                       T, H, KVH, scale, scale * kLog2e, qkv);
+                       T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots);
     SERAPH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(attn_bwd_dq_kernel<D>, gq, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dQ, seq_starts, batch,
-                       T, H, KVH, scale, scale * kLog2e, qq);
+    if (ds) {
+        dim3 gds((unsigned)std::min<int64_t>(ceil_div(T, 128) * H, (int64_t)num_compute_units() * 2));
+        hipLaunchKernelGGL(attn_bwd_dq_ds_kernel<D>, gds, dim3(kAttnThreads), 0, st, K, ds, dQ, seq_starts, batch, T, H, KVH, scale, ds_slots, qq);
+    } else {
+        hipLaunchKernelGGL(attn_bwd_dq_kernel<D>, gq, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dQ, seq_starts, batch,
+                           T, H, KVH, scale, scale * kLog2e, qq);
+    }
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }
@@ -689,12 +817,29 @@ int seraph_attention_forward(const float* Q, const float* K, const float* V, flo
     return rc;
 }
 
+size_t seraph_attention_backward_ws_bytes_banded(int64_t T, int heads, int kv_heads, int head_dim, int64_t max_seq_len) {
+    (void)kv_heads;
+    if (T <= 0 || heads <= 0 || head_dim <= 0) return 0;
+    if (max_seq_len <= 0 || max_seq_len > T) max_seq_len = T;
+    return attn_ws_layout(T, heads, head_dim, nullptr, nullptr) + ds_band_bytes(T, heads, max_seq_len);
+}
+
 int seraph_attention_backward(const float* Q, const float* K, const float* V, const float* dO,
                               const float* attn_out, const float* lse,
                               float* dQ, float* dK, float* dV,
                               const uint32_t* seq_starts, int batch, int64_t T,
                               int heads, int kv_heads, int head_dim, float scale,
                               void* ws, size_t ws_bytes, seraph_stream_t s) {
+    return seraph_attention_backward_banded(Q, K, V, dO, attn_out, lse, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads,
+                                            head_dim, scale, T, ws, ws_bytes, s);
+}
+
+int seraph_attention_backward_banded(const float* Q, const float* K, const float* V, const float* dO,
+                                     const float* attn_out, const float* lse,
+                                     float* dQ, float* dK, float* dV,
+                                     const uint32_t* seq_starts, int batch, int64_t T,
+                                     int heads, int kv_heads, int head_dim, float scale, int64_t max_seq_len,
+                                     void* ws, size_t ws_bytes, seraph_stream_t s) {
     if (T == 0) return SERAPH_OK;
     SERAPH_REQUIRE(Q && K && V && dO && dQ && dK && dV, "attention_backward: NULL pointer");
     int rc = check_attn_shape("attention_backward", T, heads, kv_heads, head_dim);
@@ -709,6 +854,11 @@ int seraph_attention_backward(const float* Q, const float* K, const float* V, co
     }
     AttnWs w;
     attn_ws_layout(T, heads, head_dim, (char*)ws, &w);
+    // the 5-product path needs the dS band behind the fixed part of the scratch
+    if (max_seq_len <= 0 || max_seq_len > T) max_seq_len = T;
+    const bool banded = ws_bytes >= seraph_attention_backward_ws_bytes_banded(T, heads, kv_heads, head_dim, max_seq_len);
+    float* ds = banded ? w.ds : nullptr;
+    const int ds_slots = banded ? ds_slot_count(max_seq_len) : 0;
     hipStream_t st = as_stream(s);
     const float* O = attn_out;
     const float* L = lse;
@@ -722,9 +872,9 @@ int seraph_attention_backward(const float* Q, const float* K, const float* V, co
         O = w.out; L = w.lse;
     }
     switch (head_dim) {
-        case 32: return run_backward<32>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, st);
-        case 64: return run_backward<64>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, st);
-        default: return run_backward<128>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, st);
+        case 32: return run_backward<32>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, st);
+        case 64: return run_backward<64>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, st);
+        default: return run_backward<128>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, st);
     }
 }
 

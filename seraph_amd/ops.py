@@ -104,18 +104,25 @@ def attention_forward(Q, K, V, heads, kv_heads, head_dim, seq_starts=None, scale
 
 
 def attention_backward(Q, K, V, dO, heads, kv_heads, head_dim, seq_starts=None, scale=None, out=None, lse=None,
-                       dK=None, dV=None):
+                       dK=None, dV=None, max_seq_len=None):
+    """max_seq_len: a bound on the longest packed sequence; when given, the scratch is sized for the
+    dS band and the 5-product path runs (seraph_attention_backward_banded)."""
     T = Q.shape[0]
     dQ = torch.empty_like(Q)
     dK = torch.zeros_like(K) if dK is None else dK
     dV = torch.zeros_like(V) if dV is None else dV
     scale = head_dim ** -0.5 if scale is None else scale
-    nbytes = kernels().seraph_attention_backward_ws_bytes(i64(T), C.c_int(heads), C.c_int(kv_heads), C.c_int(head_dim))
+    if max_seq_len is None:
+        nbytes = kernels().seraph_attention_backward_ws_bytes(i64(T), C.c_int(heads), C.c_int(kv_heads), C.c_int(head_dim))
+    else:
+        nbytes = kernels().seraph_attention_backward_ws_bytes_banded(i64(T), C.c_int(heads), C.c_int(kv_heads),
+                                                                     C.c_int(head_dim), i64(max_seq_len))
     ws = _workspace(nbytes)
-    check(kernels().seraph_attention_backward(_p(Q), _p(K), _p(V), _p(dO), _p(out), _p(lse), _p(dQ), _p(dK), _p(dV),
-                                              _p(seq_starts), C.c_int(_batch(seq_starts)), i64(T), C.c_int(heads),
-                                              C.c_int(kv_heads), C.c_int(head_dim), f32(scale), _p(ws), sz(nbytes),
-                                              _stream()), "attention_backward")
+    check(kernels().seraph_attention_backward_banded(_p(Q), _p(K), _p(V), _p(dO), _p(out), _p(lse), _p(dQ), _p(dK), _p(dV),
+                                                     _p(seq_starts), C.c_int(_batch(seq_starts)), i64(T), C.c_int(heads),
+                                                     C.c_int(kv_heads), C.c_int(head_dim), f32(scale),
+                                                     i64(T if max_seq_len is None else max_seq_len), _p(ws), sz(nbytes),
+                                                     _stream()), "attention_backward")
     return dQ, dK, dV
 
 

@@ -70,13 +70,15 @@ void vulkan_batch_attention_backward(vulkan_context_t* ctx, vulkan_buffer_t* Q, 
                                      vulkan_buffer_t* grad_V, int seq_len, int num_heads, int kv_heads, int head_dim) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !Q || !K || !V || !grad_out || !grad_Q || !grad_K || !grad_V) return;
-    size_t need = seraph_attention_backward_ws_bytes(seq_len, num_heads, kv_heads, head_dim);
+    /* one sequence of known length: scratch for the dS band (5 matrix products) unless that is huge */
+    size_t need = seraph_attention_backward_ws_bytes_banded(seq_len, num_heads, kv_heads, head_dim, seq_len);
+    if (need > ((size_t)8 << 30)) need = seraph_attention_backward_ws_bytes(seq_len, num_heads, kv_heads, head_dim);
     void* ws = hip_backend_scratch(ctx, need);
     if (!ws) return;
     float scale = 1.0f / sqrtf((float)head_dim);          /* :1168 */
-    HIP_OP(ctx, "batch_attention_backward", seraph_attention_backward(FPTR(Q), FPTR(K), FPTR(V), FPTR(grad_out), NULL, NULL,
+    HIP_OP(ctx, "batch_attention_backward", seraph_attention_backward_banded(FPTR(Q), FPTR(K), FPTR(V), FPTR(grad_out), NULL, NULL,
                                                                      FPTR(grad_Q), FPTR(grad_K), FPTR(grad_V), NULL, 1, seq_len,
-                                                                     num_heads, kv_heads, head_dim, scale, ws, st->ws_bytes, st->stream));
+                                                                     num_heads, kv_heads, head_dim, scale, seq_len, ws, need, st->stream));
 }
 
 void hip_batch_attention_backward_packed(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulkan_buffer_t* K, vulkan_buffer_t* V,

@@ -53,6 +53,9 @@ struct hip_trainer {
     uint32_t* h_stage;           /* pinned: tokens | targets | starts */
     void* ws;
     size_t ws_bytes;
+    void* attn_ws;               /* attention-backward scratch incl. the dS band; grown to the longest sequence seen */
+    size_t attn_ws_bytes;
+    int64_t max_seq_len;         /* of the current batch */
     size_t device_bytes;
     /* bookkeeping of src/train.c:5439-5463 */
     int accumulation_counter, optimizer_step;
@@ -180,6 +183,8 @@ int64_t hip_lora_param_count(const hip_model_config_t* cfg) {
 }
 
 /* ------------------------------------------------------------------ create / free */
+static const size_t kAttnBandLimit = (size_t)24 << 30;
+
 static size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 static int dev_alloc(hip_trainer_t* t, void** p, size_t bytes) {
@@ -269,8 +274,7 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
         if ((size_t)(p - t->act_arena) > t->act_bytes) { fprintf(stderr, "ERROR: activation arena layout overflow\n"); goto fail; }
     }
     t->ws_bytes = max_sz(seraph_rmsnorm_backward_ws_bytes(max_tokens, cfg->hidden),
-                         max_sz(seraph_attention_backward_ws_bytes(max_tokens, cfg->heads, cfg->kv_heads, cfg->head_dim),
-                                seraph_embedding_backward_ws_bytes(max_tokens, cfg->vocab)));
+                         seraph_embedding_backward_ws_bytes(max_tokens, cfg->vocab));
     if (dev_alloc(t, &t->ws, t->ws_bytes)) goto fail;
     if (seraph_hip_host_alloc((void**)&t->h_stage, ((size_t)2 * max_tokens + max_batch + 1) * 4) != SERAPH_OK) goto fail;
     if (seraph_hip_stream_sync(t->stream) != SERAPH_OK) goto fail;
@@ -291,6 +295,7 @@ void hip_trainer_free(hip_trainer_t* t) {
     seraph_hip_free(t->LP); seraph_hip_free(t->LG); seraph_hip_free(t->LM); seraph_hip_free(t->LV);
     seraph_hip_free(t->act_arena);
     seraph_hip_free(t->ws);
+    seraph_hip_free(t->attn_ws);
     seraph_hip_host_free(t->h_stage);
     for (int i = 0; i < 4; i++) seraph_hip_event_destroy(t->ev[i]);
     if (t->op_ev) {
@@ -377,12 +382,27 @@ static int upload_batch(hip_trainer_t* t, const int* tokens, int T, const int* s
     for (int b = 0; b <= batch; b++) st[b] = seq_starts ? (uint32_t)seq_starts[b] : (b == 0 ? 0u : (uint32_t)T);
     if (st[0] != 0 || st[batch] != (uint32_t)T) { fprintf(stderr, "ERROR: seq_starts must run from 0 to total_tokens\n"); return -1; }
     t->attn_pairs = 0.0;
+    t->max_seq_len = 1;
     for (int b = 0; b < batch; b++) {
+        if (st[b + 1] > st[b] && (int64_t)(st[b + 1] - st[b]) > t->max_seq_len) t->max_seq_len = st[b + 1] - st[b];
         if (st[b + 1] > st[b]) t->attn_pairs += 0.5 * (double)(st[b + 1] - st[b]) * (double)(st[b + 1] - st[b] + 1);
         if (st[b + 1] <= st[b]) { fprintf(stderr, "ERROR: empty or decreasing sequence %d in seq_starts\n", b); return -1; }
         for (uint32_t i = st[b]; i < st[b + 1]; i++) {                     /* src/train_cuda.c:2029-2043 */
             tok[i] = tokens[i] < 0 ? 0u : (uint32_t)tokens[i];
             tgt[i] = (i + 1 < st[b + 1]) ? (tokens[i + 1] < 0 ? 0u : (uint32_t)tokens[i + 1]) : 0u;
+        }
+    }
+    /* attention-backward scratch: the dS band for this batch's longest sequence when it stays under
+     * kAttnBandLimit bytes (5 matrix products), else the fixed part only (7 products) */
+    {
+        const hip_model_config_t* c = &t->cfg;
+        size_t need = seraph_attention_backward_ws_bytes_banded(T, c->heads, c->kv_heads, c->head_dim, t->max_seq_len);
+        if (need > kAttnBandLimit) need = seraph_attention_backward_ws_bytes(T, c->heads, c->kv_heads, c->head_dim);
+        if (need > t->attn_ws_bytes) {
+            CK(seraph_hip_stream_sync(t->stream));
+            if (t->attn_ws) { seraph_hip_free(t->attn_ws); t->device_bytes -= t->attn_ws_bytes; t->attn_ws = NULL; t->attn_ws_bytes = 0; }
+            if (dev_alloc(t, &t->attn_ws, need)) return -1;
+            t->attn_ws_bytes = need;
         }
     }
     CK(seraph_hip_h2d(t->d_tokens, tok, (size_t)T * 4, t->stream));
@@ -507,8 +527,8 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
             lora_backward(t, t->g_hidden, a->attn_out, LW + t->LL.A[3], LW + t->LL.B[3], LGW + t->LL.A[3], LGW + t->LL.B[3], T, qd, h)) return -1.0f;
         OP("fill", 0.0, 4.0 * (double)(T * kv), seraph_fill_u32(t->g_k, 0, (size_t)(T * kv), s));                               /* src/train.c:5221-5222 */
         OP("fill", 0.0, 4.0 * (double)(T * kv), seraph_fill_u32(t->g_v, 0, (size_t)(T * kv), s));
-        OP("attention_backward", 10.0 * D * t->attn_pairs * H, 0.0, seraph_attention_backward(a->q, a->k, a->v, t->g_attn, a->attn_out, a->lse, t->g_q, t->g_k, t->g_v,
-                                     starts, batch, T, H, KVH, D, scale, t->ws, t->ws_bytes, s));
+        OP("attention_backward", 10.0 * D * t->attn_pairs * H, 0.0, seraph_attention_backward_banded(a->q, a->k, a->v, t->g_attn, a->attn_out, a->lse, t->g_q, t->g_k, t->g_v,
+                                     starts, batch, T, H, KVH, D, scale, t->max_seq_len, t->attn_ws, t->attn_ws_bytes, s));
         OP("rope", 0.0, 8.0 * (double)(T * qd), seraph_rope(t->g_q, t->g_q, starts, batch, T, H, D, theta, 1, s));
         OP("rope", 0.0, 8.0 * (double)(T * kv), seraph_rope(t->g_k, t->g_k, starts, batch, T, KVH, D, theta, 1, s));
         if (!lora) {

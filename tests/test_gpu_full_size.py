@@ -166,7 +166,7 @@ def test_attention_backward_b8_h16_s1024_d64(ops, orc):
     Q, K, V, dO = (trandn(Tt, H * D, seed=20 + i, std=sc) for i in range(4))
     starts = torch.arange(0, Tt + 1, S, device="cuda", dtype=torch.int32)
     O, L = ops.attention_forward(Q, K, V, H, H, D, starts)
-    dQ, dK, dV = ops.attention_backward(Q, K, V, dO, H, H, D, starts, out=O, lse=L)
+    dQ, dK, dV = ops.attention_backward(Q, K, V, dO, H, H, D, starts, out=O, lse=L, max_seq_len=S)
     for b in (0, 5):                                     # packed sequences are independent: check two whole ones
         sl = slice(b * S, (b + 1) * S)
         q, k, v, g = (host(t[sl]) for t in (Q, K, V, dO))
@@ -174,8 +174,11 @@ def test_attention_backward_b8_h16_s1024_d64(ops, orc):
         rq, rk, rv = orc.attention_backward(q, k, v, g, H, H, D)
         parity(O[sl], ro, f"attention out seq {b}"); parity(L[sl], rl, f"lse seq {b}")
         parity(dQ[sl], rq, f"dQ seq {b}"); parity(dK[sl], rk, f"dK seq {b}"); parity(dV[sl], rv, f"dV seq {b}")
-    again = ops.attention_backward(Q, K, V, dO, H, H, D, starts, out=O, lse=L)
+    again = ops.attention_backward(Q, K, V, dO, H, H, D, starts, out=O, lse=L, max_seq_len=S)
     assert all(torch.equal(a, b) for a, b in zip((dQ, dK, dV), again))          # no atomics: reruns are bit-identical
+    seven = ops.attention_backward(Q, K, V, dO, H, H, D, starts, out=O, lse=L)  # small scratch: 7-product path
+    parity(seven[0], host(dQ), "dQ, 7-product vs 5-product path", atol=1e-6)
+    assert torch.equal(seven[1], dK) and torch.equal(seven[2], dV)
     rec = ops.attention_backward(Q, K, V, dO, H, H, D, starts)                    # recompute path (no saved O / LSE)
     for a, b, name in zip((dQ, dK, dV), rec, ("dQ", "dK", "dV")):
         parity(a, host(b), f"{name} saved vs recomputed statistics", atol=1e-6)
@@ -190,7 +193,7 @@ def test_attention_backward_16384_tokens_gqa_d128(ops, orc):
     K, V = trandn(T, KVH * D, seed=32, std=sc), trandn(T, KVH * D, seed=33, std=sc)
     starts = torch.tensor(bounds, device="cuda", dtype=torch.int32)
     O, L = ops.attention_forward(Q, K, V, H, KVH, D, starts)
-    dQ, dK, dV = ops.attention_backward(Q, K, V, dO, H, KVH, D, starts, out=O, lse=L)
+    dQ, dK, dV = ops.attention_backward(Q, K, V, dO, H, KVH, D, starts, out=O, lse=L, max_seq_len=4096)
     sl = slice(bounds[-2], T)                            # the short sequence, whole, against the oracle
     q, k, v, g = (host(t[sl]) for t in (Q, K, V, dO))
     ro, _ = orc.attention_forward(q, k, v, H, KVH, D)
@@ -203,9 +206,10 @@ def test_attention_backward_16384_tokens_gqa_d128(ops, orc):
     rq, _, _ = orc.attention_backward(q, k, v, g, H, KVH, D)
     parity(O[p], ro, "prefix out"); parity(dQ[p], rq, "prefix dQ")
     # linearity in dO over the whole batch, and bit-identical reruns
-    d2 = ops.attention_backward(Q, K, V, 2.0 * dO, H, KVH, D, starts, out=O, lse=L)
+    d2 = ops.attention_backward(Q, K, V, 2.0 * dO, H, KVH, D, starts, out=O, lse=L, max_seq_len=4096)
     for a, b, name in zip((dQ, dK, dV), d2, ("dQ", "dK", "dV")):
         assert torch.equal(2.0 * a, b), name               # scaling by 2 is exact in FP32
-    again = ops.attention_backward(Q, K, V, dO, H, KVH, D, starts, out=O, lse=L)
-    assert all(torch.equal(a, b) for a, b in zip((dQ, dK, dV), again))
+    seven = ops.attention_backward(Q, K, V, dO, H, KVH, D, starts, out=O, lse=L)     # small scratch: 7-product path
+    parity(seven[0], host(dQ), "dQ, 7-product vs 5-product path", atol=1e-6)
+    assert torch.equal(seven[1], dK) and torch.equal(seven[2], dV)
     assert bool(torch.isfinite(dQ).all() and torch.isfinite(dK).all() and torch.isfinite(dV).all())

@@ -295,9 +295,13 @@ def test_attention_forward(ops, orc, starts, H, KVH, D):
         parity(o2, ro, "attention out, unpacked call")
 
 
-@pytest.mark.parametrize("starts,H,KVH,D", ATTN_CASES)
+ATTN_CASES_BWD = ATTN_CASES + [([0, 700, 731, 1500], 4, 2, 64), ([0, 513, 1030], 2, 1, 128), ([0, 90, 1000], 2, 2, 32)]
+
+
+@pytest.mark.parametrize("starts,H,KVH,D", ATTN_CASES_BWD)
 @pytest.mark.parametrize("saved", [False, True])
-def test_attention_backward(ops, orc, starts, H, KVH, D, saved):
+@pytest.mark.parametrize("banded", [False, True])
+def test_attention_backward(ops, orc, starts, H, KVH, D, saved, banded):
     Q, K, V, dO = _attn_inputs(2, starts, H, KVH, D)
     su = np.array(starts, np.uint32)
     sd = dev(su.view(np.int32))
@@ -306,8 +310,10 @@ def test_attention_backward(ops, orc, starts, H, KVH, D, saved):
     out = lse = None
     if saved:
         out, lse = ops.attention_forward(dev(Q), dev(K), dev(V), H, KVH, D, sd)
+    # banded: scratch sized for the dS band of the longest sequence -> dQ from stored dS (5 products)
+    msl = int(np.diff(starts).max()) if banded else None
     dQ, dK, dV = ops.attention_backward(dev(Q), dev(K), dev(V), dev(dO), H, KVH, D, sd, out=out, lse=lse,
-                                        dK=dev(base), dV=dev(base))
+                                        dK=dev(base), dV=dev(base), max_seq_len=msl)
     parity(dQ, rdQ, "dQ"); parity(dK, rdK, "dK"); parity(dV, rdV, "dV")
 
 
@@ -317,6 +323,10 @@ def test_attention_backward_is_deterministic(ops):
     a = [host(t) for t in ops.attention_backward(dev(Q), dev(K), dev(V), dev(dO), 4, 2, 64, sd)]
     b = [host(t) for t in ops.attention_backward(dev(Q), dev(K), dev(V), dev(dO), 4, 2, 64, sd)]
     assert all((x == y).all() for x, y in zip(a, b))
+    c = [host(t) for t in ops.attention_backward(dev(Q), dev(K), dev(V), dev(dO), 4, 2, 64, sd, max_seq_len=400)]
+    d = [host(t) for t in ops.attention_backward(dev(Q), dev(K), dev(V), dev(dO), 4, 2, 64, sd, max_seq_len=400)]
+    assert all((x == y).all() for x, y in zip(c, d))
+    assert (a[1] == c[1]).all() and (a[2] == c[2]).all()      # dK, dV come from the same kernel either way
 
 
 def test_attention_rejects_unsupported_head_dim(ops):
