@@ -426,6 +426,107 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_kerne
         }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Small outputs with a long K (weight gradients of narrow layers, the rank-sized LoRA products):
+// too few 64x64 tiles to occupy the chip.  Here a workgroup owns a 32x32 tile of C and its four
+// waves split every 32-deep K stage between them (wave w takes the 8-deep slab w); the four
+// partial accumulators are added in a fixed order through LDS, so the result does not depend on
+// timing.  Same loaders and staging as the pipelined kernel.
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_kernel(const float* __restrict__ A,
+                                                                               const float* __restrict__ B,
+                                                                               float* __restrict__ C,
+                                                                               int64_t M, int64_t N, int64_t K,
+                                                                               int accumulate, int nbm, int nbn) {
+    constexpr int BT = 32;
+    constexpr int A_FLOATS = lds_floats<BT, A_KC>(), B_FLOATS = lds_floats<BT, B_KC>();
+    __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
+    __shared__ __attribute__((aligned(16))) float lds_b[2][B_FLOATS];
+    __shared__ __attribute__((aligned(16))) float red[4][BT * BT];
+    (void)nbm;
+    const int pm = blockIdx.x / nbn, pn = blockIdx.x % nbn;
+    const int64_t m0 = (int64_t)pm * BT, n0 = (int64_t)pn * BT;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int64_t lda = A_KC ? K : M, ldb = B_KC ? K : N;
+
+    v16f acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+
+    FastLoader<BT, A_KC> la;
+    FastLoader<BT, B_KC> lb;
+    la.init(lda, m0, M);
+    lb.init(ldb, n0, N);
+    const float* ta = A_KC ? A + m0 * lda : A + m0;
+    const float* tb = B_KC ? B + n0 * ldb : B + n0;
+    const int64_t step_a = A_KC ? kBK : kBK * lda, step_b = B_KC ? kBK : kBK * ldb;
+    const int nk = (int)(K / kBK);
+    // this wave's slab of a stage: k = 8*wave + 4h + q
+    const int fa_off = A_KC ? r * (kBK + kPadK) + 8 * wave + 4 * h : (8 * wave + 4 * h) * (BT + kPadM) + r;
+    const int fb_off = B_KC ? r * (kBK + kPadK) + 8 * wave + 4 * h : (8 * wave + 4 * h) * (BT + kPadM) + r;
+
+    la.template load<0>(ta);
+    lb.template load<0>(tb);
+    if (nk > 1) { ta += step_a; tb += step_b; }
+    la.template load<1>(ta);
+    lb.template load<1>(tb);
+    if (nk > 2) { ta += step_a; tb += step_b; }
+    la.template store<0>(lds_a[0]);
+    lb.template store<0>(lds_b[0]);
+    __syncthreads();
+
+    auto stage = [&](auto parity, int kt) {
+        constexpr int CUR = decltype(parity)::value;
+        la.template load<CUR>(ta);
+        lb.template load<CUR>(tb);
+        const bool adv = kt + 3 < nk;
+        ta += adv ? step_a : 0;
+        tb += adv ? step_b : 0;
+        float fa[4], fb[4];
+        if (A_KC) {
+            const float4 t = *reinterpret_cast<const float4*>(lds_a[CUR] + fa_off);
+            fa[0] = t.x; fa[1] = t.y; fa[2] = t.z; fa[3] = t.w;
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; q++) fa[q] = lds_a[CUR][fa_off + q * (BT + kPadM)];
+        }
+        if (B_KC) {
+            const float4 t = *reinterpret_cast<const float4*>(lds_b[CUR] + fb_off);
+            fb[0] = t.x; fb[1] = t.y; fb[2] = t.z; fb[3] = t.w;
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; q++) fb[q] = lds_b[CUR][fb_off + q * (BT + kPadM)];
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[q], fb[q], acc, 0, 0, 0);
+        la.template store<CUR ^ 1>(lds_a[CUR ^ 1]);
+        lb.template store<CUR ^ 1>(lds_b[CUR ^ 1]);
+        __syncthreads();
+    };
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+        stage(std::integral_constant<int, 0>{}, kt);
+        stage(std::integral_constant<int, 1>{}, kt + 1);
+    }
+    if (kt < nk) stage(std::integral_constant<int, 0>{}, kt);
+
+    // fixed-order sum of the four partial tiles
+#pragma unroll
+    for (int v = 0; v < 16; v++) red[wave][(8 * (v >> 2) + 4 * h + (v & 3)) * BT + r] = acc[v];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < BT * BT / kGemmThreads; i++) {
+        const int e = threadIdx.x + kGemmThreads * i;
+        const int64_t row = m0 + e / BT, col = n0 + e % BT;
+        if (row < M && col < N) {
+            const float v = ((red[0][e] + red[1][e]) + red[2][e]) + red[3][e];
+            float* dst = C + row * N + col;
+            *dst = accumulate ? *dst + v : v;
+        }
+    }
+}
+
 // The pipelined kernel needs whole K stages, and every per-lane offset inside a tile panel
 // (up to 128 rows of a k-contiguous operand, 32 rows of the other kind, 128 rows of C) in 32 bits.
 static bool pipelined_ok(int64_t M, int64_t N, int64_t K, int tA, int tB) {
@@ -476,6 +577,12 @@ static bool use_big_tiles(int64_t M, int64_t N) {
     return ceil_div(M, 128) * ceil_div(N, 128) >= num_compute_units();
 }
 
+// Fewer 64x64 tiles than compute units and a K long enough to be worth splitting between waves.
+static bool use_splitk(int64_t M, int64_t N, int64_t K, int tA, int tB) {
+    return !use_big_tiles(M, N) && ceil_div(M, 64) * ceil_div(N, 64) < num_compute_units() && K >= 256 &&
+           pipelined_ok(M, N, K, tA, tB);
+}
+
 extern "C" const char* seraph_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int transpose_A, int transpose_B) {
     // names for 16-byte aligned operands (the case the training step always has)
     static const char* generic[2][4] = {
@@ -490,6 +597,9 @@ extern "C" const char* seraph_gemm_kernel_name(int64_t M, int64_t N, int64_t K, 
          "seraph::gemm_f32_mfma_pipelined_kernel<2, 2, false, false>", "seraph::gemm_f32_mfma_pipelined_kernel<2, 2, false, true>"}};
     const int64_t lda = transpose_A ? M : K, ldb = transpose_B ? K : N;
     const bool fast = lda % 4 == 0 && ldb % 4 == 0 && pipelined_ok(M, N, K, transpose_A, transpose_B);
+    static const char* splitk[4] = {"seraph::gemm_f32_mfma_splitk_kernel<true, false>", "seraph::gemm_f32_mfma_splitk_kernel<true, true>",
+                                    "seraph::gemm_f32_mfma_splitk_kernel<false, false>", "seraph::gemm_f32_mfma_splitk_kernel<false, true>"};
+    if (fast && use_splitk(M, N, K, transpose_A, transpose_B)) return splitk[(transpose_A ? 2 : 0) + (transpose_B ? 1 : 0)];
     return (fast ? pipelined : generic)[use_big_tiles(M, N) ? 1 : 0][(transpose_A ? 2 : 0) + (transpose_B ? 1 : 0)];
 }
 
@@ -503,5 +613,18 @@ extern "C" int seraph_gemm(const float* A, const float* B, float* C, int64_t M, 
     hipStream_t st = as_stream(s);
     if (use_big_tiles(M, N))
         return launch_gemm<2, 2>(A, B, C, M, N, K, transpose_A, transpose_B, accumulate, vec, st);
+    if (vec && use_splitk(M, N, K, transpose_A, transpose_B)) {
+        const int64_t nbm = ceil_div(M, 32), nbn = ceil_div(N, 32);
+        const dim3 grid((unsigned)(nbm * nbn)), block(kGemmThreads);
+#define GOSK(AKC, BKC) \
+    hipLaunchKernelGGL((gemm_f32_mfma_splitk_kernel<AKC, BKC>), grid, block, 0, st, A, B, C, M, N, K, accumulate, (int)nbm, (int)nbn)
+        if (!transpose_A && !transpose_B) GOSK(true, false);
+        else if (!transpose_A && transpose_B) GOSK(true, true);
+        else if (transpose_A && !transpose_B) GOSK(false, false);
+        else GOSK(false, true);
+#undef GOSK
+        SERAPH_LAUNCH_CHECK();
+        return SERAPH_OK;
+    }
     return launch_gemm<1, 1>(A, B, C, M, N, K, transpose_A, transpose_B, accumulate, vec, st);
 }

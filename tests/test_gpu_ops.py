@@ -131,7 +131,8 @@ def test_cross_entropy_grad_packed(ops, orc):
 @pytest.mark.parametrize("tA,tB", [(0, 0), (1, 0), (0, 1), (1, 1)])
 @pytest.mark.parametrize("M,N,K", [(256, 384, 512), (67, 35, 129), (300, 16, 260), (16, 520, 300), (130, 140, 16),
                                    (1024, 2048, 96), (1, 1, 1), (260, 132, 64), (2052, 2500, 64), (2051, 2499, 32),
-                                   (4, 4, 32), (2176, 2048, 160)])
+                                   (4, 4, 32), (2176, 2048, 160), (512, 512, 2048), (2048, 16, 2048), (16, 2048, 2048),
+                                   (100, 36, 512), (8, 4, 4096)])
 def test_gemm_forms(ops, orc, tA, tB, M, N, K):
     r = rng(M * 7 + N * 3 + K + 2 * tA + tB)
     A = r.standard_normal((K, M) if tA else (M, K)).astype(np.float32)
