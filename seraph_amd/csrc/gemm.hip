@@ -378,26 +378,60 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_kerne
         const bool adv = kt + 3 < nk;
         ta += adv ? step_a : 0;
         tb += adv ? step_b : 0;
-        __builtin_amdgcn_sched_group_barrier(0x020, 2 * FastLoader<BM, A_KC>::kSlots, 0);     // VMEM reads first
+        // Source order: everything a slab needs is requested before its matrix instructions.  The
+        // group barriers then deal the memory instructions out one at a time between consecutive
+        // matrix instructions (a 32x32x2 takes 64 cycles and lets other instruction types issue
+        // meanwhile), so no burst of loads, LDS writes or the barrier leaves the matrix pipe idle.
+        constexpr int kPairs = kMfmaPerSlab < 8 ? kMfmaPerSlab : 8;
+        constexpr int kRest = kMfmaPerSlab - kPairs;
+        auto deal = [&](auto mask) {                       // kPairs x { 1 MFMA, 1 instruction of `mask` }
+#pragma unroll
+            for (int g = 0; g < kPairs; g++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(decltype(mask)::value, 1, 0);
+            }
+        };
+        constexpr std::integral_constant<int, 0x020> kVmem{};
+        constexpr std::integral_constant<int, 0x100> kDsRead{};
         read_slab(sa, sb, 1, 1);
         mfma_slab(0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerSlab, 0);
+        if (kRest > 0) {
+            deal(kVmem);                                   // global loads of tile kt+2
+#pragma unroll
+            for (int g = 0; g < kRest; g++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);     // fragment reads of slab 1
+            }
+        } else {
+            __builtin_amdgcn_sched_group_barrier(0x020, 2 * FastLoader<BM, A_KC>::kSlots, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerSlab, 0);
+        }
         read_slab(sa, sb, 2, 0);
         mfma_slab(1);
+        deal(kDsRead);
         __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerSlab, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, kRest, 0);
         read_slab(sa, sb, 3, 1);
-        mfma_slab(0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerSlab, 0);
         la.template store<CUR ^ 1>(lds_a[CUR ^ 1]);
         lb.template store<CUR ^ 1>(lds_b[CUR ^ 1]);
+        mfma_slab(0);
+        deal(kDsRead);
+        __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
+        if (kRest > 0) {
+#pragma unroll
+            for (int g = 0; g < kRest; g++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);     // LDS writes of tile kt+1
+            }
+        }
+        __builtin_amdgcn_sched_group_barrier(0x200, 32, 0);
         __syncthreads();
         read_slab(lds_a[CUR ^ 1], lds_b[CUR ^ 1], 0, 0);
         mfma_slab(1);
+        deal(kDsRead);
         __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerSlab, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, kRest, 0);
     };
     int kt = 0;
     for (; kt + 1 < nk; kt += 2) {
