@@ -162,7 +162,7 @@ struct Tile32 {
 // ---------------------------------------------------------------- forward
 // grid (query tiles of 128, heads); wave w owns queries i0+32w .. +31; key/value tiles of 32.
 template <int D>
-__global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_fwd_kernel(const float* __restrict__ Q, const float* __restrict__ K,
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_kernel(const float* __restrict__ Q, const float* __restrict__ K,
                                                                 const float* __restrict__ V, float* __restrict__ O,
                                                                 float* __restrict__ LSE, const uint32_t* __restrict__ seq_starts, int batch,
                                                                 int64_t T, int H, int KVH, float scale_log2e,
@@ -406,11 +406,18 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
     tq.sstore(sQ[0]); tg.sstore(sG[0]); stats_store(0);
     __syncthreads();
 
-    for (int it = 0; it < iters; it++) {
+    // One iteration = one 32-query tile of one query head against the workgroup's 128 keys.  Only the
+    // first query tiles of a head (the diagonal) leave some wave without a visible key, so the loop is
+    // written twice: with the per-wave test for those, and as straight-line code for the rest, where
+    // every wave works.  (A conditional around the accumulating matrix instructions in the main
+    // loop makes the compiler shuttle the 128 dK/dV accumulator registers in and out of the
+    // accumulation register file on every iteration.)
+    const bool wave_has_keys = jw0 < T;
+    auto iteration = [&](int it, auto may_skip) {
         const int cur = it & 1;
         const int64_t i0 = j0 + 32 * (int64_t)(it % nq);
         if (it + 1 < iters) { tiles_load(it + 1); stats_load(it + 1); }
-        if (i0 + 31 >= jw0 && jw0 < T) {                        // some query of the tile can see this wave's keys
+        if (!decltype(may_skip)::value || (i0 + 31 >= jw0 && wave_has_keys)) {   // some query of the tile can see this wave's keys
             v16f s, dp;
 #pragma unroll
             for (int v = 0; v < 16; v++) { s[v] = 0.0f; dp[v] = 0.0f; }
@@ -443,7 +450,7 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
             if (DS) {
                 // dS tile (32 queries x 32 keys, row-major) for the dQ pass: band slot = query tile - key tile
                 const int qt = (int)(i0 >> 5), slot = qt - (int)(jw0 >> 5);
-                if (slot < ds_slots) {
+                if (slot >= 0 && slot < ds_slots) {
                     const int head = kvh * G + it / nq;
                     float* tile = DS + ((((int64_t)head * ((T + 31) >> 5) + qt) * ds_slots + slot) << 10);
 #pragma unroll
@@ -464,6 +471,16 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
         }
         if (it + 1 < iters) { tq.sstore(sQ[cur ^ 1]); tg.sstore(sG[cur ^ 1]); stats_store(cur ^ 1); }
         __syncthreads();
+    };
+    {
+        // waves without keys (ragged end of the token axis) never take the straight-line copy
+        const int ndiag = j0 + 127 < T ? (nq < 4 ? nq : 4) : nq;
+        int it = 0;
+        for (int g = 0; g < G; g++) {
+            int n = 0;
+            for (; n < ndiag; n++, it++) iteration(it, std::true_type{});
+            for (; n < nq; n++, it++) iteration(it, std::false_type{});
+        }
     }
 
 #pragma unroll
@@ -745,8 +762,8 @@ static int acquire_tile_queue(unsigned int** out) {
 }
 
 // Resident workgroups for a persistent launch: as many as fit per CU, never more than there are tiles.
-static unsigned persistent_grid(int64_t items, int D) {
-    int64_t cap = (int64_t)num_compute_units() * (D <= 64 ? 2 : 1);
+static unsigned persistent_grid(int64_t items, int per_cu) {
+    int64_t cap = (int64_t)num_compute_units() * per_cu;
     return (unsigned)(items < cap ? items : cap);
 }
 
@@ -756,7 +773,7 @@ static int run_forward(const float* Q, const float* K, const float* V, float* O,
     unsigned int* queue = nullptr;
     int rc = acquire_tile_queue(&queue);
     if (rc != SERAPH_OK) return rc;
-    dim3 grid(persistent_grid(ceil_div(T, 128) * H, D));
+    dim3 grid(persistent_grid(ceil_div(T, 128) * H, 2));
     hipLaunchKernelGGL(attn_fwd_kernel<D>, grid, dim3(kAttnThreads), 0, st, Q, K, V, O, lse, seq_starts, batch, T, H, KVH, scale * kLog2e, queue);
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
@@ -772,7 +789,7 @@ static int run_backward(const float* Q, const float* K, const float* V, const fl
     int rc = acquire_tile_queue(&qkv);
     if (rc == SERAPH_OK) rc = acquire_tile_queue(&qq);
     if (rc != SERAPH_OK) return rc;
-    dim3 gkv(persistent_grid(ceil_div(T, 128) * KVH, D)), gq(persistent_grid(ceil_div(T, 128) * H, D));
+    dim3 gkv(persistent_grid(ceil_div(T, 128) * KVH, D <= 64 ? 2 : 1)), gq(persistent_grid(ceil_div(T, 128) * H, D <= 64 ? 2 : 1));
     hipLaunchKernelGGL(attn_bwd_dkv_kernel<D>, gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dK, dV, seq_starts, batch,
                        T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots);
     SERAPH_LAUNCH_CHECK();
