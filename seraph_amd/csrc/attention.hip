@@ -140,14 +140,26 @@ struct Tile32 {
     static constexpr int LD = D + 4;
     static constexpr int kSlots = 32 * D / 4 / kAttnThreads;
     float4 r[kSlots];
-    // rows row0..row0+31 of a token-major matrix with `stride` floats per token, columns col0..col0+D-1
+    // rows row0..row0+31 of a token-major matrix with `stride` floats per token, columns col0..col0+D-1.
+    // One buffer descriptor per tile (scalar registers): origin at the tile's first element, extent up to
+    // the end of token T-1, so rows past the end read as zeros without a per-lane predicate, and the
+    // per-lane part of the address is a 32-bit offset that needs no 64-bit arithmetic.
     __device__ __forceinline__ void gload(const float* __restrict__ base, int64_t row0, int64_t T, int64_t stride, int col0) {
+        const float* origin = base + row0 * stride + col0;
+        const int64_t left = T - row0;
+        int64_t bytes = left > 0 ? left * stride * 4 - (int64_t)col0 * 4 : 0;
+        if (bytes > 0xffffffffLL) bytes = 0xffffffffLL;
+        const uint64_t o = reinterpret_cast<uint64_t>(origin);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)o), hi = __builtin_amdgcn_readfirstlane((uint32_t)(o >> 32));
+        const uint32_t nb = __builtin_amdgcn_readfirstlane((uint32_t)bytes);
+        const __amdgpu_buffer_rsrc_t rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(((uint64_t)hi << 32) | lo), 0, (int)nb, 0x00020000);
+        const int st4 = (int)stride * 4;
 #pragma unroll
         for (int u = 0; u < kSlots; u++) {
             const int f = threadIdx.x + kAttnThreads * u;
-            const int row = f / (D / 4), c4 = f % (D / 4);
-            const int64_t t = row0 + row;
-            r[u] = t < T ? *reinterpret_cast<const float4*>(base + t * stride + col0 + 4 * c4) : make_float4(0.f, 0.f, 0.f, 0.f);
+            const int off = (f / (D / 4)) * st4 + 16 * (f % (D / 4));
+            r[u] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0));
         }
     }
     __device__ __forceinline__ void sstore(float* __restrict__ lds) const {
@@ -321,7 +333,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const float* __restrict
 
 // ---------------------------------------------------------------- backward: dK, dV
 // grid (key tiles of 128, kv heads); wave w owns keys j0+32w .. +31 for every query head of the group.
-template <int D>
+template <int D, bool WRITE_DS>
 __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_kernel(const float* __restrict__ Q, const float* __restrict__ K,
                                                                     const float* __restrict__ V, const float* __restrict__ dO,
                                                                     const float* __restrict__ LSE, const float* __restrict__ DELTA,
@@ -383,13 +395,26 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
     Tile32<D> tq, tg;
     float st_lse = 0.f, st_del = 0.f;
     int st_ss = INT_MAX;
+    // Sequence of each lane's query: queries advance by 32 per iteration, so the lane keeps a cursor into
+    // the offsets table and steps it forward (usually not at all) instead of searching every time.
+    const int seq_j0 = seqs.g ? seqs.find((int)(j0 < T ? j0 : T - 1)) : 0;
+    int seq_cur = seq_j0;
     auto stats_load = [&](int it) {
         const int head = kvh * G + it / nq;
         const int64_t i = j0 + 32 * (int64_t)(it % nq) + (threadIdx.x & 31);
         if (threadIdx.x < 32) {
             st_lse = i < T ? LSE[i * H + head] * kLog2e : 0.f;
             st_del = i < T ? DELTA[i * H + head] : 0.f;
-            st_ss = i < T ? seqs.start_of((int)i) : INT_MAX;
+            if (it % nq == 0) seq_cur = seq_j0;
+            st_ss = INT_MAX;
+            if (i < T) {
+                st_ss = 0;
+                if (seqs.g) {
+                    const uint32_t* tab = seqs.s ? seqs.s : seqs.g;
+                    while ((int64_t)tab[seq_cur + 1] <= i) seq_cur++;      // i < T = tab[batch]: terminates
+                    st_ss = (int)tab[seq_cur];
+                }
+            }
         }
     };
     auto stats_store = [&](int buf) {
@@ -416,20 +441,46 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
     auto iteration = [&](int it, auto may_skip) {
         const int cur = it & 1;
         const int64_t i0 = j0 + 32 * (int64_t)(it % nq);
-        if (it + 1 < iters) { tiles_load(it + 1); stats_load(it + 1); }
+        // No branch around the loads and the LDS staging: past the last tile the same tile is simply
+        // fetched and staged again.  (Loads and stores share one in-order counter; behind a branch the
+        // compiler must wait for everything, including the dS stores, before it may touch the tile.)
+        const int nxt = it + 1 < iters ? it + 1 : it;
+        tiles_load(nxt);
+        stats_load(nxt);
         if (!decltype(may_skip)::value || (i0 + 31 >= jw0 && wave_has_keys)) {   // some query of the tile can see this wave's keys
             v16f s, dp;
 #pragma unroll
             for (int v = 0; v < 16; v++) { s[v] = 0.0f; dp[v] = 0.0f; }
+            {
+                // operands of step s8+1 are requested from LDS before the 8 matrix instructions of step s8
+                float4 fa[2], fb[2], fv[2];
+                auto fetch = [&](int s8, int buf) {
+                    fa[buf] = *reinterpret_cast<const float4*>(&sQ[cur][r * LD + s8 * 8 + 4 * h]);
+                    fb[buf] = *reinterpret_cast<const float4*>(&sG[cur][r * LD + s8 * 8 + 4 * h]);
+                    if (kVinLds) fv[buf] = *reinterpret_cast<const float4*>(&sVt[(32 * w + r) * LD + s8 * 8 + 4 * h]);
+                };
+                fetch(0, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
 #pragma unroll
-            for (int s8 = 0; s8 < D / 8; s8++) {
-                const float4 a = *reinterpret_cast<const float4*>(&sQ[cur][r * LD + s8 * 8 + 4 * h]);
-                const float4 b = *reinterpret_cast<const float4*>(&sG[cur][r * LD + s8 * 8 + 4 * h]);
-                const float4 vv = kVinLds ? *reinterpret_cast<const float4*>(&sVt[(32 * w + r) * LD + s8 * 8 + 4 * h]) : vf[kVinLds ? 0 : s8];
-                s = mfma(a.x, kf[s8].x, s); dp = mfma(b.x, vv.x, dp);
-                s = mfma(a.y, kf[s8].y, s); dp = mfma(b.y, vv.y, dp);
-                s = mfma(a.z, kf[s8].z, s); dp = mfma(b.z, vv.z, dp);
-                s = mfma(a.w, kf[s8].w, s); dp = mfma(b.w, vv.w, dp);
+                for (int s8 = 0; s8 < D / 8; s8++) {
+                    if (s8 + 1 < D / 8) fetch(s8 + 1, (s8 + 1) & 1);
+                    const float4 a = fa[s8 & 1], b = fb[s8 & 1];
+                    const float4 vv = kVinLds ? fv[s8 & 1] : vf[kVinLds ? 0 : s8];
+                    s = mfma(a.x, kf[s8].x, s); dp = mfma(b.x, vv.x, dp);
+                    s = mfma(a.y, kf[s8].y, s); dp = mfma(b.y, vv.y, dp);
+                    s = mfma(a.z, kf[s8].z, s); dp = mfma(b.z, vv.z, dp);
+                    s = mfma(a.w, kf[s8].w, s); dp = mfma(b.w, vv.w, dp);
+                    if (s8 + 1 < D / 8) {
+#pragma unroll
+                        for (int g = 0; g < 3; g++) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                        }
+                        __builtin_amdgcn_sched_group_barrier(0x008, 5, 0);
+                    } else {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+                    }
+                }
             }
 #pragma unroll
             for (int g = 0; g < 4; g++) {
@@ -447,29 +498,65 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
                     dp[v] = p * (dp[v] - del_p[e]);
                 }
             }
-            if (DS) {
-                // dS tile (32 queries x 32 keys, row-major) for the dQ pass: band slot = query tile - key tile
+            if (!decltype(may_skip)::value) {
+                // Straight-line copy: stage the next tile now, ahead of the dS stores.  Loads and stores share
+                // one completion counter that the compiler must treat as unordered once both kinds are
+                // pending, so waiting for the tile's loads after the stores were issued would also wait
+                // for the stores.
+                tq.sstore(sQ[cur ^ 1]); tg.sstore(sG[cur ^ 1]); stats_store(cur ^ 1);
+            }
+            if (WRITE_DS) {
+                // dS tile (32 queries x 32 keys, row-major) for the dQ pass: band slot = query tile - key tile.
+                // A tile outside the band (it is all zeros: another sequence) goes to a spare tile behind the band.
                 const int qt = (int)(i0 >> 5), slot = qt - (int)(jw0 >> 5);
-                if (slot >= 0 && slot < ds_slots) {
-                    const int head = kvh * G + it / nq;
-                    float* tile = DS + ((((int64_t)head * ((T + 31) >> 5) + qt) * ds_slots + slot) << 10);
+                const int head = kvh * G + it / nq;
+                const int64_t ntile = (int64_t)H * ((T + 31) >> 5) * ds_slots;
+                int64_t tidx = (((int64_t)head * ((T + 31) >> 5) + qt) * ds_slots + slot);
+                tidx = (slot >= 0 && slot < ds_slots) ? tidx : ntile;
+                const uint64_t ta = reinterpret_cast<uint64_t>(DS + (tidx << 10));
+                const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)ta), hi = __builtin_amdgcn_readfirstlane((uint32_t)(ta >> 32));
+                const __amdgpu_buffer_rsrc_t rs =
+                    __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(((uint64_t)hi << 32) | lo), 0, 4096, 0x00020000);
+                const int lane_off = (4 * h * 32 + r) * 4;
 #pragma unroll
-                    for (int v = 0; v < 16; v++) tile[acc_row(v, h) * 32 + r] = dp[v];
+                for (int v = 0; v < 16; v++) {
+                    const float val = dp[v];
+                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), rs, lane_off + (8 * (v >> 2) + (v & 3)) * 128, 0, 0);
                 }
             }
+            {
+                DVec<DB> go[2], qq[2];
+                auto fetch = [&](int v, int buf) {
+                    go[buf] = lds_dvec<DB>(&sG[cur][acc_row(v, h) * LD], r);
+                    qq[buf] = lds_dvec<DB>(&sQ[cur][acc_row(v, h) * LD], r);
+                };
+                fetch(0, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int il = acc_row(v, h);
-                const DVec<DB> go = lds_dvec<DB>(&sG[cur][il * LD], r);
-                const DVec<DB> qq = lds_dvec<DB>(&sQ[cur][il * LD], r);
+                for (int v = 0; v < 16; v++) {
+                    if (v + 1 < 16) fetch(v + 1, (v + 1) & 1);
 #pragma unroll
-                for (int db = 0; db < DB; db++) {
-                    dv[db] = mfma(s[v], go.v[db], dv[db]);
-                    dk[db] = mfma(dp[v], qq.v[db], dk[db]);
+                    for (int db = 0; db < DB; db++) {
+                        dv[db] = mfma(s[v], go[v & 1].v[db], dv[db]);
+                        dk[db] = mfma(dp[v], qq[v & 1].v[db], dk[db]);
+                    }
+                    if (v + 1 < 16) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                        if (2 * DB - 2 > 0) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);     // one LDS write of the next tile
+                            __builtin_amdgcn_sched_group_barrier(0x008, 2 * DB - 3, 0);
+                        }
+                    } else {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 2 * DB, 0);
+                    }
                 }
             }
         }
-        if (it + 1 < iters) { tq.sstore(sQ[cur ^ 1]); tg.sstore(sG[cur ^ 1]); stats_store(cur ^ 1); }
+        if (decltype(may_skip)::value) { tq.sstore(sQ[cur ^ 1]); tg.sstore(sG[cur ^ 1]); stats_store(cur ^ 1); }
         __syncthreads();
     };
     {
@@ -726,7 +813,7 @@ struct AttnWs { float* lse; float* delta; float* out; float* ds; };
 // tile that holds the start of the longest sequence allowed.
 static int ds_slot_count(int64_t max_seq_len) { return (int)((max_seq_len + 31) / 32) + 1; }
 static size_t ds_band_bytes(int64_t T, int H, int64_t max_seq_len) {
-    return (size_t)H * (size_t)((T + 31) / 32) * (size_t)ds_slot_count(max_seq_len) * 4096;
+    return ((size_t)H * (size_t)((T + 31) / 32) * (size_t)ds_slot_count(max_seq_len) + 1) * 4096;     // + one spare tile
 }
 
 static size_t a256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -790,8 +877,12 @@ static int run_backward(const float* Q, const float* K, const float* V, const fl
     if (rc == SERAPH_OK) rc = acquire_tile_queue(&qq);
     if (rc != SERAPH_OK) return rc;
     dim3 gkv(persistent_grid(ceil_div(T, 128) * KVH, D <= 64 ? 2 : 1)), gq(persistent_grid(ceil_div(T, 128) * H, D <= 64 ? 2 : 1));
-    hipLaunchKernelGGL(attn_bwd_dkv_kernel<D>, gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dK, dV, seq_starts, batch,
-                       T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots);
+    if (ds)
+        hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, true>), gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dK, dV, seq_starts, batch,
+                           T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots);
+    else
+        hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, false>), gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dK, dV, seq_starts, batch,
+                           T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots);
     SERAPH_LAUNCH_CHECK();
     if (ds) {
         dim3 gds((unsigned)std::min<int64_t>(ceil_div(T, 128) * H, (int64_t)num_compute_units() * 2));
