@@ -104,6 +104,45 @@ def measured_traffic(kernel, workload):
     return None
 
 
+def gemm_table(w):
+    """Every GEMM shape of one training step of workload `w`, timed alone through the C ABI and,
+    beside it, torch.matmul (hipBLASLt) on the same operands; prints one line per shape."""
+    import torch
+    from seraph_amd import ops
+    ops.init(0)
+
+    def timeit(fn, iters=5, warm=2):
+        for _ in range(warm):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(iters):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / iters
+
+    T, h, f, V = w["batch"] * w["seq"], w["hidden"], w["ffn"], w["vocab"]
+    qd, kv, L = w["heads"] * w["head_dim"], w["kv_heads"] * w["head_dim"], w["layers"]
+    tot = [0.0, 0.0]
+    for name, o, i, per_step in (("q", qd, h, L), ("k/v", kv, h, 2 * L), ("o", h, qd, L), ("gate/up", f, h, 2 * L),
+                                 ("down", h, f, L), ("lm head", V, h, 1)):
+        for form, M, N, K, tA, tB in ((f"fwd {name} NT", T, o, i, 0, 1), (f"dgrad {name} NN", T, i, o, 0, 0),
+                                      (f"wgrad {name} TN", o, i, T, 1, 0)):
+            A = torch.randn((K, M) if tA else (M, K), device="cuda")
+            B = torch.randn((N, K) if tB else (K, N), device="cuda")
+            C = torch.empty(M, N, device="cuda")
+            ms = timeit(lambda: ops.gemm(A, B, M, N, K, tA, tB, out=C))
+            ref = timeit(lambda: torch.matmul(A.T if tA else A, B.T if tB else B, out=C))
+            tot[0] += per_step * ms
+            tot[1] += per_step * ref
+            print(f"{form:18s} {M:6d} x {N:6d} x {K:6d}: {ms:8.3f} ms {2 * M * N * K / ms / 1e9:6.1f} TFLOP/s | "
+                  f"hipBLASLt {ref:8.3f} ms {2 * M * N * K / ref / 1e9:6.1f} TFLOP/s | x{per_step} per step", flush=True)
+            del A, B, C
+    print(f"GEMM time per step: this library {tot[0]:.1f} ms, hipBLASLt {tot[1]:.1f} ms")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -114,7 +153,12 @@ def main():
     ap.add_argument("--pmc-calibration", action="store_true")
     ap.add_argument("--no-op-timing", action="store_true",
                     help="do not bracket every kernel-library call with an event pair (no roofline / kernels objects)")
+    ap.add_argument("--gemm-table", action="store_true",
+                    help="instead of the benchmark, time every GEMM shape of the workload's step beside hipBLASLt")
     args = ap.parse_args()
+    if args.gemm_table:
+        gemm_table(WORKLOADS[args.workload])
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
                  "(value is the one GPU's throughput)")
