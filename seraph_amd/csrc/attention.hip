@@ -364,22 +364,22 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
     // This wave's 32 keys as B operands (lane = key, k = d).  K always lives in registers; V
     // does too for head_dim <= 64, but at 128 the two fragments plus the dK/dV accumulators
     // exceed the register file, so V for the workgroup's 128 keys is parked in LDS instead.
-    constexpr bool kVinLds = D > 64;
+    constexpr bool kVinLds = D >= 64;
     __shared__ __attribute__((aligned(16))) float sVt[kVinLds ? 128 * LD : 4];
     float4 kf[D / 8], vf[kVinLds ? 1 : D / 8];
 #pragma unroll
     for (int s8 = 0; s8 < D / 8; s8++) {
         kf[s8] = col_ok ? *reinterpret_cast<const float4*>(K + j_lane * kw + kvh * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
+        kf[s8].x *= scale_log2e; kf[s8].y *= scale_log2e; kf[s8].z *= scale_log2e; kf[s8].w *= scale_log2e;   // S comes out in base-2 units
         if (!kVinLds)
             vf[s8] = col_ok ? *reinterpret_cast<const float4*>(V + j_lane * kw + kvh * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     if (kVinLds) {
-        Tile32<D> tvv;
+        Tile32<D> tvv[4];                                   // all four loads in flight before the first LDS write
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            tvv.gload(V, j0 + 32 * q, T, kw, kvh * D);
-            tvv.sstore(sVt + q * 32 * LD);
-        }
+        for (int q = 0; q < 4; q++) tvv[q].gload(V, j0 + 32 * q, T, kw, kvh * D);
+#pragma unroll
+        for (int q = 0; q < 4; q++) tvv[q].sstore(sVt + q * 32 * LD);
     }
     v16f dk[DB], dv[DB];
 #pragma unroll
@@ -482,20 +482,36 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
                     }
                 }
             }
+            // K was scaled by scale*log2(e) when it was loaded, so s is already the base-2 logit.  A tile whose
+            // keys all precede its queries and all lie inside the sequence of its last (hence every) query
+            // needs no mask: p = 2^(s - lse) for every element.
+            const int ss_last = __builtin_amdgcn_readfirstlane(sSS[cur][31]);        // INT_MAX if the tile runs past T
+            const bool interior = (jw0 + 31 <= i0) && ((int)jw0 >= ss_last);
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const float4 lse4 = *reinterpret_cast<const float4*>(&sLse[cur][8 * g + 4 * h]);
                 const float4 del4 = *reinterpret_cast<const float4*>(&sDel[cur][8 * g + 4 * h]);
-                const int4 ss4 = *reinterpret_cast<const int4*>(&sSS[cur][8 * g + 4 * h]);
-                const float* lse_p = &lse4.x; const float* del_p = &del4.x; const int* ss_p = &ss4.x;
+                const float* lse_p = &lse4.x; const float* del_p = &del4.x;
+                if (interior) {
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int v = 4 * g + e;
-                    const int i = (int)i0 + 8 * g + 4 * h + e;
-                    const bool valid = ((int)j_lane <= i) && ((int)j_lane >= ss_p[e]);     // ss = INT_MAX for i >= T
-                    const float p = valid ? fast_exp2(s[v] * scale_log2e - lse_p[e]) : 0.0f;
-                    s[v] = p;
-                    dp[v] = p * (dp[v] - del_p[e]);
+                    for (int e = 0; e < 4; e++) {
+                        const int v = 4 * g + e;
+                        const float p = fast_exp2(s[v] - lse_p[e]);
+                        s[v] = p;
+                        dp[v] = p * (dp[v] - del_p[e]);
+                    }
+                } else {
+                    const int4 ss4 = *reinterpret_cast<const int4*>(&sSS[cur][8 * g + 4 * h]);
+                    const int* ss_p = &ss4.x;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int v = 4 * g + e;
+                        const int i = (int)i0 + 8 * g + 4 * h + e;
+                        const bool valid = ((int)j_lane <= i) && ((int)j_lane >= ss_p[e]);     // ss = INT_MAX for i >= T
+                        const float p = valid ? fast_exp2(s[v] - lse_p[e]) : 0.0f;
+                        s[v] = p;
+                        dp[v] = p * (dp[v] - del_p[e]);
+                    }
                 }
             }
             if (!decltype(may_skip)::value) {
