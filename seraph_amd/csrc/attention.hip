@@ -341,7 +341,8 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
                                                                     const uint32_t* __restrict__ seq_starts, int batch,
                                                                     int64_t T, int H, int KVH, float scale, float scale_log2e,
                                                                     unsigned int* __restrict__ queue,
-                                                                    float* __restrict__ DS, int ds_slots) {
+                                                                    float* __restrict__ DS, int ds_slots,
+                                                                    int split, float* __restrict__ partK, float* __restrict__ partV) {
     constexpr int LD = D + 4, DB = D / 32;
     __shared__ __attribute__((aligned(16))) float sQ[2][32 * LD];
     __shared__ __attribute__((aligned(16))) float sG[2][32 * LD];     // dO
@@ -352,11 +353,16 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
     __shared__ int sItem;
     const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
     const int G = H / KVH;
-    const TileQueue tq_{queue, &sItem, (int)((T + 127) / 128) * KVH};
+    // With few key tiles (short batches) the longest item, the first key tile of a sequence looping over
+    // every query tile of every head of its group, is the critical path.  `split` > 1 deals the
+    // iterations of each (key tile, kv head) round-robin to that many work items; each writes its partial
+    // dK/dV to its own slice of partK/partV and a second kernel adds the slices in a fixed order.
+    const TileQueue tq_{queue, &sItem, (int)((T + 127) / 128) * KVH * split};
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
     for (int item = tq_.next(); item >= 0; item = tq_.next()) {
-    const int kvh = item % KVH;
-    const int64_t j0 = (int64_t)(item / KVH) * 128;            // early keys of a sequence are the long ones
+    const int sub = item % split;
+    const int kvh = (item / split) % KVH;
+    const int64_t j0 = (int64_t)(item / split / KVH) * 128;    // early keys of a sequence are the long ones
     const int64_t jw0 = j0 + 32 * w, j_lane = jw0 + r;
     const bool col_ok = j_lane < T;
     const int64_t qw = (int64_t)H * D, kw = (int64_t)KVH * D;
@@ -398,14 +404,14 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
     // Sequence of each lane's query: queries advance by 32 per iteration, so the lane keeps a cursor into
     // the offsets table and steps it forward (usually not at all) instead of searching every time.
     const int seq_j0 = seqs.g ? seqs.find((int)(j0 < T ? j0 : T - 1)) : 0;
-    int seq_cur = seq_j0;
+    int seq_cur = seq_j0, seq_head = -1;
     auto stats_load = [&](int it) {
         const int head = kvh * G + it / nq;
         const int64_t i = j0 + 32 * (int64_t)(it % nq) + (threadIdx.x & 31);
         if (threadIdx.x < 32) {
             st_lse = i < T ? LSE[i * H + head] * kLog2e : 0.f;
             st_del = i < T ? DELTA[i * H + head] : 0.f;
-            if (it % nq == 0) seq_cur = seq_j0;
+            if (head != seq_head) { seq_cur = seq_j0; seq_head = head; }     // a new head starts over at the key tile
             st_ss = INT_MAX;
             if (i < T) {
                 st_ss = 0;
@@ -427,7 +433,10 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
         tg.gload(dO, i0, T, qw, head * D);
     };
 
-    tiles_load(0); stats_load(0);
+    {
+        const int first = sub < iters ? sub : iters - 1;      // an item without iterations still stages a valid tile
+        tiles_load(first); stats_load(first);
+    }
     tq.sstore(sQ[0]); tg.sstore(sG[0]); stats_store(0);
     __syncthreads();
 
@@ -438,13 +447,13 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
     // loop makes the compiler shuttle the 128 dK/dV accumulator registers in and out of the
     // accumulation register file on every iteration.)
     const bool wave_has_keys = jw0 < T;
-    auto iteration = [&](int it, auto may_skip) {
-        const int cur = it & 1;
+    auto iteration = [&](int it, int li, auto may_skip) {
+        const int cur = li & 1;
         const int64_t i0 = j0 + 32 * (int64_t)(it % nq);
         // No branch around the loads and the LDS staging: past the last tile the same tile is simply
         // fetched and staged again.  (Loads and stores share one in-order counter; behind a branch the
         // compiler must wait for everything, including the dS stores, before it may touch the tile.)
-        const int nxt = it + 1 < iters ? it + 1 : it;
+        const int nxt = it + split < iters ? it + split : it;
         tiles_load(nxt);
         stats_load(nxt);
         if (!decltype(may_skip)::value || (i0 + 31 >= jw0 && wave_has_keys)) {   // some query of the tile can see this wave's keys
@@ -578,38 +587,59 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
     {
         // waves without keys (ragged end of the token axis) never take the straight-line copy
         const int ndiag = j0 + 127 < T ? (nq < 4 ? nq : 4) : nq;
-        int it = 0;
+        int li = 0;
         for (int g = 0; g < G; g++) {
-            int n = 0;
-            for (; n < ndiag; n++, it++) iteration(it, std::true_type{});
-            for (; n < nq; n++, it++) iteration(it, std::false_type{});
+            int n = ((sub - g * nq) % split + split) % split;      // this item's first query tile of head g
+            for (; n < ndiag; n += split, li++) iteration(g * nq + n, li, std::true_type{});
+            for (; n < nq; n += split, li++) iteration(g * nq + n, li, std::false_type{});
         }
     }
+    const bool rmw = split <= 1;                               // else: plain store into this item's slice
+    float* outK = rmw ? dK : partK + (int64_t)sub * T * kw;
+    float* outV = rmw ? dV : partV + (int64_t)sub * T * kw;
 
 #pragma unroll
     for (int v = 0; v < 16; v++) {
         const int64_t j = jw0 + acc_row(v, h);
         if (j < T) {
-            float* pk = dK + j * kw + kvh * D + DB * r;        // lane r owns features DB*r .. DB*r+DB-1
-            float* pv = dV + j * kw + kvh * D + DB * r;
+            float* pk = outK + j * kw + kvh * D + DB * r;      // lane r owns features DB*r .. DB*r+DB-1
+            float* pv = outV + j * kw + kvh * D + DB * r;
             if (DB == 4) {
-                float4 a = *reinterpret_cast<float4*>(pk), b = *reinterpret_cast<float4*>(pv);
+                float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+                if (rmw) { a = *reinterpret_cast<float4*>(pk); b = *reinterpret_cast<float4*>(pv); }
                 a.x += dk[0][v] * scale; a.y += dk[1 % DB][v] * scale; a.z += dk[2 % DB][v] * scale; a.w += dk[3 % DB][v] * scale;
                 b.x += dv[0][v]; b.y += dv[1 % DB][v]; b.z += dv[2 % DB][v]; b.w += dv[3 % DB][v];
                 *reinterpret_cast<float4*>(pk) = a; *reinterpret_cast<float4*>(pv) = b;
             } else if (DB == 2) {
-                float2 a = *reinterpret_cast<float2*>(pk), b = *reinterpret_cast<float2*>(pv);
+                float2 a = make_float2(0.f, 0.f), b = a;
+                if (rmw) { a = *reinterpret_cast<float2*>(pk); b = *reinterpret_cast<float2*>(pv); }
                 a.x += dk[0][v] * scale; a.y += dk[1 % DB][v] * scale;
                 b.x += dv[0][v]; b.y += dv[1 % DB][v];
                 *reinterpret_cast<float2*>(pk) = a; *reinterpret_cast<float2*>(pv) = b;
             } else {
-                pk[0] += dk[0][v] * scale;
-                pv[0] += dv[0][v];
+                pk[0] = (rmw ? pk[0] : 0.f) + dk[0][v] * scale;
+                pv[0] = (rmw ? pv[0] : 0.f) + dv[0][v];
             }
         }
     }
     }   // tile queue
     tq_.leave();
+}
+
+// dK += sum of the split items' slices, in slice order (likewise dV)
+__global__ __launch_bounds__(256) void attn_split_reduce_kernel(float* __restrict__ dK, float* __restrict__ dV,
+                                                                const float* __restrict__ partK, const float* __restrict__ partV,
+                                                                int64_t n4, int split) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+        float4 a = reinterpret_cast<float4*>(dK)[i], b = reinterpret_cast<float4*>(dV)[i];
+        for (int p = 0; p < split; p++) {
+            const float4 x = reinterpret_cast<const float4*>(partK)[p * n4 + i], y = reinterpret_cast<const float4*>(partV)[p * n4 + i];
+            a.x += x.x; a.y += x.y; a.z += x.z; a.w += x.w;
+            b.x += y.x; b.y += y.y; b.z += y.z; b.w += y.w;
+        }
+        reinterpret_cast<float4*>(dK)[i] = a;
+        reinterpret_cast<float4*>(dV)[i] = b;
+    }
 }
 
 // ---------------------------------------------------------------- backward: dQ
@@ -823,7 +853,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const f
 }
 
 // ---------------------------------------------------------------- host side
-struct AttnWs { float* lse; float* delta; float* out; float* ds; };
+struct AttnWs { float* lse; float* delta; float* out; float* partK; float* partV; float* ds; };
+constexpr int kMaxSplit = 4;
 
 // Band of dS tiles: for every head and 32-query tile, the key tiles from the diagonal down to the
 // tile that holds the start of the longest sequence allowed.
@@ -834,12 +865,16 @@ static size_t ds_band_bytes(int64_t T, int H, int64_t max_seq_len) {
 
 static size_t a256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-static size_t attn_ws_layout(int64_t T, int H, int D, char* base, AttnWs* w) {
+static size_t attn_ws_layout(int64_t T, int H, int KVH, int D, char* base, AttnWs* w) {
     size_t o = 0;
     auto take = [&](size_t bytes) { char* p = base ? base + o : nullptr; o += a256(bytes); return p; };
     char* c = take((size_t)T * H * 4); char* d = take((size_t)T * H * 4);
     char* e = take((size_t)T * H * D * 4);
-    if (w) { w->lse = (float*)c; w->delta = (float*)d; w->out = (float*)e; w->ds = base ? (float*)(base + o) : nullptr; }
+    char* pk = take((size_t)kMaxSplit * T * KVH * D * 4); char* pv = take((size_t)kMaxSplit * T * KVH * D * 4);
+    if (w) {
+        w->lse = (float*)c; w->delta = (float*)d; w->out = (float*)e; w->partK = (float*)pk; w->partV = (float*)pv;
+        w->ds = base ? (float*)(base + o) : nullptr;
+    }
     return o;
 }
 
@@ -885,20 +920,31 @@ static int run_forward(const float* Q, const float* K, const float* V, float* O,
 template <int D>
 static int run_backward(const float* Q, const float* K, const float* V, const float* dO, const float* O, const float* lse,
                         float* delta, float* dQ, float* dK, float* dV, const uint32_t* seq_starts, int batch,
-                        int64_t T, int H, int KVH, float scale, float* ds, int ds_slots, hipStream_t st) {
+                        int64_t T, int H, int KVH, float scale, float* ds, int ds_slots, float* partK, float* partV, hipStream_t st) {
     hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)ceil_div(T, 4)), dim3(256), 0, st, dO, O, delta, T, H);
     SERAPH_LAUNCH_CHECK();
     unsigned int *qkv = nullptr, *qq = nullptr;
     int rc = acquire_tile_queue(&qkv);
     if (rc == SERAPH_OK) rc = acquire_tile_queue(&qq);
     if (rc != SERAPH_OK) return rc;
-    dim3 gkv(persistent_grid(ceil_div(T, 128) * KVH, D <= 64 ? 2 : 1)), gq(persistent_grid(ceil_div(T, 128) * H, D <= 64 ? 2 : 1));
+    const int per_cu = D <= 64 ? 2 : 1;
+    const int64_t kv_items = ceil_div(T, 128) * KVH, slots = (int64_t)num_compute_units() * per_cu;
+    // fewer (key tile, kv head) items than resident workgroups: split each between several of them
+    int split = (int)(slots / kv_items);
+    split = split < 1 ? 1 : (split > kMaxSplit ? kMaxSplit : split);
+    dim3 gkv(persistent_grid(kv_items * split, per_cu)), gq(persistent_grid(ceil_div(T, 128) * H, per_cu));
     if (ds)
         hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, true>), gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dK, dV, seq_starts, batch,
-                           T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots);
+                           T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots, split, partK, partV);
     else
         hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, false>), gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dK, dV, seq_starts, batch,
-                           T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots);
+                           T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots, split, partK, partV);
+    if (split > 1) {
+        SERAPH_LAUNCH_CHECK();
+        const int64_t n4 = T * KVH * D / 4;
+        hipLaunchKernelGGL(attn_split_reduce_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(n4, 256), 4096)), dim3(256), 0, st,
+                           dK, dV, partK, partV, n4, split);
+    }
     SERAPH_LAUNCH_CHECK();
     if (ds) {
         dim3 gds((unsigned)std::min<int64_t>(ceil_div(T, 128) * H, (int64_t)num_compute_units() * 2));
@@ -920,7 +966,7 @@ extern "C" {
 size_t seraph_attention_backward_ws_bytes(int64_t T, int heads, int kv_heads, int head_dim) {
     (void)kv_heads;
     if (T <= 0 || heads <= 0 || head_dim <= 0) return 0;
-    return attn_ws_layout(T, heads, head_dim, nullptr, nullptr);
+    return attn_ws_layout(T, heads, kv_heads, head_dim, nullptr, nullptr);
 }
 
 int seraph_attention_forward(const float* Q, const float* K, const float* V, float* out, float* lse,
@@ -945,7 +991,7 @@ size_t seraph_attention_backward_ws_bytes_banded(int64_t T, int heads, int kv_he
     (void)kv_heads;
     if (T <= 0 || heads <= 0 || head_dim <= 0) return 0;
     if (max_seq_len <= 0 || max_seq_len > T) max_seq_len = T;
-    return attn_ws_layout(T, heads, head_dim, nullptr, nullptr) + ds_band_bytes(T, heads, max_seq_len);
+    return attn_ws_layout(T, heads, kv_heads, head_dim, nullptr, nullptr) + ds_band_bytes(T, heads, max_seq_len);
 }
 
 int seraph_attention_backward(const float* Q, const float* K, const float* V, const float* dO,
@@ -977,7 +1023,7 @@ int seraph_attention_backward_banded(const float* Q, const float* K, const float
         return SERAPH_ERR_WORKSPACE;
     }
     AttnWs w;
-    attn_ws_layout(T, heads, head_dim, (char*)ws, &w);
+    attn_ws_layout(T, heads, kv_heads, head_dim, (char*)ws, &w);
     // the 5-product path needs the dS band behind the fixed part of the scratch
     if (max_seq_len <= 0 || max_seq_len > T) max_seq_len = T;
     const bool banded = ws_bytes >= seraph_attention_backward_ws_bytes_banded(T, heads, kv_heads, head_dim, max_seq_len);
@@ -996,9 +1042,9 @@ int seraph_attention_backward_banded(const float* Q, const float* K, const float
         O = w.out; L = w.lse;
     }
     switch (head_dim) {
-        case 32: return run_backward<32>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, st);
-        case 64: return run_backward<64>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, st);
-        default: return run_backward<128>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, st);
+        case 32: return run_backward<32>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, w.partK, w.partV, st);
+        case 64: return run_backward<64>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, w.partK, w.partV, st);
+        default: return run_backward<128>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, w.partK, w.partV, st);
     }
 }
 
