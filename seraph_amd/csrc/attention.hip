@@ -134,6 +134,41 @@ struct TileQueue {
     }
 };
 
+// Longest tiles first.  Within one sequence the tile index already orders the work, but a packed batch
+// repeats the long-to-short ramp once per sequence, and the long tiles of the last sequence would
+// start late and finish alone.  Every workgroup therefore ranks the tiles by their length (number of
+// 32-wide tiles on the other axis) once, in LDS, and maps queue position -> tile through that ranking.
+// All workgroups compute the same permutation.  Very many tiles (more than kMaxOrder) or very few (where
+// the ranking costs more than it saves) keep the natural order of one sequence: ascending for key tiles,
+// descending for query tiles.
+constexpr int kMaxOrder = 1024;
+constexpr int kMinOrder = 32;
+struct TileOrder {
+    const int* order;      // LDS, or NULL = natural order
+    int n;
+    bool descending;
+    __device__ __forceinline__ int operator()(int rank) const { return order ? order[rank] : (descending ? n - 1 - rank : rank); }
+};
+template <typename LenFn>
+__device__ __forceinline__ TileOrder rank_tiles_by_length(int* lens, int* order, int n, bool descending, LenFn len) {
+    TileOrder t{nullptr, n, descending};
+    if (n > kMaxOrder || n < kMinOrder) return t;
+    for (int i = threadIdx.x; i < n; i += (int)blockDim.x) lens[i] = len(i);
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += (int)blockDim.x) {
+        const int me = lens[i];
+        int rank = 0;
+        for (int j = 0; j < n; j++) {
+            const int o = lens[j];
+            rank += (o > me) || (o == me && j < i);
+        }
+        order[rank] = i;
+    }
+    __syncthreads();
+    t.order = order;
+    return t;
+}
+
 // ---------------------------------------------------------------- tile staging (32 rows x D)
 template <int D>
 struct Tile32 {
@@ -187,10 +222,16 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_kernel(const float* 
     const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
     const int nqt = (int)((T + 127) / 128);
     const TileQueue tq_{queue, &sItem, nqt * H};
+    __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
+    // key tiles a 128-query tile runs over: from the start of its first query's sequence to its last query
+    const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, [&](int q) {
+        const int64_t a = (int64_t)q * 128, z = (a + 127 < T - 1) ? a + 127 : T - 1;
+        return (int)((z + 1 - (seqs.start_of((int)a) / 32) * 32 + 31) / 32);
+    });
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
     for (int item = tq_.next(); item >= 0; item = tq_.next()) {
     const int head = item % H, kvh = head / (H / KVH);
-    const int qt = nqt - 1 - item / H;                         // long rows first
+    const int qt = by_len(item / H);                           // long rows first
     const int64_t i0 = (int64_t)qt * 128;
     const int64_t iw0 = i0 + 32 * w, i_lane = iw0 + r;
     const bool row_ok = i_lane < T;
@@ -357,12 +398,19 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
     // every query tile of every head of its group, is the critical path.  `split` > 1 deals the
     // iterations of each (key tile, kv head) round-robin to that many work items; each writes its partial
     // dK/dV to its own slice of partK/partV and a second kernel adds the slices in a fixed order.
-    const TileQueue tq_{queue, &sItem, (int)((T + 127) / 128) * KVH * split};
+    const int nkt = (int)((T + 127) / 128);
+    const TileQueue tq_{queue, &sItem, nkt * KVH * split};
+    __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
+    // query tiles a 128-key tile is visible to: up to the end of its last key's sequence
+    const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nkt, false, [&](int k) {
+        const int64_t a = (int64_t)k * 128, z = (a + 127 < T - 1) ? a + 127 : T - 1;
+        return (int)((seqs.end_of((int)z) - a + 31) / 32);
+    });
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
     for (int item = tq_.next(); item >= 0; item = tq_.next()) {
     const int sub = item % split;
     const int kvh = (item / split) % KVH;
-    const int64_t j0 = (int64_t)(item / split / KVH) * 128;    // early keys of a sequence are the long ones
+    const int64_t j0 = (int64_t)by_len(item / split / KVH) * 128;    // long key tiles (early keys of a sequence) first
     const int64_t jw0 = j0 + 32 * w, j_lane = jw0 + r;
     const bool col_ok = j_lane < T;
     const int64_t qw = (int64_t)H * D, kw = (int64_t)KVH * D;
@@ -659,10 +707,15 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dq_k
     const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
     const int nqt = (int)((T + 127) / 128);
     const TileQueue tq_{queue, &sItem, nqt * H};
+    __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
+    const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, [&](int q) {
+        const int64_t a = (int64_t)q * 128, z = (a + 127 < T - 1) ? a + 127 : T - 1;
+        return (int)((z + 1 - (seqs.start_of((int)a) / 32) * 32 + 31) / 32);
+    });
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
     for (int item = tq_.next(); item >= 0; item = tq_.next()) {
     const int head = item % H, kvh = head / (H / KVH);
-    const int qt = nqt - 1 - item / H;
+    const int qt = by_len(item / H);
     const int64_t i0 = (int64_t)qt * 128;
     const int64_t iw0 = i0 + 32 * w, i_lane = iw0 + r;
     const bool row_ok = i_lane < T;
@@ -767,10 +820,15 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const f
     const int nqt = (int)((T + 127) / 128);
     const int64_t nqt32 = (T + 31) >> 5;
     const TileQueue tq_{queue, &sItem, nqt * H};
+    __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
+    const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, [&](int q) {
+        const int64_t a = (int64_t)q * 128, z = (a + 127 < T - 1) ? a + 127 : T - 1;
+        return (int)((z + 1 - (seqs.start_of((int)a) / 32) * 32 + 31) / 32);
+    });
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
     for (int item = tq_.next(); item >= 0; item = tq_.next()) {
     const int head = item % H, kvh = head / (H / KVH);
-    const int qt128 = nqt - 1 - item / H;
+    const int qt128 = by_len(item / H);
     const int64_t i0 = (int64_t)qt128 * 128;
     const int64_t iw0 = i0 + 32 * w;
     const int64_t qw = (int64_t)H * D, kw = (int64_t)KVH * D;
