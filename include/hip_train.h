@@ -26,6 +26,7 @@
 
 #include <stddef.h>
 #include <stdint.h>
+#include <stdio.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -53,6 +54,23 @@ typedef struct hip_trainer hip_trainer_t;
 int64_t hip_param_count(const hip_model_config_t* cfg);
 int64_t hip_lora_param_count(const hip_model_config_t* cfg);
 
+/* Float offsets of every tensor inside the parameter arena (gradients and moments share them):
+ * tensor X of layer l starts at layer0 + l * layer_stride + X. */
+typedef struct {
+    int64_t embed, final_norm, layer0, layer_stride;
+    int64_t in_norm, q, k, v, o, post_norm, gate, up, down;
+    int64_t count;
+} hip_param_layout_t;
+void hip_param_layout(const hip_model_config_t* cfg, hip_param_layout_t* out);
+
+/* Same for the adapter arena; index 0..6 = q k v o gate up down, offset -1 = adapter not selected.
+ * A is [rank, in_dim], B is [out_dim, rank] (src/lora.c:54-81). */
+typedef struct {
+    int64_t A[7], B[7], in_dim[7], out_dim[7];
+    int64_t layer_stride, count;
+} hip_lora_layout_t;
+void hip_lora_layout(const hip_model_config_t* cfg, hip_lora_layout_t* out);
+
 /* ext_* are optional caller-owned DEVICE arenas of hip_param_count floats (NULL: allocated
  * here).  In LoRA mode (cfg->lora_rank > 0) only ext_params is used: the base model is frozen
  * and the adapter arenas are always owned by the trainer.  Returns NULL on failure with the
@@ -66,7 +84,11 @@ void hip_trainer_free(hip_trainer_t* t);
  * 4 lora params, 5 lora grads, 6 lora m, 7 lora v.  Return 0 on success. */
 int hip_trainer_upload(hip_trainer_t* t, int which, const float* host, int64_t count);
 int hip_trainer_download(hip_trainer_t* t, int which, float* host, int64_t count);
+/* the same for `count` floats starting `offset` floats into the arena (tensor-by-tensor loading) */
+int hip_trainer_upload_at(hip_trainer_t* t, int which, int64_t offset, const float* host, int64_t count);
+int hip_trainer_download_at(hip_trainer_t* t, int which, int64_t offset, float* host, int64_t count);
 void* hip_trainer_device_ptr(hip_trainer_t* t, int which);
+int64_t hip_trainer_arena_count(hip_trainer_t* t, int which);     /* floats in that arena; 0 if the mode has none */
 
 /* One packed step.  tokens_packed[total_tokens]; seq_starts[batch_size + 1] (NULL with
  * batch_size 1 = one sequence).  Negative ids are treated as 0 (src/train.c:4473).
@@ -76,6 +98,34 @@ float hip_train_step_full_batch(hip_trainer_t* t, const int* tokens_packed, int 
                                 const int* seq_starts, int batch_size, int run_optimizer);
 float hip_train_step_lora_batch(hip_trainer_t* t, const int* tokens_packed, int total_tokens,
                                 const int* seq_starts, int batch_size, int run_optimizer);
+
+/* Forward and loss only, as cuda_eval_forward (src/train_cuda.c:2672-2810): no gradient, no
+ * bookkeeping change.  hip_evaluate walks a validation set the way cuda_evaluate does
+ * (src/train_cuda.c:2812-2847): one sequence per sample, truncated to max_seq_len, at most
+ * max_eval_samples evenly spaced samples (0 = all); returns the mean loss (-1 if none), perplexity
+ * in *out_perplexity. */
+float hip_eval_forward_batch(hip_trainer_t* t, const int* tokens_packed, int total_tokens,
+                             const int* seq_starts, int batch_size);
+float hip_evaluate(hip_trainer_t* t, const int* val_tokens, int num_val_tokens, const int* offsets, int num_samples,
+                   int max_seq_len, int max_eval_samples, float* out_perplexity);
+
+/* Resume support: the learning rate and the two counters of src/train.c:5439-5463
+ * (state->optimizer_step, state->accumulation_counter); a negative counter is left unchanged. */
+void  hip_trainer_set_schedule(hip_trainer_t* t, float learning_rate, int optimizer_step, int accumulation_counter);
+int   hip_trainer_accumulation_counter(const hip_trainer_t* t);
+
+/* NaN/Inf flag lattice of the reference's --debug-nan-check (src/train.c:4499-4546): with it on,
+ * a step checks the same buffers at the same points into the same flag indices
+ *   [0..9] global checkpoints, [10 + l] hidden after layer l, [10 + L + 5l + k] attention-backward
+ *   checkpoints of layer l, [10 + 6L + l] grad_hidden after layer l's backward, [10 + 7L + 0..4]
+ *   embedding weight / gradient / m / v before AdamW and weight after it,
+ * holds AdamW back until the flags have been read, skips it when any is set and returns NAN
+ * (src/train.c:5446-5448, :5486-5660).  hip_trainer_nan_flags copies the last step's flags and
+ * returns their count; hip_trainer_nan_report prints the "- buffer: ..." lines. */
+int   hip_trainer_enable_nan_check(hip_trainer_t* t, int on);
+int   hip_trainer_nan_detected(const hip_trainer_t* t);
+int   hip_trainer_nan_flags(const hip_trainer_t* t, uint32_t* out, int max);
+void  hip_trainer_nan_report(const hip_trainer_t* t, FILE* out);
 
 int   hip_trainer_optimizer_step(const hip_trainer_t* t);
 float hip_trainer_last_lr(const hip_trainer_t* t);

@@ -60,6 +60,11 @@ struct hip_trainer {
     /* bookkeeping of src/train.c:5439-5463 */
     int accumulation_counter, optimizer_step;
     float last_lr;
+    /* NaN/Inf flag lattice of src/train.c:4499-4546 (off unless enabled) */
+    int nan_check, nan_detected;
+    uint32_t* d_nan_flags;
+    uint32_t* h_nan_flags;
+    uint32_t nan_flag_count;
     double attn_pairs;           /* sum over sequences of S(S+1)/2 for the current batch */
     void* ev[4];
     float phase_ms[3];
@@ -164,6 +169,31 @@ static void make_layouts(hip_trainer_t* t) {
     }
     t->LL.stride = o;
     t->nlora = o * c->layers;
+}
+
+void hip_param_layout(const hip_model_config_t* cfg, hip_param_layout_t* out) {
+    hip_trainer_t tmp;
+    memset(&tmp, 0, sizeof(tmp));
+    tmp.cfg = *cfg;
+    make_layouts(&tmp);
+    out->embed = tmp.off_embed; out->final_norm = tmp.off_final_norm; out->layer0 = tmp.off_layer0;
+    out->layer_stride = tmp.L.stride;
+    out->in_norm = tmp.L.in_norm; out->q = tmp.L.q; out->k = tmp.L.k; out->v = tmp.L.v; out->o = tmp.L.o;
+    out->post_norm = tmp.L.post_norm; out->gate = tmp.L.gate; out->up = tmp.L.up; out->down = tmp.L.down;
+    out->count = tmp.nparams;
+}
+
+void hip_lora_layout(const hip_model_config_t* cfg, hip_lora_layout_t* out) {
+    hip_trainer_t tmp;
+    memset(&tmp, 0, sizeof(tmp));
+    tmp.cfg = *cfg;
+    make_layouts(&tmp);
+    for (int p = 0; p < 7; p++) {
+        out->A[p] = tmp.LL.A[p]; out->B[p] = tmp.LL.B[p];
+        out->in_dim[p] = tmp.LL.in[p]; out->out_dim[p] = tmp.LL.out[p];
+    }
+    out->layer_stride = tmp.LL.stride;
+    out->count = tmp.nlora;
 }
 
 int64_t hip_param_count(const hip_model_config_t* cfg) {
@@ -296,6 +326,8 @@ void hip_trainer_free(hip_trainer_t* t) {
     seraph_hip_free(t->act_arena);
     seraph_hip_free(t->ws);
     seraph_hip_free(t->attn_ws);
+    seraph_hip_free(t->d_nan_flags);
+    free(t->h_nan_flags);
     seraph_hip_host_free(t->h_stage);
     for (int i = 0; i < 4; i++) seraph_hip_event_destroy(t->ev[i]);
     if (t->op_ev) {
@@ -326,6 +358,36 @@ int hip_trainer_download(hip_trainer_t* t, int which, float* host, int64_t count
     float* d = t ? arena_of(t, which, &n) : NULL;
     if (!d || !host || count != n) return -1;
     return seraph_hip_d2h(host, d, (size_t)n * 4, t->stream) == SERAPH_OK ? 0 : -1;
+}
+
+int hip_trainer_upload_at(hip_trainer_t* t, int which, int64_t offset, const float* host, int64_t count) {
+    int64_t n = 0;
+    float* d = t ? arena_of(t, which, &n) : NULL;
+    if (!d || !host || offset < 0 || count < 0 || offset + count > n) return -1;
+    if (count == 0) return 0;
+    return seraph_hip_h2d(d + offset, host, (size_t)count * 4, t->stream) == SERAPH_OK ? 0 : -1;
+}
+
+int hip_trainer_download_at(hip_trainer_t* t, int which, int64_t offset, float* host, int64_t count) {
+    int64_t n = 0;
+    float* d = t ? arena_of(t, which, &n) : NULL;
+    if (!d || !host || offset < 0 || count < 0 || offset + count > n) return -1;
+    if (count == 0) return 0;
+    return seraph_hip_d2h(host, d + offset, (size_t)count * 4, t->stream) == SERAPH_OK ? 0 : -1;
+}
+
+void hip_trainer_set_schedule(hip_trainer_t* t, float learning_rate, int optimizer_step, int accumulation_counter) {
+    if (!t) return;
+    t->opt.learning_rate = learning_rate;
+    if (optimizer_step >= 0) t->optimizer_step = optimizer_step;
+    if (accumulation_counter >= 0) t->accumulation_counter = accumulation_counter;
+}
+
+int hip_trainer_accumulation_counter(const hip_trainer_t* t) { return t ? t->accumulation_counter : -1; }
+
+int64_t hip_trainer_arena_count(hip_trainer_t* t, int which) {
+    int64_t n = 0;
+    return (t && arena_of(t, which, &n)) ? n : 0;
 }
 
 void* hip_trainer_device_ptr(hip_trainer_t* t, int which) {
@@ -411,8 +473,23 @@ static int upload_batch(hip_trainer_t* t, const int* tokens, int T, const int* s
     return 0;
 }
 
+/* One flag of the lattice: flags[idx] |= 1 when the buffer holds a NaN or Inf. */
+#define NANCHK(ptr, n, idx)                                                                              \
+    do {                                                                                                 \
+        if (t->nan_check)                                                                                \
+            OP("nan_check", 0.0, 4.0 * (double)(n), seraph_nan_check((ptr), (size_t)(n), t->d_nan_flags, (idx), s)); \
+    } while (0)
+
+static int nan_flags_any(hip_trainer_t* t) {
+    if (seraph_hip_d2h(t->h_nan_flags, t->d_nan_flags, (size_t)t->nan_flag_count * 4, t->stream) != SERAPH_OK) return -1;
+    for (uint32_t i = 0; i < t->nan_flag_count; i++) if (t->h_nan_flags[i]) return 1;
+    return 0;
+}
+
+enum { STEP_TRAIN = 0, STEP_EVAL = 1 };
+
 static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, const int* seq_starts, int batch,
-                      int run_optimizer) {
+                      int run_optimizer, int mode) {
     if (!t || !tokens || total_tokens < 2 || batch < 1) return -1.0f;
     if (total_tokens > t->max_tokens || batch > t->max_batch) {
         fprintf(stderr, "ERROR: batch of %d tokens / %d sequences exceeds the trainer's capacity (%d / %d)\n",
@@ -435,7 +512,16 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
     if (upload_batch(t, tokens, total_tokens, seq_starts, batch)) return -1.0f;
     const uint32_t* starts = t->d_starts;
 
-    if (t->accumulation_counter == 0) {                                  /* src/train.c:4399-4400 */
+    /* flag indices, src/train.c:4499-4537 */
+    const uint32_t nan_fwd = 10u, nan_bwd = nan_fwd + (uint32_t)NL, nan_gh = nan_bwd + 5u * (uint32_t)NL,
+                   nan_opt = nan_gh + (uint32_t)NL;
+    if (t->nan_check) {
+        CK(seraph_fill_u32(t->d_nan_flags, 0, t->nan_flag_count, s));
+        t->nan_detected = 0;
+        NANCHK(P + t->off_embed, V * h, nan_opt + 0u);                       /* src/train.c:4548-4554 */
+    }
+
+    if (mode == STEP_TRAIN && t->accumulation_counter == 0) {            /* src/train.c:4399-4400 */
         if (lora) OP("fill", 0.0, 4.0 * (double)t->nlora, seraph_fill_u32(t->LG, 0, (size_t)t->nlora, s));
         else OP("fill", 0.0, 4.0 * (double)t->nparams, seraph_fill_u32(t->G, 0, (size_t)t->nparams, s));
     }
@@ -443,6 +529,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
 
     /* ---------------- forward */
     OP("embed_lookup", 0.0, 8.0 * (double)(T * h), seraph_embed_lookup(t->d_tokens, P + t->off_embed, t->act[0].layer_in, T, h, V, s));
+    NANCHK(t->act[0].layer_in, T * h, 7u);
     for (int l = 0; l < NL; l++) {
         const float* W = P + t->off_layer0 + t->L.stride * l;
         const float* LW = lora ? t->LP + t->LL.stride * l : NULL;
@@ -470,9 +557,13 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         GEMM(a->ffn_h, W + t->L.down, t->tmp_h, T, h, f, 0, 1, 0);
         if (lora && t->LL.A[6] >= 0 && lora_forward_add(t, a->ffn_h, t->tmp_h, LW + t->LL.A[6], LW + t->LL.B[6], T, f, h)) return -1.0f;
         OP("add", 0.0, 12.0 * (double)(T * h), seraph_add(a->post_in, t->tmp_h, next, (size_t)(T * h), s));
+        NANCHK(next, T * h, nan_fwd + (uint32_t)l);
     }
     OP("rmsnorm", 0.0, 8.0 * (double)(T * h), seraph_rmsnorm(t->final_in, P + t->off_final_norm, t->xn_final, T, h, eps, s));
+    NANCHK(t->xn_final, T * h, 2u);
+    NANCHK(t->final_in, T * h, 6u);
     GEMM(t->xn_final, P + t->off_embed, t->logits, T, V, h, 0, 1, 0);      /* tied head, src/train.c:4869-4872 */
+    NANCHK(t->logits, T * V, 1u);
 
     /* ---------------- loss: gradient written over the logits */
     OP("cross_entropy_grad", 0.0, 8.0 * (double)T * (double)V + 8.0 * (double)T, seraph_cross_entropy_grad(t->logits, t->d_targets, t->logits, t->loss_rows, starts, batch, T, V, num_valid, s));
@@ -484,14 +575,24 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         red_out = (red_out == t->red_a) ? t->red_b : t->red_a;
     }
     CK(seraph_hip_event_record(t->ev[1], s));
+    if (mode == STEP_EVAL) {                                               /* src/train_cuda.c:2792-2809 */
+        float eval_sum = 0.0f;
+        CK(seraph_hip_d2h(&eval_sum, red_in, sizeof(float), s));
+        op_fold(t);
+        return eval_sum / (float)num_valid;
+    }
 
     /* ---------------- backward */
     float* glog = t->logits;
+    NANCHK(glog, T * V, 3u);
     GEMM(glog, P + t->off_embed, t->g_hidden, T, h, V, 0, 0, 0);            /* LM head dgrad */
+    NANCHK(t->g_hidden, T * h, 4u);
     if (!lora) GEMM(glog, t->xn_final, t->G + t->off_embed, V, h, T, 1, 0, 1); /* LM head wgrad */
     OP("rmsnorm_backward", 0.0, 12.0 * (double)(T * h), seraph_rmsnorm_backward(t->final_in, P + t->off_final_norm, t->g_hidden, t->g_tmp,
                                lora ? t->scratch_gs : t->G + t->off_final_norm, T, h, eps, t->ws, t->ws_bytes, s));
+    NANCHK(t->g_tmp, T * h, 5u);
     { float* sw = t->g_hidden; t->g_hidden = t->g_tmp; t->g_tmp = sw; }                   /* grad_hidden = grad_tmp (copy, src/train.c:5089) */
+    NANCHK(t->g_hidden, T * h, 0u);
 
     for (int l = NL - 1; l >= 0; l--) {
         const float* W = P + t->off_layer0 + t->L.stride * l;
@@ -523,13 +624,18 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         /* attention */
         if (!lora) GEMM(t->g_hidden, a->attn_out, GW + t->L.o, h, qd, T, 1, 0, 1);
         GEMM(t->g_hidden, W + t->L.o, t->g_attn, T, qd, h, 0, 0, 0);
+        NANCHK(t->g_attn, T * qd, nan_bwd + 5u * (uint32_t)l + 0u);
         if (lora && t->LL.A[3] >= 0 &&
             lora_backward(t, t->g_hidden, a->attn_out, LW + t->LL.A[3], LW + t->LL.B[3], LGW + t->LL.A[3], LGW + t->LL.B[3], T, qd, h)) return -1.0f;
         OP("fill", 0.0, 4.0 * (double)(T * kv), seraph_fill_u32(t->g_k, 0, (size_t)(T * kv), s));                               /* src/train.c:5221-5222 */
         OP("fill", 0.0, 4.0 * (double)(T * kv), seraph_fill_u32(t->g_v, 0, (size_t)(T * kv), s));
         OP("attention_backward", 10.0 * D * t->attn_pairs * H, 0.0, seraph_attention_backward_banded(a->q, a->k, a->v, t->g_attn, a->attn_out, a->lse, t->g_q, t->g_k, t->g_v,
                                      starts, batch, T, H, KVH, D, scale, t->max_seq_len, t->attn_ws, t->attn_ws_bytes, s));
+        NANCHK(t->g_q, T * qd, nan_bwd + 5u * (uint32_t)l + 1u);
+        NANCHK(t->g_k, T * kv, nan_bwd + 5u * (uint32_t)l + 2u);
+        NANCHK(t->g_v, T * kv, nan_bwd + 5u * (uint32_t)l + 3u);
         OP("rope", 0.0, 8.0 * (double)(T * qd), seraph_rope(t->g_q, t->g_q, starts, batch, T, H, D, theta, 1, s));
+        NANCHK(t->g_q, T * qd, nan_bwd + 5u * (uint32_t)l + 4u);
         OP("rope", 0.0, 8.0 * (double)(T * kv), seraph_rope(t->g_k, t->g_k, starts, batch, T, KVH, D, theta, 1, s));
         if (!lora) {
             GEMM(t->g_q, a->xn_attn, GW + t->L.q, qd, h, T, 1, 0, 1);
@@ -548,8 +654,11 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         OP("rmsnorm_backward", 0.0, 12.0 * (double)(T * h), seraph_rmsnorm_backward(a->layer_in, W + t->L.in_norm, t->g_xn, t->g_tmp,
                                    lora ? t->scratch_gs : GW + t->L.in_norm, T, h, eps, t->ws, t->ws_bytes, s));
         OP("add", 0.0, 12.0 * (double)(T * h), seraph_add(t->g_tmp, t->g_hidden, t->g_hidden, (size_t)(T * h), s));
+        NANCHK(t->g_hidden, T * h, nan_gh + (uint32_t)l);
     }
+    NANCHK(t->g_hidden, T * h, 8u);
     if (!lora) OP("embedding_backward", 0.0, 12.0 * (double)(T * h), seraph_embedding_backward(t->d_tokens, t->g_hidden, t->G + t->off_embed, T, h, V, t->ws, t->ws_bytes, s));
+    if (!lora) NANCHK(t->G + t->off_embed, V * h, 9u);
     CK(seraph_hip_event_record(t->ev[2], s));
 
     /* ---------------- optimizer (src/train.c:5439-5463, LoRA :6617-6640) */
@@ -563,14 +672,39 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
             if ((float)t->optimizer_step < warm) lr = t->opt.learning_rate * ((float)t->optimizer_step / warm);
             lr = lr / (float)accum;
             t->last_lr = lr;
+            if (t->nan_check) {
+                /* the optimizer waits for the flags so that a NaN cannot reach the weights
+                 * (src/train.c:5446-5448, :5472-5660); then grad/m/v of the embedding are checked
+                 * before AdamW and the embedding after it (:5662-5720) */
+                int any = nan_flags_any(t);
+                if (any) {
+                    t->nan_detected = 1;
+                    op_fold(t);
+                    return any < 0 ? -1.0f : NAN;
+                }
+                if (!lora) {
+                    NANCHK(t->G + t->off_embed, V * h, nan_opt + 1u);
+                    NANCHK(t->M + t->off_embed, V * h, nan_opt + 2u);
+                    NANCHK(t->V + t->off_embed, V * h, nan_opt + 3u);
+                }
+            }
             if (lora) OP("adamw", 0.0, 28.0 * (double)t->nlora, seraph_adamw(t->LP, t->LG, t->LM, t->LV, (size_t)t->nlora, lr, t->opt.beta1, t->opt.beta2,
                                       t->opt.weight_decay, t->opt.eps, t->optimizer_step, t->opt.clip, s));
             else OP("adamw", 0.0, 28.0 * (double)t->nparams, seraph_adamw(t->P, t->G, t->M, t->V, (size_t)t->nparams, lr, t->opt.beta1, t->opt.beta2,
                                  t->opt.weight_decay, t->opt.eps, t->optimizer_step, t->opt.clip, s));
+            if (t->nan_check && !lora) NANCHK(t->P + t->off_embed, V * h, nan_opt + 4u);
         }
         t->accumulation_counter = 0;
     }
     CK(seraph_hip_event_record(t->ev[3], s));
+    if (t->nan_check) {
+        int any = nan_flags_any(t);
+        if (any) {
+            t->nan_detected = 1;
+            op_fold(t);
+            return any < 0 ? -1.0f : NAN;
+        }
+    }
 
     float loss_sum = 0.0f;
     CK(seraph_hip_d2h(&loss_sum, red_in, sizeof(float), s));               /* waits for the whole step */
@@ -582,11 +716,90 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
 float hip_train_step_full_batch(hip_trainer_t* t, const int* tokens_packed, int total_tokens,
                                 const int* seq_starts, int batch_size, int run_optimizer) {
     if (!t || t->lora) { fprintf(stderr, "ERROR: trainer is not in full-weight mode\n"); return -1.0f; }
-    return run_step(t, tokens_packed, total_tokens, seq_starts, batch_size, run_optimizer);
+    return run_step(t, tokens_packed, total_tokens, seq_starts, batch_size, run_optimizer, STEP_TRAIN);
 }
 
 float hip_train_step_lora_batch(hip_trainer_t* t, const int* tokens_packed, int total_tokens,
                                 const int* seq_starts, int batch_size, int run_optimizer) {
     if (!t || !t->lora) { fprintf(stderr, "ERROR: trainer is not in LoRA mode\n"); return -1.0f; }
-    return run_step(t, tokens_packed, total_tokens, seq_starts, batch_size, run_optimizer);
+    return run_step(t, tokens_packed, total_tokens, seq_starts, batch_size, run_optimizer, STEP_TRAIN);
+}
+
+float hip_eval_forward_batch(hip_trainer_t* t, const int* tokens_packed, int total_tokens,
+                             const int* seq_starts, int batch_size) {
+    if (!t) return -1.0f;
+    return run_step(t, tokens_packed, total_tokens, seq_starts, batch_size, 0, STEP_EVAL);
+}
+
+/* src/train_cuda.c:2812-2847 */
+float hip_evaluate(hip_trainer_t* t, const int* val_tokens, int num_val_tokens, const int* offsets, int num_samples,
+                   int max_seq_len, int max_eval_samples, float* out_perplexity) {
+    if (out_perplexity) *out_perplexity = 0.0f;
+    if (!t || !val_tokens || !offsets || num_samples <= 0) return -1.0f;
+    const int max_eval = max_eval_samples > 0 ? max_eval_samples : num_samples;
+    const int stride = num_samples > max_eval ? num_samples / max_eval : 1;
+    double total = 0.0;
+    int valid = 0;
+    for (int i = 0; i < num_samples; i += stride) {
+        const int start = offsets[i];
+        const int end = (i + 1 < num_samples) ? offsets[i + 1] : num_val_tokens;
+        int len = end - start;
+        if (len > max_seq_len) len = max_seq_len;
+        if (len > t->max_tokens) len = t->max_tokens;
+        if (len < 2) continue;
+        const float loss = hip_eval_forward_batch(t, val_tokens + start, len, NULL, 1);
+        if (loss >= 0.0f && !isnan(loss)) { total += loss; valid++; }
+    }
+    const float avg = valid > 0 ? (float)(total / valid) : -1.0f;
+    if (out_perplexity) *out_perplexity = avg > 0.0f ? expf(avg) : 0.0f;
+    return avg;
+}
+
+int hip_trainer_enable_nan_check(hip_trainer_t* t, int on) {
+    if (!t) return -1;
+    if (on && !t->d_nan_flags) {
+        t->nan_flag_count = 10u + 7u * (uint32_t)t->cfg.layers + 5u;       /* src/train.c:4525-4537 */
+        if (dev_alloc(t, (void**)&t->d_nan_flags, (size_t)t->nan_flag_count * 4)) return -1;
+        t->h_nan_flags = (uint32_t*)calloc(t->nan_flag_count, sizeof(uint32_t));
+        if (!t->h_nan_flags) return -1;
+    }
+    t->nan_check = on ? 1 : 0;
+    return 0;
+}
+
+int hip_trainer_nan_detected(const hip_trainer_t* t) { return t ? t->nan_detected : 0; }
+
+int hip_trainer_nan_flags(const hip_trainer_t* t, uint32_t* out, int max) {
+    if (!t || !t->h_nan_flags) return 0;
+    int n = (int)t->nan_flag_count < max ? (int)t->nan_flag_count : max;
+    if (out) memcpy(out, t->h_nan_flags, (size_t)n * 4);
+    return (int)t->nan_flag_count;
+}
+
+/* names the first poisoned buffers the way src/train.c:5500-5560 does */
+void hip_trainer_nan_report(const hip_trainer_t* t, FILE* out) {
+    if (!t || !t->h_nan_flags || !out) return;
+    static const char* const global_names[10] = {
+        "grad_hidden (after final rmsnorm backward)", "logits", "hidden_norm (input to LM head)", "grad_logits",
+        "grad_hidden (after LM head backward)", "grad_tmp_hidden (final rmsnorm backward output)",
+        "final_input (input to final rmsnorm)", "hidden (after embedding lookup)",
+        "grad_hidden (before embedding_backward)", "g_embed (after embedding_backward)"};
+    const uint32_t* fl = t->h_nan_flags;
+    const int NL = t->cfg.layers;
+    const uint32_t fwd = 10u, bwd = fwd + (uint32_t)NL, gh = bwd + 5u * (uint32_t)NL, opt = gh + (uint32_t)NL;
+    for (int i = 0; i < 10; i++) if (fl[i]) fprintf(out, "  - buffer: %s\n", global_names[i]);
+    for (int l = 0; l < NL; l++) if (fl[fwd + l]) { fprintf(out, "  - buffer: hidden after layer=%d (first)\n", l); break; }
+    if (fl[opt + 0]) fprintf(out, "  - buffer: w_embed (weights already poisoned)\n");
+    for (int l = NL - 1; l >= 0; l--) if (fl[gh + l]) { fprintf(out, "  - buffer: grad_hidden after backward of layer=%d (first)\n", l); break; }
+    static const char* const bwd_names[5] = {"grad_attn (input to attn backward)", "grad_q (pre rope_backward)",
+        "grad_k (post attn backward)", "grad_v (post attn backward)", "grad_q (post rope_backward)"};
+    for (int l = NL - 1; l >= 0; l--) {
+        int hit = 0;
+        for (int k = 0; k < 5 && !hit; k++) if (fl[bwd + 5u * l + k]) { fprintf(out, "  - buffer: %s layer=%d\n", bwd_names[k], l); hit = 1; }
+        if (hit) break;
+    }
+    if (fl[opt + 1]) fprintf(out, "  - buffer: g_embed (pre AdamW)\n");
+    if (fl[opt + 2]) fprintf(out, "  - buffer: m_embed (pre AdamW)\n");
+    if (fl[opt + 3]) fprintf(out, "  - buffer: v_embed (pre AdamW)\n");
+    if (fl[opt + 4]) fprintf(out, "  - buffer: w_embed (post AdamW)\n");
 }

@@ -27,6 +27,16 @@ class OpStat(C.Structure):
                 ("bytes", C.c_double)]
 
 
+class ParamLayout(C.Structure):
+    _fields_ = [(n, C.c_int64) for n in ("embed", "final_norm", "layer0", "layer_stride", "in_norm", "q", "k", "v", "o",
+                                         "post_norm", "gate", "up", "down", "count")]
+
+
+class LoraLayout(C.Structure):
+    _fields_ = [("A", C.c_int64 * 7), ("B", C.c_int64 * 7), ("in_dim", C.c_int64 * 7), ("out_dim", C.c_int64 * 7),
+                ("layer_stride", C.c_int64), ("count", C.c_int64)]
+
+
 PARAMS, GRADS, ADAM_M, ADAM_V, LORA_PARAMS, LORA_GRADS, LORA_M, LORA_V = range(8)
 
 
@@ -66,6 +76,22 @@ def _lib():
         lib.hip_trainer_enable_op_timing.argtypes = [C.c_void_p, C.c_int]
         lib.hip_trainer_reset_op_stats.argtypes = [C.c_void_p]
         lib.hip_trainer_op_stats.argtypes = [C.c_void_p, C.POINTER(OpStat), C.c_int]
+        lib.hip_trainer_upload_at.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_void_p, C.c_int64]
+        lib.hip_trainer_download_at.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_void_p, C.c_int64]
+        lib.hip_trainer_arena_count.restype = C.c_int64
+        lib.hip_trainer_arena_count.argtypes = [C.c_void_p, C.c_int]
+        lib.hip_eval_forward_batch.restype = C.c_float
+        lib.hip_eval_forward_batch.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int]
+        lib.hip_evaluate.restype = C.c_float
+        lib.hip_evaluate.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int,
+                                     C.POINTER(C.c_float)]
+        lib.hip_trainer_set_schedule.argtypes = [C.c_void_p, C.c_float, C.c_int, C.c_int]
+        lib.hip_trainer_accumulation_counter.argtypes = [C.c_void_p]
+        lib.hip_trainer_enable_nan_check.argtypes = [C.c_void_p, C.c_int]
+        lib.hip_trainer_nan_detected.argtypes = [C.c_void_p]
+        lib.hip_trainer_nan_flags.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
+        lib.hip_param_layout.argtypes = [C.POINTER(ModelConfig), C.POINTER(ParamLayout)]
+        lib.hip_lora_layout.argtypes = [C.POINTER(ModelConfig), C.POINTER(LoraLayout)]
         lib._seraph_train_bound = True
     return lib
 
@@ -76,6 +102,18 @@ def param_count(cfg):
 
 def lora_param_count(cfg):
     return int(_lib().hip_lora_param_count(C.byref(cfg)))
+
+
+def param_layout(cfg):
+    out = ParamLayout()
+    _lib().hip_param_layout(C.byref(cfg), C.byref(out))
+    return out
+
+
+def lora_layout(cfg):
+    out = LoraLayout()
+    _lib().hip_lora_layout(C.byref(cfg), C.byref(out))
+    return out
 
 
 class Trainer:
@@ -125,6 +163,47 @@ class Trainer:
         if loss < 0:
             raise SeraphError("training step failed (see stderr)")
         return float(loss)
+
+    def eval_forward(self, tokens, seq_starts=None):
+        """Forward and loss only (cuda_eval_forward of the reference); changes no state."""
+        tokens = np.ascontiguousarray(tokens, np.int32)
+        batch, sp = 1, None
+        if seq_starts is not None:
+            seq_starts = np.ascontiguousarray(seq_starts, np.int32)
+            batch = seq_starts.size - 1
+            sp = seq_starts.ctypes.data_as(C.c_void_p)
+        return float(_lib().hip_eval_forward_batch(self._h, tokens.ctypes.data_as(C.c_void_p), tokens.size, sp, batch))
+
+    def evaluate(self, val_tokens, offsets, max_seq_len, max_eval_samples=0):
+        """(mean loss, perplexity) over a validation set, sample by sample (cuda_evaluate of the reference)."""
+        val_tokens = np.ascontiguousarray(val_tokens, np.int32)
+        offsets = np.ascontiguousarray(offsets, np.int32)
+        ppl = C.c_float(0.0)
+        loss = _lib().hip_evaluate(self._h, val_tokens.ctypes.data_as(C.c_void_p), val_tokens.size,
+                                   offsets.ctypes.data_as(C.c_void_p), offsets.size - 1, max_seq_len, max_eval_samples,
+                                   C.byref(ppl))
+        return float(loss), float(ppl.value)
+
+    def set_schedule(self, learning_rate, optimizer_step=-1, accumulation_counter=-1):
+        _lib().hip_trainer_set_schedule(self._h, learning_rate, optimizer_step, accumulation_counter)
+
+    @property
+    def accumulation_counter(self):
+        return int(_lib().hip_trainer_accumulation_counter(self._h))
+
+    def enable_nan_check(self, on=True):
+        if _lib().hip_trainer_enable_nan_check(self._h, 1 if on else 0) != 0:
+            raise SeraphError("could not allocate the NaN flags")
+
+    @property
+    def nan_detected(self):
+        return bool(_lib().hip_trainer_nan_detected(self._h))
+
+    def nan_flags(self):
+        n = _lib().hip_trainer_nan_flags(self._h, None, 0)
+        out = np.zeros(n, np.uint32)
+        _lib().hip_trainer_nan_flags(self._h, out.ctypes.data_as(C.c_void_p), n)
+        return out
 
     @property
     def optimizer_step(self):
