@@ -1,8 +1,9 @@
 """Builds the native libraries in-tree.
 
   seraph_amd/lib/libseraph_hip.so          HIP kernels + C ABI (hipcc, gfx950 only)
-  seraph_amd/lib/libseraph_hip_backend.so  host C: vulkan_* compatible backend and the
-                                           packed training-step drivers (gcc, no HIP headers)
+  seraph_amd/lib/libseraph_hip_backend.so  host C: vulkan_* compatible backend, the packed
+                                           training-step drivers and the file formats (gcc, no HIP headers)
+  seraph_amd/bin/seraph-train-hip          the batched training front end (gcc)
 
 Run as `python -m seraph_amd.build` (add --force to rebuild everything).
 """
@@ -27,7 +28,10 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I", INCLUD
 CC = os.environ.get("CC", "gcc")
 C_FLAGS = ["-O2", "-std=gnu11", "-fPIC", "-Wall", "-Wextra", "-I", INCLUDE, "-I", SRC]
 
+CLI = os.path.join(HERE, "cli")
+BIN = os.path.join(HERE, "bin")
 KERNEL_LIB = os.path.join(LIB, "libseraph_hip.so")
+TRAIN_BIN = os.path.join(BIN, "seraph-train-hip")
 BACKEND_LIB = os.path.join(LIB, "libseraph_hip_backend.so")
 
 
@@ -80,10 +84,23 @@ def build_backend(force=False):
     return BACKEND_LIB
 
 
+def build_cli(force=False):
+    src = os.path.join(CLI, "seraph_train_hip.c")
+    if not os.path.exists(src):
+        return None
+    os.makedirs(BIN, exist_ok=True)
+    deps = [src, BACKEND_LIB] + [os.path.join(INCLUDE, f) for f in os.listdir(INCLUDE)]
+    if force or _newer(TRAIN_BIN, deps):
+        _run([CC] + [f for f in C_FLAGS if f != "-fPIC"] + ["-o", TRAIN_BIN, src, "-L", LIB, "-lseraph_hip_backend",
+             "-lseraph_hip", "-Wl,-rpath,$ORIGIN/../lib", "-lm"])
+    return TRAIN_BIN
+
+
 def build_all(force=False):
     k = build_kernels(force)
     b = build_backend(force)
-    return k, b
+    c = build_cli(force)
+    return k, b, c
 
 
 if __name__ == "__main__":

@@ -38,7 +38,8 @@ def test_kernel_library_exports_its_header(libs):
 
 def test_backend_exports_the_reference_api_and_additions(libs):
     _, b = libs
-    names = declared("hip_backend.h") + declared("hip_train.h")
+    names = declared("hip_backend.h") + declared("hip_train.h") + declared("hip_train_io.h")
+    assert "hip_ttok_load" in names and "hip_eval_forward_batch" in names and "hip_trainer_nan_flags" in names
     missing = [n for n in names if not hasattr(b, n)]
     assert not missing, missing
     # the 40 symbols an unmodified train.o leaves undefined (nm -u on the reference object)

@@ -1,0 +1,268 @@
+"""The batched front end (seraph_amd/bin/seraph-train-hip) and the trainer features around the
+step - evaluation, NaN flag lattice, checkpoints and exact resume - against the CPU oracle.
+
+The front end is run as a user would run it: a model directory (config.json + BF16
+safetensors), a .ttok file, the reference's options.  Its printed losses are compared with the
+oracle stepping the same packed batches from the same BF16-rounded weights (printed with four
+decimals: tolerance 1.5e-4), its exact-resume file with the oracle's weights and moments at
+|got - ref| <= 1e-5 + 1e-4 |ref|, its BF16 checkpoint with the truncated oracle weights to one
+BF16 ulp."""
+import json
+import os
+import re
+import struct
+import subprocess
+
+import numpy as np
+import pytest
+import torch
+
+from tests.test_gpu_step import ATOL, RTOL, check_tensors, init_params, tensor_slices
+from tests.test_io_formats import named_tensors, reference_pack, write_ttok
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "seraph_amd", "bin", "seraph-train-hip")
+SHAPE = dict(hidden=64, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=96, vocab=160)
+
+
+@pytest.fixture(scope="module")
+def tr():
+    from seraph_amd import trainer
+    return trainer
+
+
+def make_model_dir(path, orc, shape, seed):
+    from safetensors.torch import save_file
+    from seraph_amd.trainer import model_config
+    os.makedirs(path, exist_ok=True)
+    ocfg = orc.make_config(**shape, rms_eps=1e-5, rope_theta=10000.0)
+    cfg = model_config(**shape, rms_eps=1e-5, rope_theta=10000.0)
+    p = init_params(orc, ocfg, seed)
+    p = torch.from_numpy(p).to(torch.bfloat16).to(torch.float32).numpy()             # what a BF16 file can hold
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in named_tensors(cfg, p).items()},
+              os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump({"model_type": "qwen2", "vocab_size": shape["vocab"], "hidden_size": shape["hidden"],
+                   "num_hidden_layers": shape["layers"], "intermediate_size": shape["ffn"],
+                   "num_attention_heads": shape["heads"], "num_key_value_heads": shape["kv_heads"],
+                   "head_dim": shape["head_dim"], "rms_norm_eps": 1e-6, "rope_theta": 10000.0}, f)
+    return ocfg, cfg, p
+
+
+def make_samples(seed, n, vocab, lo=1, hi=30):
+    r = np.random.default_rng(seed)
+    return [r.integers(0, vocab, size=int(r.integers(lo, hi + 1))).astype(np.int32) for _ in range(n)]
+
+
+def run_cli(args, timeout=170):
+    print("seraph-train-hip", " ".join(map(str, args)), flush=True)
+    p = subprocess.run([BIN] + [str(a) for a in args], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=timeout)
+    return p.returncode, p.stdout, p.stderr
+
+
+def step_losses(stdout):
+    return [(int(m.group(1)), float(m.group(2))) for m in re.finditer(r"Step (\d+)/\d+ \| Loss: ([0-9.]+|nan|-nan)", stdout)]
+
+
+def oracle_run(orc, ocfg, p, batches, lr, accum=1):
+    """Steps the oracle through packed batches with the reference's schedule; returns losses, weights, m, v."""
+    m, v = np.zeros_like(p), np.zeros_like(p)
+    losses, grads, opt_step, counter = [], None, 0, 0
+    for tokens, starts in batches:
+        loss, g = orc.step_full(ocfg, p, np.asarray(tokens, np.int32), np.asarray(starts, np.int32),
+                                grads0=grads if counter else None)
+        losses.append(loss)
+        grads = g
+        counter += 1
+        if counter >= accum:
+            opt_step += 1
+            p, m, v = orc.adamw(p, g, m, v, orc.lr_schedule(lr, opt_step, accum), 0.9, 0.999, 0.01, 1e-8, opt_step)
+            counter = 0
+    return losses, p, m, v
+
+
+def read_optim(path):
+    from safetensors import safe_open
+    with safe_open(path + ".optim", framework="np") as f:
+        return f.get_tensor("params"), f.get_tensor("adam.m"), f.get_tensor("adam.v")
+
+
+def test_front_end_full_training_matches_oracle(tmp_path, orc):
+    assert os.path.exists(BIN), "seraph_amd/bin/seraph-train-hip is not built"
+    mdir, ckpt = str(tmp_path / "model"), str(tmp_path / "ckpt")
+    ocfg, cfg, p0 = make_model_dir(mdir, orc, SHAPE, seed=11)
+    samples = make_samples(12, 17, SHAPE["vocab"])
+    samples[4] = samples[4][:1]                                   # skipped: nothing to predict
+    samples[7] = np.concatenate([samples[7]] * 3)[:50]            # truncated to --max-seq
+    write_ttok(os.path.join(mdir, "train.ttok"), samples, vocab=SHAPE["vocab"])
+    rc, out, err = run_cli([mdir, os.path.join(mdir, "train.ttok"), "--full-training", "--batch", 3, "--max-seq", 24,
+                            "--lr", 2e-3, "--log-every", 1, "--save-every", 4, "--checkpoint", ckpt])
+    assert rc == 0, err[-2000:]
+    tokens = np.concatenate(samples)
+    offsets = np.concatenate([[0], np.cumsum([len(s) for s in samples])]).tolist()
+    batches = reference_pack(tokens.tolist(), offsets, 3, 24)
+    ref_losses, rp, rm, rv = oracle_run(orc, ocfg, p0.copy(), batches, 2e-3)
+    got = step_losses(out)
+    assert [s for s, _ in got] == list(range(1, len(batches) + 1))
+    assert np.allclose([l for _, l in got], ref_losses, atol=1.5e-4), (got, ref_losses)
+    assert f"batch={len(batches[0][1]) - 1}" in out
+
+    final = os.path.join(ckpt, "checkpoint_final.safetensors")
+    gp, gm, gv = read_optim(final)
+    sl = tensor_slices(ocfg)
+    check_tensors(gp, rp, sl, "weight")
+    check_tensors(gm, rm, sl, "adam m")
+    check_tensors(gv, rv, sl, "adam v")
+    from seraph_amd import io as sio
+    bf = sio.checkpoint_load(final, cfg)
+    assert np.array_equal(bf.view(np.uint32), gp.view(np.uint32) & np.uint32(0xFFFF0000))     # truncation of what was trained
+    st = sio.train_state_load(final)
+    assert st["step"] == len(batches) and st["optimizer_step"] == len(batches) and st["epoch"] == 0
+    assert abs(st["loss"] - ref_losses[-1]) < 1e-5 * max(1.0, ref_losses[-1])
+    assert os.path.exists(os.path.join(ckpt, "checkpoint_4.safetensors.state"))
+    log = open(os.path.join(ckpt, "train.log")).read()
+    assert len(step_losses(log)) == len(batches)
+
+
+def test_front_end_resume_continues_exactly(tmp_path, orc):
+    mdir = str(tmp_path / "model")
+    ocfg, cfg, p0 = make_model_dir(mdir, orc, SHAPE, seed=21)
+    samples = make_samples(22, 12, SHAPE["vocab"], lo=8, hi=20)
+    ttok = os.path.join(mdir, "train.ttok")
+    write_ttok(ttok, samples, vocab=SHAPE["vocab"])
+    common = [mdir, ttok, "--full-training", "--batch", 2, "--max-seq", 32, "--lr", 1e-3, "--log-every", 1, "--save-every", 0]
+    rc, out_all, err = run_cli(common + ["--checkpoint", tmp_path / "a"])
+    assert rc == 0, err[-2000:]
+    rc, out_1, err = run_cli(common + ["--checkpoint", tmp_path / "b", "--max-steps", 3])
+    assert rc == 0, err[-2000:]
+    # second epoch from the three-step checkpoint: same schedule position, same moments
+    rc, out_2, err = run_cli(common + ["--checkpoint", tmp_path / "c", "--epochs", 2, "--max-steps", 2,
+                                       "--resume", tmp_path / "b" / "checkpoint_final.safetensors"])
+    assert rc == 0, err[-2000:]
+    assert "Loaded FP32 weights and Adam moments" in out_2 and "step 3" in out_2
+    tokens = np.concatenate(samples)
+    offsets = np.concatenate([[0], np.cumsum([len(s) for s in samples])]).tolist()
+    batches = reference_pack(tokens.tolist(), offsets, 2, 32)
+    ref_losses, rp, rm, rv = oracle_run(orc, ocfg, p0.copy(), batches[:3] + batches[:2], 1e-3)
+    got = [l for _, l in step_losses(out_1)] + [l for _, l in step_losses(out_2)]
+    assert np.allclose(got, ref_losses, atol=1.5e-4), (got, ref_losses)
+    gp, gm, gv = read_optim(str(tmp_path / "c" / "checkpoint_final.safetensors"))
+    sl = tensor_slices(ocfg)
+    check_tensors(gp, rp, sl, "weight after resume")
+    check_tensors(gv, rv, sl, "adam v after resume")
+
+
+def test_front_end_lora_and_validation(tmp_path, orc):
+    mdir = str(tmp_path / "model")
+    ocfg0, cfg0, p0 = make_model_dir(mdir, orc, SHAPE, seed=31)
+    samples = make_samples(32, 10, SHAPE["vocab"], lo=6, hi=24)
+    ttok = os.path.join(mdir, "train.ttok")
+    write_ttok(ttok, samples, vocab=SHAPE["vocab"])
+    val = make_samples(33, 5, SHAPE["vocab"], lo=2, hi=24)
+    vtok = os.path.join(mdir, "val.ttok")
+    write_ttok(vtok, val, vocab=SHAPE["vocab"])
+    ckpt = tmp_path / "l"
+    rc, out, err = run_cli([mdir, ttok, "--batch", 2, "--max-seq", 32, "--lr", 1e-3, "--log-every", 1, "--lora-rank", 4,
+                            "--lora-alpha", 8, "--seed", 77, "--val", vtok, "--eval-every", 2, 0, "--checkpoint", ckpt])
+    assert rc == 0, err[-2000:]
+    from seraph_amd import io as sio
+    from seraph_amd.trainer import model_config
+    shape = dict(SHAPE, lora_rank=4, lora_alpha=8.0, lora_mask=0b0000101)
+    ocfg = orc.make_config(**shape, rms_eps=1e-5, rope_theta=10000.0)
+    cfg = model_config(**shape, rms_eps=1e-5, rope_theta=10000.0)
+    lp = sio.lora_init(cfg, 77)
+    tokens = np.concatenate(samples)
+    offsets = np.concatenate([[0], np.cumsum([len(s) for s in samples])]).tolist()
+    batches = reference_pack(tokens.tolist(), offsets, 2, 32)
+    m, v = np.zeros_like(lp), np.zeros_like(lp)
+    ref_losses, val_losses = [], []
+    for i, (tk, ss) in enumerate(batches, 1):
+        loss, g = orc.step_lora(ocfg, p0, lp, np.asarray(tk, np.int32), np.asarray(ss, np.int32))
+        ref_losses.append(loss)
+        lp, m, v = orc.adamw(lp, g, m, v, orc.lr_schedule(1e-3, i, 1), 0.9, 0.999, 0.01, 1e-8, i)
+        if i % 2 == 0:                                            # src/train_cuda.c:2812-2847: mean of per-sample losses
+            per = [orc.step_lora(ocfg, p0, lp, s[:32], np.array([0, min(len(s), 32)], np.int32))[0] for s in val if len(s) >= 2]
+            val_losses.append(float(np.mean(per)))
+    got = [l for _, l in step_losses(out)]
+    assert np.allclose(got, ref_losses, atol=1.5e-4), (got, ref_losses)
+    got_val = [float(x) for x in re.findall(r"\[VAL\] Step \d+ \| Val Loss: ([0-9.]+)", out)]
+    assert np.allclose(got_val, val_losses, atol=1.5e-4), (got_val, val_losses)
+    saved = sio.lora_load(str(ckpt / "checkpoint_final.bin"), cfg)
+    bad = np.abs(saved - lp) > ATOL + RTOL * np.abs(lp)
+    assert not bad.any()
+    raw = open(ckpt / "checkpoint_final.bin", "rb").read()
+    assert struct.unpack_from("<IIiif", raw) == (0x4C4F5241, 2, SHAPE["layers"], 4, 8.0)
+
+
+def test_eval_forward_changes_nothing_and_matches_the_step_loss(tr, orc):
+    shape = dict(hidden=64, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=96, vocab=101)
+    ocfg = orc.make_config(**shape)
+    cfg = tr.model_config(**shape)
+    p = init_params(orc, ocfg, 41)
+    starts = np.array([0, 30, 31, 64], np.int32)
+    tok = np.random.default_rng(42).integers(0, 101, 64).astype(np.int32)
+    ref_loss, _ = orc.step_full(ocfg, p, tok, starts)
+    t = tr.Trainer(cfg, tr.optim_config(1e-3, gradient_accumulation_steps=2), max_tokens=64, max_batch=3)
+    t.upload(tr.PARAMS, p)
+    t.step(tok, starts)                                           # first micro-step: gradients pending
+    g_before = t.download(tr.GRADS)
+    loss = t.eval_forward(tok, starts)
+    assert abs(loss - ref_loss) < 1e-5 * max(1.0, abs(ref_loss))
+    assert t.accumulation_counter == 1 and t.optimizer_step == 0
+    assert np.array_equal(t.download(tr.GRADS), g_before) and np.array_equal(t.download(tr.PARAMS), p)
+    # evaluate(): per-sample mean and perplexity, truncation and the <2 token skip
+    offsets = np.array([0, 30, 31, 64], np.int32)
+    per = [orc.step_full(ocfg, p, tok[a:min(b, a + 20)], np.array([0, min(b - a, 20)], np.int32))[0]
+           for a, b in zip(offsets[:-1], offsets[1:]) if b - a >= 2]
+    vl, ppl = t.evaluate(tok, offsets, max_seq_len=20)
+    assert abs(vl - np.mean(per)) < 1e-5 * max(1.0, abs(vl)) and abs(ppl - np.exp(vl)) < 1e-3 * ppl
+    t.close()
+
+
+def test_nan_lattice_flags_the_first_poisoned_buffers_and_protects_the_weights(tr, orc):
+    shape = dict(hidden=64, layers=3, heads=4, kv_heads=2, head_dim=32, ffn=96, vocab=101)
+    ocfg = orc.make_config(**shape)
+    cfg = tr.model_config(**shape)
+    p = init_params(orc, ocfg, 51)
+    tok = np.random.default_rng(52).integers(0, 101, 48).astype(np.int32)
+    starts = np.array([0, 20, 48], np.int32)
+    L = tr.param_layout(cfg)
+    NL = shape["layers"]
+    fwd, bwd, gh, opt = 10, 10 + NL, 10 + 6 * NL, 10 + 7 * NL              # src/train.c:4525-4537
+
+    t = tr.Trainer(cfg, tr.optim_config(1e-3), max_tokens=48, max_batch=2)
+    t.enable_nan_check()
+    t.upload(tr.PARAMS, p)
+    loss = t.step(tok, starts)                                   # clean step: no flag, optimizer runs
+    assert np.isfinite(loss) and not t.nan_detected and t.optimizer_step == 1
+    flags = t.nan_flags()
+    assert flags.size == 10 + 7 * NL + 5 and not flags.any()
+
+    # poison the down projection of layer 1: hidden is clean after layer 0, not after layer 1
+    before = t.download(tr.PARAMS)
+    bad = before.copy()
+    bad[L.layer0 + 1 * L.layer_stride + L.down + 5] = np.nan
+    t.upload(tr.PARAMS, bad)
+    loss = t.step(tok, starts)
+    assert np.isnan(loss) and t.nan_detected
+    flags = t.nan_flags()
+    assert flags[7] == 0 and flags[fwd + 0] == 0 and flags[fwd + 1] == 1 and flags[fwd + 2] == 1
+    assert flags[1] == 1 and flags[2] == 1 and flags[6] == 1 and flags[3] == 1 and flags[4] == 1
+    assert flags[opt + 0] == 0                                   # the embedding itself was clean
+    assert all(flags[bwd + 5 * l + 0] == 1 for l in range(NL)) and flags[gh + 0] == 1 and flags[8] == 1
+    assert t.optimizer_step == 2                                 # counted (src/train.c:5452), but AdamW did not run:
+    after = t.download(tr.PARAMS)
+    assert np.array_equal(np.isnan(after), np.isnan(bad)) and np.array_equal(after[~np.isnan(bad)], bad[~np.isnan(bad)])
+    m = t.download(tr.ADAM_M)
+    assert np.isfinite(m).all()
+
+    # an Inf in the embedding is caught by the very first check
+    t.upload(tr.PARAMS, before)
+    worse = before.copy()
+    worse[L.embed + 3] = np.inf
+    t.upload(tr.PARAMS, worse)
+    t.step(tok, starts)
+    assert t.nan_flags()[opt + 0] == 1 and t.nan_detected
+    t.close()
