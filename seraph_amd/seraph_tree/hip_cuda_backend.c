@@ -38,9 +38,7 @@
 #include <stdlib.h>
 #include <string.h>
 
-#include "cuda_train_context.h"
-typedef struct cuda_profiler_t cuda_profiler_t;
-#include "cuda_profiler.h"
+#include "hip_cuda_backend.h"       /* Seraph's cuda_train_context.h and cuda_profiler.h */
 #include "lora.h"
 #include "seraph_hip.h"
 
