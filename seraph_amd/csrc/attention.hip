@@ -375,7 +375,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const float* __restrict
 // ---------------------------------------------------------------- backward: dK, dV
 // grid (key tiles of 128, kv heads); wave w owns keys j0+32w .. +31 for every query head of the group.
 template <int D, bool WRITE_DS>
-__global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_kernel(const float* __restrict__ Q, const float* __restrict__ K,
+__global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const float* __restrict__ Q, const float* __restrict__ K,
                                                                     const float* __restrict__ V, const float* __restrict__ dO,
                                                                     const float* __restrict__ LSE, const float* __restrict__ DELTA,
                                                                     float* __restrict__ dK, float* __restrict__ dV,
@@ -385,11 +385,14 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
                                                                     float* __restrict__ DS, int ds_slots,
                                                                     int split, float* __restrict__ partK, float* __restrict__ partV) {
     constexpr int LD = D + 4, DB = D / 32;
-    __shared__ __attribute__((aligned(16))) float sQ[2][32 * LD];
-    __shared__ __attribute__((aligned(16))) float sG[2][32 * LD];     // dO
-    __shared__ __attribute__((aligned(16))) float sLse[2][32];
-    __shared__ __attribute__((aligned(16))) float sDel[2][32];
-    __shared__ __attribute__((aligned(16))) int sSS[2][32];
+    // Query rows per iteration: two 32-row sub-tiles up to head_dim 64, so that one staging phase and
+    // one barrier serve 256 matrix instructions per wave, as one 32-row tile does at head_dim 128.
+    constexpr int QB = D <= 64 ? 2 : 1, QR = 32 * QB;
+    __shared__ __attribute__((aligned(16))) float sQ[2][QR * LD];
+    __shared__ __attribute__((aligned(16))) float sG[2][QR * LD];     // dO
+    __shared__ __attribute__((aligned(16))) float sLse[2][QR];
+    __shared__ __attribute__((aligned(16))) float sDel[2][QR];
+    __shared__ __attribute__((aligned(16))) int sSS[2][QR];
     __shared__ uint32_t sSeq[kMaxSeqLds];
     __shared__ int sItem;
     const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
@@ -443,10 +446,10 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
 
     const int64_t j_last = (j0 + 127 < T - 1) ? j0 + 127 : T - 1;
     const int64_t i_end = seqs.end_of((int)j_last);                         // queries of the last key's sequence
-    const int nq = (int)((i_end - j0 + 31) / 32);
+    const int nq = (int)((i_end - j0 + QR - 1) / QR);             // iterations per query head
     const int iters = nq * G;
 
-    Tile32<D> tq, tg;
+    Tile32<D> tq[QB], tg[QB];
     float st_lse = 0.f, st_del = 0.f;
     int st_ss = INT_MAX;
     // Sequence of each lane's query: queries advance by 32 per iteration, so the lane keeps a cursor into
@@ -455,8 +458,8 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
     int seq_cur = seq_j0, seq_head = -1;
     auto stats_load = [&](int it) {
         const int head = kvh * G + it / nq;
-        const int64_t i = j0 + 32 * (int64_t)(it % nq) + (threadIdx.x & 31);
-        if (threadIdx.x < 32) {
+        const int64_t i = j0 + QR * (int64_t)(it % nq) + (threadIdx.x & (QR - 1));
+        if (threadIdx.x < QR) {
             st_lse = i < T ? LSE[i * H + head] * kLog2e : 0.f;
             st_del = i < T ? DELTA[i * H + head] : 0.f;
             if (head != seq_head) { seq_cur = seq_j0; seq_head = head; }     // a new head starts over at the key tile
@@ -472,23 +475,30 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
         }
     };
     auto stats_store = [&](int buf) {
-        if (threadIdx.x < 32) { sLse[buf][threadIdx.x] = st_lse; sDel[buf][threadIdx.x] = st_del; sSS[buf][threadIdx.x] = st_ss; }
+        if (threadIdx.x < QR) { sLse[buf][threadIdx.x] = st_lse; sDel[buf][threadIdx.x] = st_del; sSS[buf][threadIdx.x] = st_ss; }
     };
     auto tiles_load = [&](int it) {
         const int head = kvh * G + it / nq;
-        const int64_t i0 = j0 + 32 * (int64_t)(it % nq);
-        tq.gload(Q, i0, T, qw, head * D);
-        tg.gload(dO, i0, T, qw, head * D);
+        const int64_t i0 = j0 + QR * (int64_t)(it % nq);
+#pragma unroll
+        for (int qb = 0; qb < QB; qb++) {
+            tq[qb].gload(Q, i0 + 32 * qb, T, qw, head * D);
+            tg[qb].gload(dO, i0 + 32 * qb, T, qw, head * D);
+        }
+    };
+    auto tiles_store = [&](int buf) {
+#pragma unroll
+        for (int qb = 0; qb < QB; qb++) { tq[qb].sstore(sQ[buf] + 32 * qb * LD); tg[qb].sstore(sG[buf] + 32 * qb * LD); }
     };
 
     {
         const int first = sub < iters ? sub : iters - 1;      // an item without iterations still stages a valid tile
         tiles_load(first); stats_load(first);
     }
-    tq.sstore(sQ[0]); tg.sstore(sG[0]); stats_store(0);
+    tiles_store(0); stats_store(0);
     __syncthreads();
 
-    // One iteration = one 32-query tile of one query head against the workgroup's 128 keys.  Only the
+    // One iteration = QB 32-query tiles of one query head against the workgroup's 128 keys.  Only the
     // first query tiles of a head (the diagonal) leave some wave without a visible key, so the loop is
     // written twice: with the per-wave test for those, and as straight-line code for the rest, where
     // every wave works.  (A conditional around the accumulating matrix instructions in the main
@@ -497,13 +507,16 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
     const bool wave_has_keys = jw0 < T;
     auto iteration = [&](int it, int li, auto may_skip) {
         const int cur = li & 1;
-        const int64_t i0 = j0 + 32 * (int64_t)(it % nq);
         // No branch around the loads and the LDS staging: past the last tile the same tile is simply
         // fetched and staged again.  (Loads and stores share one in-order counter; behind a branch the
         // compiler must wait for everything, including the dS stores, before it may touch the tile.)
         const int nxt = it + split < iters ? it + split : it;
         tiles_load(nxt);
         stats_load(nxt);
+#pragma unroll
+        for (int qb = 0; qb < QB; qb++) {
+        const int64_t i0 = j0 + QR * (int64_t)(it % nq) + 32 * qb;
+        const int ro = 32 * qb;                                              // this sub-tile's first row in the staged tiles
         if (!decltype(may_skip)::value || (i0 + 31 >= jw0 && wave_has_keys)) {   // some query of the tile can see this wave's keys
             v16f s, dp;
 #pragma unroll
@@ -512,8 +525,8 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
                 // operands of step s8+1 are requested from LDS before the 8 matrix instructions of step s8
                 float4 fa[2], fb[2], fv[2];
                 auto fetch = [&](int s8, int buf) {
-                    fa[buf] = *reinterpret_cast<const float4*>(&sQ[cur][r * LD + s8 * 8 + 4 * h]);
-                    fb[buf] = *reinterpret_cast<const float4*>(&sG[cur][r * LD + s8 * 8 + 4 * h]);
+                    fa[buf] = *reinterpret_cast<const float4*>(&sQ[cur][(ro + r) * LD + s8 * 8 + 4 * h]);
+                    fb[buf] = *reinterpret_cast<const float4*>(&sG[cur][(ro + r) * LD + s8 * 8 + 4 * h]);
                     if (kVinLds) fv[buf] = *reinterpret_cast<const float4*>(&sVt[(32 * w + r) * LD + s8 * 8 + 4 * h]);
                 };
                 fetch(0, 0);
@@ -542,12 +555,12 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
             // K was scaled by scale*log2(e) when it was loaded, so s is already the base-2 logit.  A tile whose
             // keys all precede its queries and all lie inside the sequence of its last (hence every) query
             // needs no mask: p = 2^(s - lse) for every element.
-            const int ss_last = __builtin_amdgcn_readfirstlane(sSS[cur][31]);        // INT_MAX if the tile runs past T
+            const int ss_last = __builtin_amdgcn_readfirstlane(sSS[cur][ro + 31]);   // INT_MAX if the tile runs past T
             const bool interior = (jw0 + 31 <= i0) && ((int)jw0 >= ss_last);
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-                const float4 lse4 = *reinterpret_cast<const float4*>(&sLse[cur][8 * g + 4 * h]);
-                const float4 del4 = *reinterpret_cast<const float4*>(&sDel[cur][8 * g + 4 * h]);
+                const float4 lse4 = *reinterpret_cast<const float4*>(&sLse[cur][ro + 8 * g + 4 * h]);
+                const float4 del4 = *reinterpret_cast<const float4*>(&sDel[cur][ro + 8 * g + 4 * h]);
                 const float* lse_p = &lse4.x; const float* del_p = &del4.x;
                 if (interior) {
 #pragma unroll
@@ -558,7 +571,7 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
                         dp[v] = p * (dp[v] - del_p[e]);
                     }
                 } else {
-                    const int4 ss4 = *reinterpret_cast<const int4*>(&sSS[cur][8 * g + 4 * h]);
+                    const int4 ss4 = *reinterpret_cast<const int4*>(&sSS[cur][ro + 8 * g + 4 * h]);
                     const int* ss_p = &ss4.x;
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
@@ -571,12 +584,12 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
                     }
                 }
             }
-            if (!decltype(may_skip)::value) {
+            if (!decltype(may_skip)::value && qb == 0) {
                 // Straight-line copy: stage the next tile now, ahead of the dS stores.  Loads and stores share
                 // one completion counter that the compiler must treat as unordered once both kinds are
                 // pending, so waiting for the tile's loads after the stores were issued would also wait
                 // for the stores.
-                tq.sstore(sQ[cur ^ 1]); tg.sstore(sG[cur ^ 1]); stats_store(cur ^ 1);
+                tiles_store(cur ^ 1); stats_store(cur ^ 1);
             }
             if (WRITE_DS) {
                 // dS tile (32 queries x 32 keys, row-major) for the dQ pass: band slot = query tile - key tile.
@@ -585,7 +598,7 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
                 const int head = kvh * G + it / nq;
                 const int64_t ntile = (int64_t)H * ((T + 31) >> 5) * ds_slots;
                 int64_t tidx = (((int64_t)head * ((T + 31) >> 5) + qt) * ds_slots + slot);
-                tidx = (slot >= 0 && slot < ds_slots) ? tidx : ntile;
+                tidx = (slot >= 0 && slot < ds_slots && qt < (int)((T + 31) >> 5)) ? tidx : ntile;
                 const uint64_t ta = reinterpret_cast<uint64_t>(DS + (tidx << 10));
                 const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)ta), hi = __builtin_amdgcn_readfirstlane((uint32_t)(ta >> 32));
                 const __amdgpu_buffer_rsrc_t rs =
@@ -600,8 +613,8 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
             {
                 DVec<DB> go[2], qq[2];
                 auto fetch = [&](int v, int buf) {
-                    go[buf] = lds_dvec<DB>(&sG[cur][acc_row(v, h) * LD], r);
-                    qq[buf] = lds_dvec<DB>(&sQ[cur][acc_row(v, h) * LD], r);
+                    go[buf] = lds_dvec<DB>(&sG[cur][(ro + acc_row(v, h)) * LD], r);
+                    qq[buf] = lds_dvec<DB>(&sQ[cur][(ro + acc_row(v, h)) * LD], r);
                 };
                 fetch(0, 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
@@ -629,12 +642,14 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dkv_
                 }
             }
         }
-        if (decltype(may_skip)::value) { tq.sstore(sQ[cur ^ 1]); tg.sstore(sG[cur ^ 1]); stats_store(cur ^ 1); }
+        }   // sub-tiles
+        if (decltype(may_skip)::value) { tiles_store(cur ^ 1); stats_store(cur ^ 1); }
         __syncthreads();
     };
     {
         // waves without keys (ragged end of the token axis) never take the straight-line copy
-        const int ndiag = j0 + 127 < T ? (nq < 4 ? nq : 4) : nq;
+        constexpr int kDiag = (4 + QB - 1) / QB;               // iterations that reach into the 128-key diagonal block
+        const int ndiag = j0 + 127 < T ? (nq < kDiag ? nq : kDiag) : nq;
         int li = 0;
         for (int g = 0; g < G; g++) {
             int n = ((sub - g * nq) % split + split) % split;      // this item's first query tile of head g
