@@ -95,7 +95,7 @@ __device__ __forceinline__ SeqTable load_seq_table(const uint32_t* __restrict__ 
     SeqTable st;
     st.g = seq_starts; st.s = nullptr; st.batch = batch; st.T = T;
     if (seq_starts && batch + 1 <= kMaxSeqLds) {
-        for (int i = threadIdx.x; i <= batch; i += kAttnThreads) lds[i] = seq_starts[i];
+        for (int i = threadIdx.x; i <= batch; i += (int)blockDim.x) lds[i] = seq_starts[i];
         st.s = lds;
     }
     __syncthreads();
@@ -353,13 +353,28 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_kernel(const float* 
 }
 
 // ---------------------------------------------------------------- delta = rowsum(dO * O)
-// one wave per token; a head's D values are spread over D/4 consecutive lanes
+// one wave per token; a head's D values are spread over D/4 consecutive lanes.  The wave also looks up the first
+// token of its token's sequence once, so the dK/dV kernel reads it like any other row statistic instead of
+// walking the offsets table for every (key tile, head) it visits the row for.
 template <int D>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const float* __restrict__ dO, const float* __restrict__ O,
-                                                         float* __restrict__ delta, int64_t T, int H) {
+                                                         float* __restrict__ delta, int64_t T, int H,
+                                                         const uint32_t* __restrict__ seq_starts, int batch, int* __restrict__ row_start) {
     const int lane = threadIdx.x & 63;
     const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= T) return;
+    if (lane == 0) {
+        int start = 0;
+        if (seq_starts) {
+            int lo = 0, hi = batch;                            // last sequence whose start is <= t
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if ((int64_t)seq_starts[mid + 1] <= t) lo = mid + 1; else hi = mid;
+            }
+            start = (int)seq_starts[lo];
+        }
+        row_start[t] = start;
+    }
     const int64_t qw = (int64_t)H * D;
     constexpr int LPH = D / 4;                                  // lanes per head
     for (int64_t c = lane * 4; c < qw; c += 256) {
@@ -378,6 +393,7 @@ template <int D, bool WRITE_DS>
 __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const float* __restrict__ Q, const float* __restrict__ K,
                                                                     const float* __restrict__ V, const float* __restrict__ dO,
                                                                     const float* __restrict__ LSE, const float* __restrict__ DELTA,
+                                                                    const int* __restrict__ ROWSTART,
                                                                     float* __restrict__ dK, float* __restrict__ dV,
                                                                     const uint32_t* __restrict__ seq_starts, int batch,
                                                                     int64_t T, int H, int KVH, float scale, float scale_log2e,
@@ -390,9 +406,12 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
     constexpr int QB = D <= 64 ? 2 : 1, QR = 32 * QB;
     __shared__ __attribute__((aligned(16))) float sQ[2][QR * LD];
     __shared__ __attribute__((aligned(16))) float sG[2][QR * LD];     // dO
-    __shared__ __attribute__((aligned(16))) float sLse[2][QR];
-    __shared__ __attribute__((aligned(16))) float sDel[2][QR];
-    __shared__ __attribute__((aligned(16))) int sSS[2][QR];
+    // Row statistics of the staged queries.  With two sub-tiles every lane of the workgroup stores (lanes past the
+    // QR rows into a dummy tail), which keeps the pipelined iteration free of branches: one scheduling region.
+    constexpr int SR = QB == 2 ? kAttnThreads : QR;
+    __shared__ __attribute__((aligned(16))) float sLse[2][SR];
+    __shared__ __attribute__((aligned(16))) float sDel[2][SR];
+    __shared__ __attribute__((aligned(16))) int sSS[2][SR];
     __shared__ uint32_t sSeq[kMaxSeqLds];
     __shared__ int sItem;
     const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
@@ -427,16 +446,15 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
 #pragma unroll
     for (int s8 = 0; s8 < D / 8; s8++) {
         kf[s8] = col_ok ? *reinterpret_cast<const float4*>(K + j_lane * kw + kvh * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
-        kf[s8].x *= scale_log2e; kf[s8].y *= scale_log2e; kf[s8].z *= scale_log2e; kf[s8].w *= scale_log2e;   // S comes out in base-2 units
         if (!kVinLds)
             vf[s8] = col_ok ? *reinterpret_cast<const float4*>(V + j_lane * kw + kvh * D + s8 * 8 + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
+    // Every global load of the item's set-up (K, V, the first query tile and its row statistics) is requested
+    // before the first result is used, so the set-up costs one memory round trip.
+    Tile32<D> tvv[kVinLds ? 4 : 1];
     if (kVinLds) {
-        Tile32<D> tvv[4];                                   // all four loads in flight before the first LDS write
 #pragma unroll
         for (int q = 0; q < 4; q++) tvv[q].gload(V, j0 + 32 * q, T, kw, kvh * D);
-#pragma unroll
-        for (int q = 0; q < 4; q++) tvv[q].sstore(sVt + q * 32 * LD);
     }
     v16f dk[DB], dv[DB];
 #pragma unroll
@@ -452,34 +470,31 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
     Tile32<D> tq[QB], tg[QB];
     float st_lse = 0.f, st_del = 0.f;
     int st_ss = INT_MAX;
-    // Sequence of each lane's query: queries advance by 32 per iteration, so the lane keeps a cursor into
-    // the offsets table and steps it forward (usually not at all) instead of searching every time.
-    const int seq_j0 = seqs.g ? seqs.find((int)(j0 < T ? j0 : T - 1)) : 0;
-    int seq_cur = seq_j0, seq_head = -1;
-    auto stats_load = [&](int it) {
-        const int head = kvh * G + it / nq;
-        const int64_t i = j0 + QR * (int64_t)(it % nq) + (threadIdx.x & (QR - 1));
-        if (threadIdx.x < QR) {
-            st_lse = i < T ? LSE[i * H + head] * kLog2e : 0.f;
-            st_del = i < T ? DELTA[i * H + head] : 0.f;
-            if (head != seq_head) { seq_cur = seq_j0; seq_head = head; }     // a new head starts over at the key tile
-            st_ss = INT_MAX;
-            if (i < T) {
-                st_ss = 0;
-                if (seqs.g) {
-                    const uint32_t* tab = seqs.s ? seqs.s : seqs.g;
-                    while ((int64_t)tab[seq_cur + 1] <= i) seq_cur++;      // i < T = tab[batch]: terminates
-                    st_ss = (int)tab[seq_cur];
-                }
-            }
+    // Row statistics (log-sum-exp, delta, first token of the row's sequence) of the staged queries; lanes past the
+    // QR rows repeat them.  Iterations are named by (hg, n): query head hg of the kv head's group and the n-th run
+    // of QR queries.  Rows past the end are read from the last token and replaced when they are stored.
+    bool st_ok = false;
+    auto stats_load = [&](int hg, int n) {
+        const int head = kvh * G + hg;
+        const int64_t i = j0 + QR * (int64_t)n + (threadIdx.x & (QR - 1));
+        st_ok = i < T;
+        const int64_t ic = st_ok ? i : T - 1;
+        if (SR == kAttnThreads || threadIdx.x < QR) {
+            st_lse = LSE[ic * H + head];
+            st_del = DELTA[ic * H + head];
+            st_ss = ROWSTART[ic];
         }
     };
     auto stats_store = [&](int buf) {
-        if (threadIdx.x < QR) { sLse[buf][threadIdx.x] = st_lse; sDel[buf][threadIdx.x] = st_del; sSS[buf][threadIdx.x] = st_ss; }
+        if (SR == kAttnThreads || threadIdx.x < QR) {
+            sLse[buf][threadIdx.x] = st_ok ? st_lse * kLog2e : 0.f;
+            sDel[buf][threadIdx.x] = st_ok ? st_del : 0.f;
+            sSS[buf][threadIdx.x] = st_ok ? st_ss : INT_MAX;
+        }
     };
-    auto tiles_load = [&](int it) {
-        const int head = kvh * G + it / nq;
-        const int64_t i0 = j0 + QR * (int64_t)(it % nq);
+    auto tiles_load = [&](int hg, int n) {
+        const int head = kvh * G + hg;
+        const int64_t i0 = j0 + QR * (int64_t)n;
 #pragma unroll
         for (int qb = 0; qb < QB; qb++) {
             tq[qb].gload(Q, i0 + 32 * qb, T, qw, head * D);
@@ -493,7 +508,15 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
 
     {
         const int first = sub < iters ? sub : iters - 1;      // an item without iterations still stages a valid tile
-        tiles_load(first); stats_load(first);
+        stats_load(first / nq, first % nq); tiles_load(first / nq, first % nq);
+    }
+#pragma unroll
+    for (int s8 = 0; s8 < D / 8; s8++) {   // S comes out in base-2 units
+        kf[s8].x *= scale_log2e; kf[s8].y *= scale_log2e; kf[s8].z *= scale_log2e; kf[s8].w *= scale_log2e;
+    }
+    if (kVinLds) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) tvv[q].sstore(sVt + q * 32 * LD);
     }
     tiles_store(0); stats_store(0);
     __syncthreads();
@@ -505,17 +528,16 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
     // loop makes the compiler shuttle the 128 dK/dV accumulator registers in and out of the
     // accumulation register file on every iteration.)
     const bool wave_has_keys = jw0 < T;
-    auto iteration = [&](int it, int li, auto may_skip) {
+    auto iteration = [&](int hg, int n, int li, int hg2, int n2, auto may_skip) {
         const int cur = li & 1;
         // No branch around the loads and the LDS staging: past the last tile the same tile is simply
         // fetched and staged again.  (Loads and stores share one in-order counter; behind a branch the
         // compiler must wait for everything, including the dS stores, before it may touch the tile.)
-        const int nxt = it + split < iters ? it + split : it;
-        tiles_load(nxt);
-        stats_load(nxt);
+        stats_load(hg2, n2);
+        tiles_load(hg2, n2);
 #pragma unroll
         for (int qb = 0; qb < QB; qb++) {
-        const int64_t i0 = j0 + QR * (int64_t)(it % nq) + 32 * qb;
+        const int64_t i0 = j0 + QR * (int64_t)n + 32 * qb;
         const int ro = 32 * qb;                                              // this sub-tile's first row in the staged tiles
         if (!decltype(may_skip)::value || (i0 + 31 >= jw0 && wave_has_keys)) {   // some query of the tile can see this wave's keys
             v16f s, dp;
@@ -595,7 +617,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
                 // dS tile (32 queries x 32 keys, row-major) for the dQ pass: band slot = query tile - key tile.
                 // A tile outside the band (it is all zeros: another sequence) goes to a spare tile behind the band.
                 const int qt = (int)(i0 >> 5), slot = qt - (int)(jw0 >> 5);
-                const int head = kvh * G + it / nq;
+                const int head = kvh * G + hg;
                 const int64_t ntile = (int64_t)H * ((T + 31) >> 5) * ds_slots;
                 int64_t tidx = (((int64_t)head * ((T + 31) >> 5) + qt) * ds_slots + slot);
                 tidx = (slot >= 0 && slot < ds_slots && qt < (int)((T + 31) >> 5)) ? tidx : ntile;
@@ -646,42 +668,220 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
         if (decltype(may_skip)::value) { tiles_store(cur ^ 1); stats_store(cur ^ 1); }
         __syncthreads();
     };
+    // The straight-line iteration for two sub-tiles, software-pipelined.  A SIMD runs one wave here, and while a
+    // wave's next instruction is a matrix instruction waiting for the matrix pipe nothing else issues, so the
+    // exponentials and masks only overlap with matrix work when they sit between matrix instructions of the
+    // same wave.  The two sub-tiles provide that: S/dP of sub-tile 1 carries the softmax of sub-tile 0, and
+    // dV/dK of sub-tile 0 carries the softmax of sub-tile 1.
+    auto iteration2 = [&](int hg, int n, int li, int hg2, int n2) {
+        constexpr int NS = D / 8, EPS = 16 / NS;               // S-phase steps, softmax elements per step
+        const int cur = li & 1;
+        const int64_t i00 = j0 + QR * (int64_t)n;
+        v16f s[2], dp[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) { s[t][v] = 0.0f; dp[t][v] = 0.0f; }
+        float4 fa[2], fb[2], fv[2];
+        auto sfetch = [&](int ro, int s8, int buf) {
+            fa[buf] = *reinterpret_cast<const float4*>(&sQ[cur][(ro + r) * LD + s8 * 8 + 4 * h]);
+            fb[buf] = *reinterpret_cast<const float4*>(&sG[cur][(ro + r) * LD + s8 * 8 + 4 * h]);
+            if (kVinLds) fv[buf] = *reinterpret_cast<const float4*>(&sVt[(32 * w + r) * LD + s8 * 8 + 4 * h]);
+        };
+        auto smma = [&](int t, int s8) {
+            const float4 a = fa[s8 & 1], b = fb[s8 & 1];
+            const float4 vv = kVinLds ? fv[s8 & 1] : vf[kVinLds ? 0 : s8];
+            s[t] = mfma(a.x, kf[s8].x, s[t]); dp[t] = mfma(b.x, vv.x, dp[t]);
+            s[t] = mfma(a.y, kf[s8].y, s[t]); dp[t] = mfma(b.y, vv.y, dp[t]);
+            s[t] = mfma(a.z, kf[s8].z, s[t]); dp[t] = mfma(b.z, vv.z, dp[t]);
+            s[t] = mfma(a.w, kf[s8].w, s[t]); dp[t] = mfma(b.w, vv.w, dp[t]);
+        };
+        // row statistics of four rows (accumulator rows 8g+4h .. +3 of sub-tile t), double-buffered like the operands
+        float4 lse4[2], del4[2];
+        int4 ss4[2];
+        auto stats_fetch = [&](int t, int g) {
+            lse4[g & 1] = *reinterpret_cast<const float4*>(&sLse[cur][32 * t + 8 * g + 4 * h]);
+            del4[g & 1] = *reinterpret_cast<const float4*>(&sDel[cur][32 * t + 8 * g + 4 * h]);
+            ss4[g & 1] = *reinterpret_cast<const int4*>(&sSS[cur][32 * t + 8 * g + 4 * h]);
+        };
+        // Element v of sub-tile t.  Every key of the workgroup precedes every query of a straight-line iteration, so
+        // the mask only has to drop queries of a later sequence and rows past the end (their start is INT_MAX).
+        auto soft = [&](int t, int v) {
+            const int g = v >> 2, e = v & 3;
+            const float lse = (&lse4[g & 1].x)[e], del = (&del4[g & 1].x)[e];
+            const int ssv = (&ss4[g & 1].x)[e];
+            const float p = (int)j_lane >= ssv ? fast_exp2(s[t][v] - lse) : 0.0f;
+            s[t][v] = p;
+            dp[t][v] = p * (dp[t][v] - del);
+        };
+        __amdgpu_buffer_rsrc_t ds_rs[2];
+        const int ds_lane_off = (4 * h * 32 + r) * 4;
+        auto ds_open = [&](int t) {
+            if (WRITE_DS) {
+                const int64_t i0 = i00 + 32 * t;
+                const int qt = (int)(i0 >> 5), slot = qt - (int)(jw0 >> 5);
+                const int head = kvh * G + hg;
+                const int64_t ntile = (int64_t)H * ((T + 31) >> 5) * ds_slots;
+                int64_t tidx = (((int64_t)head * ((T + 31) >> 5) + qt) * ds_slots + slot);
+                tidx = (slot >= 0 && slot < ds_slots && qt < (int)((T + 31) >> 5)) ? tidx : ntile;
+                const uint64_t ta = reinterpret_cast<uint64_t>(DS + (tidx << 10));
+                const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)ta), hi = __builtin_amdgcn_readfirstlane((uint32_t)(ta >> 32));
+                ds_rs[t] = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(((uint64_t)hi << 32) | lo), 0, 4096, 0x00020000);
+            }
+        };
+        auto ds_put = [&](int t, int v) {
+            if (WRITE_DS)
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(dp[t][v]), ds_rs[t], ds_lane_off + (8 * (v >> 2) + (v & 3)) * 128, 0, 0);
+        };
+        DVec<DB> go[2], qq[2];
+        auto dfetch = [&](int t, int v, int buf) {
+            go[buf] = lds_dvec<DB>(&sG[cur][(32 * t + acc_row(v, h)) * LD], r);
+            qq[buf] = lds_dvec<DB>(&sQ[cur][(32 * t + acc_row(v, h)) * LD], r);
+        };
+        auto dmma = [&](int t, int v) {
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                dv[db] = mfma(s[t][v], go[v & 1].v[db], dv[db]);
+                dk[db] = mfma(dp[t][v], qq[v & 1].v[db], dk[db]);
+            }
+        };
+
+        // Every step below is one scheduling region (nothing crosses the barrier that ends it), so the order of
+        // the steps is the order written here and the group barriers only arrange the inside of a step.
+        // phase 1: S/dP of sub-tile 0
+        sfetch(0, 0, 0);
+        stats_fetch(0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s8 = 0; s8 < NS; s8++) {
+            if (s8 + 1 < NS) sfetch(0, s8 + 1, (s8 + 1) & 1); else sfetch(32, 0, 0);
+            if (s8 == 0) tiles_load(hg2, n2);                  // address arithmetic and requests in the shadow of the matrix pipe
+            if (s8 == 1) stats_load(hg2, n2);
+            smma(0, s8);
+            __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // phase 2: S/dP of sub-tile 1, softmax of sub-tile 0 between its matrix instructions
+#pragma unroll
+        for (int s8 = 0; s8 < NS; s8++) {
+            if (s8 + 1 < NS) sfetch(32, s8 + 1, (s8 + 1) & 1);
+            const int g = (s8 * EPS) >> 2;
+            const bool new_g = ((s8 * EPS) & 3) == 0;
+            if (new_g) { if (g + 1 < 4) stats_fetch(0, g + 1); else stats_fetch(1, 0); }
+            smma(1, s8);
+            if (s8 < 2) ds_open(s8);
+#pragma unroll
+            for (int k = 0; k < EPS; k++) soft(0, s8 * EPS + k);
+            if (s8 + 1 < NS && new_g) __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+            else if (s8 + 1 < NS || new_g) __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+#pragma unroll
+            for (int m = 0; m < 8; m++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, EPS, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // phase 3: dV/dK of sub-tile 0 with the softmax of sub-tile 1 between its matrix instructions.  The first
+        // four steps also move the next tile to LDS (ahead of the dS stores: loads and stores share one completion
+        // counter), the others send out the dS values of sub-tile 0.
+        dfetch(0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            if (v + 1 < 16) dfetch(0, v + 1, (v + 1) & 1); else dfetch(1, 0, 0);
+            const bool new_g = (v & 3) == 0 && (v >> 2) + 1 < 4;
+            if (new_g) stats_fetch(1, (v >> 2) + 1);
+            dmma(0, v);
+            soft(1, v);
+            if (v == 0) tq[0].sstore(sQ[cur ^ 1]);
+            if (v == 1) tg[0].sstore(sG[cur ^ 1]);
+            if (v == 2) tq[1].sstore(sQ[cur ^ 1] + 32 * LD);
+            if (v == 3) { tg[1].sstore(sG[cur ^ 1] + 32 * LD); stats_store(cur ^ 1); }
+            if (v >= 4 && v < 8) { ds_put(0, 2 * (v - 4)); ds_put(0, 2 * (v - 4) + 1); }
+            if (v >= 8) ds_put(0, v);
+            if (new_g) __builtin_amdgcn_sched_group_barrier(0x100, 5, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+            for (int m = 0; m < 2 * DB; m++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, (8 + 2 * DB - 1) / (2 * DB), 0);
+                if (v < 4) __builtin_amdgcn_sched_group_barrier(0x200, (Tile32<D>::kSlots + 3 + 2 * DB - 1) / (2 * DB), 0);
+                else if (m < (v < 8 ? 2 : 1)) __builtin_amdgcn_sched_group_barrier(0x040, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // phase 4: dV/dK of sub-tile 1, its dS values leaving one per step
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            if (v + 1 < 16) dfetch(1, v + 1, (v + 1) & 1);
+            dmma(1, v);
+            ds_put(1, v);
+            if (v + 1 < 16) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x040, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2 * DB - 1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+    };
     {
         // waves without keys (ragged end of the token axis) never take the straight-line copy
         constexpr int kDiag = (4 + QB - 1) / QB;               // iterations that reach into the 128-key diagonal block
         const int ndiag = j0 + 127 < T ? (nq < kDiag ? nq : kDiag) : nq;
         int li = 0;
+        // the item's next iteration in (head, run) order, `split` places on; the last one names itself
+        auto successor = [&](int g, int n, int& g2, int& n2) {
+            g2 = g; n2 = n + split;
+            while (n2 >= nq && g2 + 1 < G) { n2 -= nq; g2++; }
+            if (n2 >= nq) { g2 = g; n2 = n; }
+        };
         for (int g = 0; g < G; g++) {
             int n = ((sub - g * nq) % split + split) % split;      // this item's first query tile of head g
-            for (; n < ndiag; n += split, li++) iteration(g * nq + n, li, std::true_type{});
-            for (; n < nq; n += split, li++) iteration(g * nq + n, li, std::false_type{});
+            int g2, n2;
+            for (; n < ndiag; n += split, li++) { successor(g, n, g2, n2); iteration(g, n, li, g2, n2, std::true_type{}); }
+            for (; n < nq; n += split, li++) {
+                successor(g, n, g2, n2);
+                if constexpr (QB == 2) iteration2(g, n, li, g2, n2); else iteration(g, n, li, g2, n2, std::false_type{});
+            }
         }
     }
     const bool rmw = split <= 1;                               // else: plain store into this item's slice
     float* outK = rmw ? dK : partK + (int64_t)sub * T * kw;
     float* outV = rmw ? dV : partV + (int64_t)sub * T * kw;
 
+    {
+        // lane r owns features DB*r .. DB*r+DB-1 of key row jw0 + acc_row(v, h).  When accumulating in place all
+        // 32 old values are requested before the first is used: one memory round trip instead of sixteen.
+        DVec<DB> oldk[16], oldv[16];
 #pragma unroll
-    for (int v = 0; v < 16; v++) {
-        const int64_t j = jw0 + acc_row(v, h);
-        if (j < T) {
-            float* pk = outK + j * kw + kvh * D + DB * r;      // lane r owns features DB*r .. DB*r+DB-1
-            float* pv = outV + j * kw + kvh * D + DB * r;
-            if (DB == 4) {
-                float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
-                if (rmw) { a = *reinterpret_cast<float4*>(pk); b = *reinterpret_cast<float4*>(pv); }
-                a.x += dk[0][v] * scale; a.y += dk[1 % DB][v] * scale; a.z += dk[2 % DB][v] * scale; a.w += dk[3 % DB][v] * scale;
-                b.x += dv[0][v]; b.y += dv[1 % DB][v]; b.z += dv[2 % DB][v]; b.w += dv[3 % DB][v];
-                *reinterpret_cast<float4*>(pk) = a; *reinterpret_cast<float4*>(pv) = b;
-            } else if (DB == 2) {
-                float2 a = make_float2(0.f, 0.f), b = a;
-                if (rmw) { a = *reinterpret_cast<float2*>(pk); b = *reinterpret_cast<float2*>(pv); }
-                a.x += dk[0][v] * scale; a.y += dk[1 % DB][v] * scale;
-                b.x += dv[0][v]; b.y += dv[1 % DB][v];
-                *reinterpret_cast<float2*>(pk) = a; *reinterpret_cast<float2*>(pv) = b;
-            } else {
-                pk[0] = (rmw ? pk[0] : 0.f) + dk[0][v] * scale;
-                pv[0] = (rmw ? pv[0] : 0.f) + dv[0][v];
+        for (int v = 0; v < 16; v++) {
+            const int64_t j = jw0 + acc_row(v, h);
+#pragma unroll
+            for (int db = 0; db < DB; db++) { oldk[v].v[db] = 0.f; oldv[v].v[db] = 0.f; }
+            if (rmw && j < T) {
+                oldk[v] = lds_dvec<DB>(outK + j * kw + kvh * D, r);
+                oldv[v] = lds_dvec<DB>(outV + j * kw + kvh * D, r);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int64_t j = jw0 + acc_row(v, h);
+            if (j < T) {
+                float* pk = outK + j * kw + kvh * D + DB * r;
+                float* pv = outV + j * kw + kvh * D + DB * r;
+                float a[DB], b[DB];
+#pragma unroll
+                for (int db = 0; db < DB; db++) { a[db] = oldk[v].v[db] + dk[db][v] * scale; b[db] = oldv[v].v[db] + dv[db][v]; }
+                if (DB == 4) {
+                    *reinterpret_cast<float4*>(pk) = make_float4(a[0], a[1 % DB], a[2 % DB], a[3 % DB]);
+                    *reinterpret_cast<float4*>(pv) = make_float4(b[0], b[1 % DB], b[2 % DB], b[3 % DB]);
+                } else if (DB == 2) {
+                    *reinterpret_cast<float2*>(pk) = make_float2(a[0], a[1 % DB]);
+                    *reinterpret_cast<float2*>(pv) = make_float2(b[0], b[1 % DB]);
+                } else {
+                    pk[0] = a[0]; pv[0] = b[0];
+                }
             }
         }
     }
@@ -926,7 +1126,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const f
 }
 
 // ---------------------------------------------------------------- host side
-struct AttnWs { float* lse; float* delta; float* out; float* partK; float* partV; float* ds; };
+struct AttnWs { float* lse; float* delta; float* out; float* partK; float* partV; int* row_start; float* ds; };
 constexpr int kMaxSplit = 4;
 
 // Band of dS tiles: for every head and 32-query tile, the key tiles from the diagonal down to the
@@ -944,8 +1144,10 @@ static size_t attn_ws_layout(int64_t T, int H, int KVH, int D, char* base, AttnW
     char* c = take((size_t)T * H * 4); char* d = take((size_t)T * H * 4);
     char* e = take((size_t)T * H * D * 4);
     char* pk = take((size_t)kMaxSplit * T * KVH * D * 4); char* pv = take((size_t)kMaxSplit * T * KVH * D * 4);
+    char* rs = take((size_t)T * 4);
     if (w) {
         w->lse = (float*)c; w->delta = (float*)d; w->out = (float*)e; w->partK = (float*)pk; w->partV = (float*)pv;
+        w->row_start = (int*)rs;
         w->ds = base ? (float*)(base + o) : nullptr;
     }
     return o;
@@ -992,25 +1194,26 @@ static int run_forward(const float* Q, const float* K, const float* V, float* O,
 
 template <int D>
 static int run_backward(const float* Q, const float* K, const float* V, const float* dO, const float* O, const float* lse,
-                        float* delta, float* dQ, float* dK, float* dV, const uint32_t* seq_starts, int batch,
+                        float* delta, int* row_start, float* dQ, float* dK, float* dV, const uint32_t* seq_starts, int batch,
                         int64_t T, int H, int KVH, float scale, float* ds, int ds_slots, float* partK, float* partV, hipStream_t st) {
-    hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)ceil_div(T, 4)), dim3(256), 0, st, dO, O, delta, T, H);
+    hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)ceil_div(T, 4)), dim3(256), 0, st, dO, O, delta, T, H, seq_starts, batch, row_start);
     SERAPH_LAUNCH_CHECK();
     unsigned int *qkv = nullptr, *qq = nullptr;
     int rc = acquire_tile_queue(&qkv);
     if (rc == SERAPH_OK) rc = acquire_tile_queue(&qq);
     if (rc != SERAPH_OK) return rc;
     const int per_cu = D <= 64 ? 2 : 1;
-    const int64_t kv_items = ceil_div(T, 128) * KVH, slots = (int64_t)num_compute_units() * per_cu;
+    constexpr int kv_per_cu = 1;                               // the dK/dV kernel's registers and LDS tiles leave room for one workgroup
+    const int64_t kv_items = ceil_div(T, 128) * KVH, slots = (int64_t)num_compute_units() * kv_per_cu;
     // fewer (key tile, kv head) items than resident workgroups: split each between several of them
     int split = (int)(slots / kv_items);
     split = split < 1 ? 1 : (split > kMaxSplit ? kMaxSplit : split);
-    dim3 gkv(persistent_grid(kv_items * split, per_cu)), gq(persistent_grid(ceil_div(T, 128) * H, per_cu));
+    dim3 gkv(persistent_grid(kv_items * split, kv_per_cu)), gq(persistent_grid(ceil_div(T, 128) * H, per_cu));
     if (ds)
-        hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, true>), gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dK, dV, seq_starts, batch,
+        hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, true>), gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, row_start, dK, dV, seq_starts, batch,
                            T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots, split, partK, partV);
     else
-        hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, false>), gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dK, dV, seq_starts, batch,
+        hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, false>), gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, row_start, dK, dV, seq_starts, batch,
                            T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots, split, partK, partV);
     if (split > 1) {
         SERAPH_LAUNCH_CHECK();
@@ -1115,9 +1318,9 @@ int seraph_attention_backward_banded(const float* Q, const float* K, const float
         O = w.out; L = w.lse;
     }
     switch (head_dim) {
-        case 32: return run_backward<32>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, w.partK, w.partV, st);
-        case 64: return run_backward<64>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, w.partK, w.partV, st);
-        default: return run_backward<128>(Q, K, V, dO, O, L, w.delta, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, w.partK, w.partV, st);
+        case 32: return run_backward<32>(Q, K, V, dO, O, L, w.delta, w.row_start, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, w.partK, w.partV, st);
+        case 64: return run_backward<64>(Q, K, V, dO, O, L, w.delta, w.row_start, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, w.partK, w.partV, st);
+        default: return run_backward<128>(Q, K, V, dO, O, L, w.delta, w.row_start, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, ds, ds_slots, w.partK, w.partV, st);
     }
 }
 
