@@ -121,7 +121,7 @@ struct TileQueue {
     __device__ __forceinline__ int next() const {
         if (threadIdx.x == 0) *slot = (int)atomicAdd(&q[0], 1u);
         __syncthreads();
-        const int item = *slot;
+        const int item = __builtin_amdgcn_readfirstlane(*slot);    // the same for every lane: keep it, and what follows from it, scalar
         __syncthreads();
         return item < total ? item : -1;
     }
@@ -147,7 +147,9 @@ struct TileOrder {
     const int* order;      // LDS, or NULL = natural order
     int n;
     bool descending;
-    __device__ __forceinline__ int operator()(int rank) const { return order ? order[rank] : (descending ? n - 1 - rank : rank); }
+    __device__ __forceinline__ int operator()(int rank) const {   // rank is uniform, and so is the answer
+        return order ? __builtin_amdgcn_readfirstlane(order[rank]) : (descending ? n - 1 - rank : rank);
+    }
 };
 template <typename LenFn>
 __device__ __forceinline__ TileOrder rank_tiles_by_length(int* lens, int* order, int n, bool descending, LenFn len) {
@@ -406,9 +408,9 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
     constexpr int QB = D <= 64 ? 2 : 1, QR = 32 * QB;
     __shared__ __attribute__((aligned(16))) float sQ[2][QR * LD];
     __shared__ __attribute__((aligned(16))) float sG[2][QR * LD];     // dO
-    // Row statistics of the staged queries.  With two sub-tiles every lane of the workgroup stores (lanes past the
-    // QR rows into a dummy tail), which keeps the pipelined iteration free of branches: one scheduling region.
-    constexpr int SR = QB == 2 ? kAttnThreads : QR;
+    // Row statistics of the staged queries.  Every lane of the workgroup stores (lanes past the QR rows into a
+    // dummy tail), which keeps the pipelined iterations free of branches: one scheduling region.
+    constexpr int SR = kAttnThreads;
     __shared__ __attribute__((aligned(16))) float sLse[2][SR];
     __shared__ __attribute__((aligned(16))) float sDel[2][SR];
     __shared__ __attribute__((aligned(16))) int sSS[2][SR];
@@ -668,6 +670,133 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
         if (decltype(may_skip)::value) { tiles_store(cur ^ 1); stats_store(cur ^ 1); }
         __syncthreads();
     };
+    // The straight-line iteration for one sub-tile (head_dim 128), in four runs of matrix instructions that carry
+    // the other work between them (a SIMD runs one wave here, and while a wave's next instruction is a matrix
+    // instruction waiting for the pipe nothing else issues): S with the first half of dP, and the next tile's
+    // requests; the second half of dP with p = 2^(s - lse); dV = P^T dO with dS = p (dP - delta) and the LDS
+    // writes of the next tile; dK = dS^T Q with the dS stores.
+    auto iteration1 = [&](int hg, int n, int li, int hg2, int n2) {
+        constexpr int NS = D / 8, NH = NS / 2, EPS = 16 / NH;  // S steps, steps per half, exponentials per step
+        static_assert(QB == 2 || (NH >= 4 && 16 % NH == 0 && EPS <= 4), "one-sub-tile pipeline: head_dim 64 or 128");
+        const int cur = li & 1;
+        const int64_t i0 = j0 + QR * (int64_t)n;
+        v16f s, dp;
+#pragma unroll
+        for (int v = 0; v < 16; v++) { s[v] = 0.0f; dp[v] = 0.0f; }
+        float4 fa[2], fah[2], fb[2], fv[2];
+        auto qfetch = [&](int s8, int buf) {
+            fa[buf] = *reinterpret_cast<const float4*>(&sQ[cur][r * LD + s8 * 8 + 4 * h]);
+            fah[buf] = *reinterpret_cast<const float4*>(&sQ[cur][r * LD + (s8 + NH) * 8 + 4 * h]);
+        };
+        auto gfetch = [&](int s8, int buf) {
+            fb[buf] = *reinterpret_cast<const float4*>(&sG[cur][r * LD + s8 * 8 + 4 * h]);
+            if (kVinLds) fv[buf] = *reinterpret_cast<const float4*>(&sVt[(32 * w + r) * LD + s8 * 8 + 4 * h]);
+        };
+        auto dpmma = [&](int s8) {
+            const float4 b = fb[s8 & 1];
+            const float4 vv = kVinLds ? fv[s8 & 1] : vf[kVinLds ? 0 : s8];
+            dp = mfma(b.x, vv.x, dp); dp = mfma(b.y, vv.y, dp); dp = mfma(b.z, vv.z, dp); dp = mfma(b.w, vv.w, dp);
+        };
+        float4 lse4[2], del4[2];
+        int4 ss4[2];
+        __amdgpu_buffer_rsrc_t ds_rs;
+        const int ds_lane_off = (4 * h * 32 + r) * 4;
+        auto ds_open = [&]() {
+            if (WRITE_DS) {
+                const int qt = (int)(i0 >> 5), slot = qt - (int)(jw0 >> 5);
+                const int head = kvh * G + hg;
+                const int64_t ntile = (int64_t)H * ((T + 31) >> 5) * ds_slots;
+                int64_t tidx = (((int64_t)head * ((T + 31) >> 5) + qt) * ds_slots + slot);
+                tidx = (slot >= 0 && slot < ds_slots && qt < (int)((T + 31) >> 5)) ? tidx : ntile;
+                const uint64_t ta = reinterpret_cast<uint64_t>(DS + (tidx << 10));
+                const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)ta), hi = __builtin_amdgcn_readfirstlane((uint32_t)(ta >> 32));
+                ds_rs = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(((uint64_t)hi << 32) | lo), 0, 4096, 0x00020000);
+            }
+        };
+        DVec<DB> go[2], qq[2];
+
+        // run 1: S over the whole head and dP over its first half
+        qfetch(0, 0); gfetch(0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s8 = 0; s8 < NH; s8++) {
+            if (s8 + 1 < NH) { qfetch(s8 + 1, (s8 + 1) & 1); gfetch(s8 + 1, (s8 + 1) & 1); } else gfetch(NH, NH & 1);
+            if (s8 == 0) tiles_load(hg2, n2);                  // address arithmetic and requests in the shadow of the matrix pipe
+            if (s8 == 1) stats_load(hg2, n2);
+            if (s8 == 2) ds_open();
+            if (s8 == NH - 1) {
+                lse4[0] = *reinterpret_cast<const float4*>(&sLse[cur][4 * h]);
+                ss4[0] = *reinterpret_cast<const int4*>(&sSS[cur][4 * h]);
+            }
+            const float4 a = fa[s8 & 1], ah = fah[s8 & 1], b = fb[s8 & 1];
+            const float4 vv = kVinLds ? fv[s8 & 1] : vf[kVinLds ? 0 : s8];
+            s = mfma(a.x, kf[s8].x, s); dp = mfma(b.x, vv.x, dp); s = mfma(ah.x, kf[s8 + NH].x, s);
+            s = mfma(a.y, kf[s8].y, s); dp = mfma(b.y, vv.y, dp); s = mfma(ah.y, kf[s8 + NH].y, s);
+            s = mfma(a.z, kf[s8].z, s); dp = mfma(b.z, vv.z, dp); s = mfma(ah.z, kf[s8 + NH].z, s);
+            s = mfma(a.w, kf[s8].w, s); dp = mfma(b.w, vv.w, dp); s = mfma(ah.w, kf[s8 + NH].w, s);
+            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // run 2: the second half of dP; every key of the workgroup precedes every query of a straight-line iteration,
+        // so the mask only drops queries of a later sequence and rows past the end (their start is INT_MAX).  The
+        // compiler moves most of the exponentials to the head of run 3; pinning them between the matrix instructions
+        // here measured slower (19.2k against 18.8k cycles per iteration).
+#pragma unroll
+        for (int s8 = NH; s8 < NS; s8++) {
+            if (s8 + 1 < NS) gfetch(s8 + 1, (s8 + 1) & 1);
+            else { go[0] = lds_dvec<DB>(&sG[cur][acc_row(0, h) * LD], r); del4[0] = *reinterpret_cast<const float4*>(&sDel[cur][4 * h]); }
+            const int v0 = (s8 - NH) * EPS;
+            if ((v0 & 3) == 0 && (v0 >> 2) + 1 < 4) {
+                lse4[((v0 >> 2) + 1) & 1] = *reinterpret_cast<const float4*>(&sLse[cur][8 * ((v0 >> 2) + 1) + 4 * h]);
+                ss4[((v0 >> 2) + 1) & 1] = *reinterpret_cast<const int4*>(&sSS[cur][8 * ((v0 >> 2) + 1) + 4 * h]);
+            }
+            dpmma(s8);
+#pragma unroll
+            for (int k = 0; k < EPS; k++) {
+                const int v = v0 + k, g = v >> 2, e = v & 3;
+                s[v] = (int)j_lane >= (&ss4[g & 1].x)[e] ? fast_exp2(s[v] - (&lse4[g & 1].x)[e]) : 0.0f;
+            }
+#pragma unroll
+            for (int m = 0; m < 4; m++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 2 * EPS, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // run 3: dV, with dS = p (dP - delta) one step ahead of its use in run 4 and the next tile's LDS writes
+        // (ahead of the dS stores: loads and stores share one completion counter)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            if (v + 1 < 16) go[(v + 1) & 1] = lds_dvec<DB>(&sG[cur][acc_row(v + 1, h) * LD], r);
+            else qq[0] = lds_dvec<DB>(&sQ[cur][acc_row(0, h) * LD], r);
+            if ((v & 3) == 0 && (v >> 2) + 1 < 4) del4[((v >> 2) + 1) & 1] = *reinterpret_cast<const float4*>(&sDel[cur][8 * ((v >> 2) + 1) + 4 * h]);
+#pragma unroll
+            for (int db = 0; db < DB; db++) dv[db] = mfma(s[v], go[v & 1].v[db], dv[db]);
+            dp[v] = s[v] * (dp[v] - (&del4[(v >> 2) & 1].x)[v & 3]);
+            if (v == 0) tq[0].sstore(sQ[cur ^ 1]);
+            if (v == 1) tg[0].sstore(sG[cur ^ 1]);
+            if (v == 2) stats_store(cur ^ 1);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+            for (int m = 0; m < DB; m++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // run 4: dK, the dS values leaving one per step
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            if (v + 1 < 16) qq[(v + 1) & 1] = lds_dvec<DB>(&sQ[cur][acc_row(v + 1, h) * LD], r);
+#pragma unroll
+            for (int db = 0; db < DB; db++) dk[db] = mfma(dp[v], qq[v & 1].v[db], dk[db]);
+            if (WRITE_DS)
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(dp[v]), ds_rs, ds_lane_off + (8 * (v >> 2) + (v & 3)) * 128, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+    };
     // The straight-line iteration for two sub-tiles, software-pipelined.  A SIMD runs one wave here, and while a
     // wave's next instruction is a matrix instruction waiting for the matrix pipe nothing else issues, so the
     // exponentials and masks only overlap with matrix work when they sit between matrix instructions of the
@@ -842,7 +971,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
             for (; n < ndiag; n += split, li++) { successor(g, n, g2, n2); iteration(g, n, li, g2, n2, std::true_type{}); }
             for (; n < nq; n += split, li++) {
                 successor(g, n, g2, n2);
-                if constexpr (QB == 2) iteration2(g, n, li, g2, n2); else iteration(g, n, li, g2, n2, std::false_type{});
+                if constexpr (QB == 2) iteration2(g, n, li, g2, n2); else iteration1(g, n, li, g2, n2);
             }
         }
     }
