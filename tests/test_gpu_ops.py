@@ -296,7 +296,11 @@ def test_attention_forward(ops, orc, starts, H, KVH, D):
         parity(o2, ro, "attention out, unpacked call")
 
 
-ATTN_CASES_BWD = ATTN_CASES + [([0, 700, 731, 1500], 4, 2, 64), ([0, 513, 1030], 2, 1, 128), ([0, 90, 1000], 2, 2, 32)]
+ATTN_CASES_BWD = ATTN_CASES + [([0, 700, 731, 1500], 4, 2, 64), ([0, 513, 1030], 2, 1, 128), ([0, 90, 1000], 2, 2, 32),
+                               # enough (key tile, kv head) items to fill the chip: every item keeps all of its iterations
+                               ([0, 600, 1111, 1500, 2100, 2650, 3333, 4100], 16, 8, 128),
+                               ([0, 600, 1111, 1500, 2100, 2650, 3333, 4100], 8, 8, 64),
+                               ([0, 77, 2000, 4100], 8, 8, 32)]
 
 
 @pytest.mark.parametrize("starts,H,KVH,D", ATTN_CASES_BWD)
