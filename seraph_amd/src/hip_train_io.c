@@ -476,8 +476,15 @@ static inline float f16_to_f32(uint16_t h) {
 static void st_convert(const st_file_t* f, const st_entry_t* e, int64_t first, int64_t count, float* dst) {
     const char* base = (const char*)f->map + f->data_base + e->begin;
     if (e->dtype == ST_F32) memcpy(dst, base + first * 4, (size_t)count * 4);
-    else if (e->dtype == ST_BF16) { const uint16_t* s = (const uint16_t*)base + first; for (int64_t i = 0; i < count; i++) dst[i] = bf16_to_f32(s[i]); }
-    else { const uint16_t* s = (const uint16_t*)base + first; for (int64_t i = 0; i < count; i++) dst[i] = f16_to_f32(s[i]); }
+    else {
+        /* a safetensors header of odd length leaves 16-bit data at odd addresses: read through memcpy */
+        const char* s = base + first * 2;
+        for (int64_t i = 0; i < count; i++) {
+            uint16_t h;
+            memcpy(&h, s + 2 * i, 2);
+            dst[i] = e->dtype == ST_BF16 ? bf16_to_f32(h) : f16_to_f32(h);
+        }
+    }
 }
 
 /* ------------------------------------------------------------------ the model's tensor list */
