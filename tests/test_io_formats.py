@@ -238,6 +238,25 @@ def test_weights_load_single_file(tmp_path, dtype):
     assert np.array_equal(got2, want)
 
 
+def test_weights_load_with_an_odd_header_length(tmp_path):
+    """Header padding is free-form, so 16-bit tensor data can start at an odd file offset."""
+    import struct
+    from safetensors.torch import save_file
+    cfg = small_cfg(layers=1)
+    arena = np.random.default_rng(5).standard_normal(param_count(cfg)).astype(np.float32)
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in named_tensors(cfg, arena).items()},
+              str(tmp_path / "even.safetensors"))
+    raw = (tmp_path / "even.safetensors").read_bytes()
+    n = struct.unpack("<Q", raw[:8])[0]
+    header, data = raw[8:8 + n], raw[8 + n:]
+    pad = b" " if (n + 1) % 2 else b"  "
+    assert (8 + n + len(pad)) % 2 == 1
+    (tmp_path / "model.safetensors").write_bytes(struct.pack("<Q", n + len(pad)) + header + pad + data)
+    got, missing = sio.weights_load(tmp_path / "model.safetensors", cfg)
+    assert missing == 0
+    assert np.array_equal(got, torch.from_numpy(arena).to(torch.bfloat16).to(torch.float32).numpy())
+
+
 def test_weights_load_shards_prefixes_and_missing(tmp_path):
     from safetensors.torch import save_file
     cfg = small_cfg(layers=2)
