@@ -105,6 +105,15 @@ int seraph_gemm(const float* A, const float* B, float* C, int64_t M, int64_t N, 
 /* Name of the kernel instantiation seraph_gemm launches for this shape with 16-byte aligned
  * operands, as a profiler prints it (no reference counterpart; used to label timings). */
 const char* seraph_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int transpose_A, int transpose_B);
+/* C (+)= alpha * op(A) op(B): the step "product, then vulkan_scale of the product" of the LoRA path
+ * (src/train.c:5778-5796, :5803-5845) as one call.  With the scratch of seraph_gemm_scaled_ws_bytes a small
+ * output with a long K is cut into runs of K that separate workgroups take and a second kernel adds in run
+ * order (deterministic); without it, or for other shapes, it is seraph_gemm followed by seraph_scale.
+ * accumulate with alpha != 1 needs the scratch path.  No reference counterpart as a single op. */
+size_t seraph_gemm_scaled_ws_bytes(int64_t M, int64_t N, int64_t K, int transpose_A, int transpose_B);
+int seraph_gemm_scaled(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
+                       int transpose_A, int transpose_B, int accumulate, float alpha,
+                       void* ws, size_t ws_bytes, seraph_stream_t s);
 
 /* ---------------------------------------------------------------- attention */
 /* vulkan_batch_attention (include/vulkan_backend.h:485-488, shaders/batch_attention_stream.comp)

@@ -24,7 +24,8 @@ def kernels():
         lib = C.CDLL(KERNEL_LIB, mode=C.RTLD_GLOBAL)
         lib.seraph_hip_last_error.restype = C.c_char_p
         for name in ("seraph_attention_backward_ws_bytes", "seraph_attention_backward_ws_bytes_banded",
-                     "seraph_rmsnorm_backward_ws_bytes", "seraph_embedding_backward_ws_bytes"):
+                     "seraph_rmsnorm_backward_ws_bytes", "seraph_embedding_backward_ws_bytes",
+                     "seraph_gemm_scaled_ws_bytes"):
             getattr(lib, name).restype = C.c_size_t
         _kernels = lib
     return _kernels

@@ -466,12 +466,15 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_kerne
 // waves split every 32-deep K stage between them (wave w takes the 8-deep slab w); the four
 // partial accumulators are added in a fixed order through LDS, so the result does not depend on
 // timing.  Same loaders and staging as the pipelined kernel.
+// With `slices` > 1 the grid's y index also cuts K into that many equal runs of stages; a workgroup then
+// stores its tile of run y, unscaled, into part[y] (M x N each) and gemm_slices_sum_kernel adds the runs.
 template <bool A_KC, bool B_KC>
 __global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_kernel(const float* __restrict__ A,
                                                                                const float* __restrict__ B,
                                                                                float* __restrict__ C,
                                                                                int64_t M, int64_t N, int64_t K,
-                                                                               int accumulate, int nbm, int nbn) {
+                                                                               int accumulate, int nbm, int nbn,
+                                                                               int slices, float* __restrict__ part) {
     constexpr int BT = 32;
     constexpr int A_FLOATS = lds_floats<BT, A_KC>(), B_FLOATS = lds_floats<BT, B_KC>();
     __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
@@ -492,10 +495,11 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_kernel(c
     FastLoader<BT, B_KC> lb;
     la.init(lda, m0, M);
     lb.init(ldb, n0, N);
-    const float* ta = A_KC ? A + m0 * lda : A + m0;
-    const float* tb = B_KC ? B + n0 * ldb : B + n0;
+    const int64_t k_run = K / slices, k0 = (int64_t)blockIdx.y * k_run;          // whole stages: the launcher sees to it
+    const float* ta = A_KC ? A + m0 * lda + k0 : A + m0 + k0 * lda;
+    const float* tb = B_KC ? B + n0 * ldb + k0 : B + n0 + k0 * ldb;
     const int64_t step_a = A_KC ? kBK : kBK * lda, step_b = B_KC ? kBK : kBK * ldb;
-    const int nk = (int)(K / kBK);
+    const int nk = (int)(k_run / kBK);
     // this wave's slab of a stage: k = 8*wave + 4h + q
     const int fa_off = A_KC ? r * (kBK + kPadK) + 8 * wave + 4 * h : (8 * wave + 4 * h) * (BT + kPadM) + r;
     const int fb_off = B_KC ? r * (kBK + kPadK) + 8 * wave + 4 * h : (8 * wave + 4 * h) * (BT + kPadM) + r;
@@ -555,10 +559,67 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_kernel(c
         const int64_t row = m0 + e / BT, col = n0 + e % BT;
         if (row < M && col < N) {
             const float v = ((red[0][e] + red[1][e]) + red[2][e]) + red[3][e];
-            float* dst = C + row * N + col;
-            *dst = accumulate ? *dst + v : v;
+            if (slices > 1) {
+                part[(int64_t)blockIdx.y * M * N + row * N + col] = v;
+            } else {
+                float* dst = C + row * N + col;
+                *dst = accumulate ? *dst + v : v;
+            }
         }
     }
+}
+
+// ---------------------------------------------------------------------------------------------
+// C[M,N] (+)= A[M,K] B[N,K]^T with K <= 32 (a rank-sized inner dimension): bound by the traffic of C, so no
+// matrix instructions.  A lane keeps its four columns' rows of B in registers, a wave walks down rows of A,
+// whose K values are the same for all lanes (scalar loads), and adds in ascending k.
+template <int K4>
+__global__ __launch_bounds__(256) void gemm_smallk_kernel(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
+                                                          int64_t M, int64_t N, int accumulate, int rows_per_wave) {
+    constexpr int K = 4 * K4;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t n = ((int64_t)blockIdx.x * 64 + lane) * 4;
+    const bool col_ok = n < N;                                  // N is a multiple of 4
+    float4 b[4][K4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int q = 0; q < K4; q++)
+            b[j][q] = col_ok ? *reinterpret_cast<const float4*>(B + (n + j) * K + 4 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
+    const int64_t m0 = ((int64_t)blockIdx.y * 4 + wave) * rows_per_wave;
+    for (int r = 0; r < rows_per_wave && m0 + r < M; r++) {
+        const float* a = A + (m0 + r) * K;
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < K4; q++) {
+            const float4 av = *reinterpret_cast<const float4*>(a + 4 * q);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                acc[j] = fmaf(av.x, b[j][q].x, acc[j]);
+                acc[j] = fmaf(av.y, b[j][q].y, acc[j]);
+                acc[j] = fmaf(av.z, b[j][q].z, acc[j]);
+                acc[j] = fmaf(av.w, b[j][q].w, acc[j]);
+            }
+        }
+        if (col_ok) {
+            float4* dst = reinterpret_cast<float4*>(C + (m0 + r) * N + n);
+            float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (accumulate) o = *dst;
+            o.x += acc[0]; o.y += acc[1]; o.z += acc[2]; o.w += acc[3];
+            *dst = o;
+        }
+    }
+}
+
+// C (+)= alpha * (part[0] + part[1] + ... ), the runs added in index order
+__global__ __launch_bounds__(256) void gemm_slices_sum_kernel(const float* __restrict__ part, float* __restrict__ C, int64_t n,
+                                                              int slices, float alpha, int accumulate) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float v = part[i];
+    for (int p = 1; p < slices; p++) v += part[(int64_t)p * n + i];
+    v *= alpha;
+    C[i] = accumulate ? C[i] + v : v;
 }
 
 // The pipelined kernel needs whole K stages, and every per-lane offset inside a tile panel
@@ -611,6 +672,12 @@ static bool use_big_tiles(int64_t M, int64_t N) {
     return ceil_div(M, 128) * ceil_div(N, 128) >= num_compute_units();
 }
 
+// A k-contiguous pair of operands with at most 32 values of k and a C of whole 16-byte groups.
+static bool use_smallk(const float* A, const float* B, const float* C, int64_t M, int64_t N, int64_t K, int tA, int tB) {
+    return !tA && tB && K >= 4 && K <= 32 && K % 4 == 0 && N % 4 == 0 && M * N >= 65536 &&
+           (!A || (aligned16(A) && aligned16(B) && aligned16(C)));
+}
+
 // Fewer 64x64 tiles than compute units and a K long enough to be worth splitting between waves.
 static bool use_splitk(int64_t M, int64_t N, int64_t K, int tA, int tB) {
     return !use_big_tiles(M, N) && ceil_div(M, 64) * ceil_div(N, 64) < num_compute_units() && K >= 256 &&
@@ -629,6 +696,10 @@ extern "C" const char* seraph_gemm_kernel_name(int64_t M, int64_t N, int64_t K, 
          "seraph::gemm_f32_mfma_pipelined_kernel<1, 1, false, false>", "seraph::gemm_f32_mfma_pipelined_kernel<1, 1, false, true>"},
         {"seraph::gemm_f32_mfma_pipelined_kernel<2, 2, true, false>", "seraph::gemm_f32_mfma_pipelined_kernel<2, 2, true, true>",
          "seraph::gemm_f32_mfma_pipelined_kernel<2, 2, false, false>", "seraph::gemm_f32_mfma_pipelined_kernel<2, 2, false, true>"}};
+    static const char* smallk[8] = {"seraph::gemm_smallk_kernel<1>", "seraph::gemm_smallk_kernel<2>", "seraph::gemm_smallk_kernel<3>",
+                                    "seraph::gemm_smallk_kernel<4>", "seraph::gemm_smallk_kernel<5>", "seraph::gemm_smallk_kernel<6>",
+                                    "seraph::gemm_smallk_kernel<7>", "seraph::gemm_smallk_kernel<8>"};
+    if (use_smallk(nullptr, nullptr, nullptr, M, N, K, transpose_A, transpose_B)) return smallk[K / 4 - 1];
     const int64_t lda = transpose_A ? M : K, ldb = transpose_B ? K : N;
     const bool fast = lda % 4 == 0 && ldb % 4 == 0 && pipelined_ok(M, N, K, transpose_A, transpose_B);
     static const char* splitk[4] = {"seraph::gemm_f32_mfma_splitk_kernel<true, false>", "seraph::gemm_f32_mfma_splitk_kernel<true, true>",
@@ -645,13 +716,26 @@ extern "C" int seraph_gemm(const float* A, const float* B, float* C, int64_t M, 
     const int64_t lda = transpose_A ? M : K, ldb = transpose_B ? K : N;
     const bool vec = (lda % 4 == 0) && (ldb % 4 == 0) && aligned16(A) && aligned16(B);
     hipStream_t st = as_stream(s);
+    if (use_smallk(A, B, C, M, N, K, transpose_A, transpose_B)) {
+        const int rows_per_wave = 8;
+        const dim3 grid((unsigned)ceil_div(N, 256), (unsigned)ceil_div(M, 4 * rows_per_wave));
+        SERAPH_REQUIRE(grid.y <= 65535u * 1024u, "gemm: too many rows");
+        switch (K / 4) {
+#define GOK(K4) case K4: hipLaunchKernelGGL(gemm_smallk_kernel<K4>, grid, dim3(256), 0, st, A, B, C, M, N, accumulate, rows_per_wave); break;
+            GOK(1) GOK(2) GOK(3) GOK(4) GOK(5) GOK(6) GOK(7) GOK(8)
+#undef GOK
+        }
+        SERAPH_LAUNCH_CHECK();
+        return SERAPH_OK;
+    }
     if (use_big_tiles(M, N))
         return launch_gemm<2, 2>(A, B, C, M, N, K, transpose_A, transpose_B, accumulate, vec, st);
     if (vec && use_splitk(M, N, K, transpose_A, transpose_B)) {
         const int64_t nbm = ceil_div(M, 32), nbn = ceil_div(N, 32);
         const dim3 grid((unsigned)(nbm * nbn)), block(kGemmThreads);
 #define GOSK(AKC, BKC) \
-    hipLaunchKernelGGL((gemm_f32_mfma_splitk_kernel<AKC, BKC>), grid, block, 0, st, A, B, C, M, N, K, accumulate, (int)nbm, (int)nbn)
+    hipLaunchKernelGGL((gemm_f32_mfma_splitk_kernel<AKC, BKC>), grid, block, 0, st, A, B, C, M, N, K, accumulate, (int)nbm, (int)nbn, 1, \
+                       (float*)nullptr)
         if (!transpose_A && !transpose_B) GOSK(true, false);
         else if (!transpose_A && transpose_B) GOSK(true, true);
         else if (transpose_A && !transpose_B) GOSK(false, false);
@@ -661,4 +745,60 @@ extern "C" int seraph_gemm(const float* A, const float* B, float* C, int64_t M, 
         return SERAPH_OK;
     }
     return launch_gemm<1, 1>(A, B, C, M, N, K, transpose_A, transpose_B, accumulate, vec, st);
+}
+
+// ---------------------------------------------------------------------------------------------
+// C (+)= alpha * op(A) op(B) for products with a small output and a long K (the rank-sized LoRA products):
+// K is cut into runs that separate workgroups take, the runs are added in a fixed order.
+constexpr int kMaxSlices = 8;
+
+// runs of at least four stages, about two workgroups per compute unit in all
+static int slice_count(int64_t M, int64_t N, int64_t K, int tA, int tB) {
+    if (!use_splitk(M, N, K, tA, tB)) return 1;
+    const int64_t tiles = ceil_div(M, 32) * ceil_div(N, 32);
+    int64_t s = 2 * (int64_t)num_compute_units() / tiles;
+    if (s > kMaxSlices) s = kMaxSlices;
+    while (s > 1 && (K % (s * kBK) != 0 || K / s < 4 * kBK)) s--;
+    return (int)(s < 1 ? 1 : s);
+}
+
+extern "C" size_t seraph_gemm_scaled_ws_bytes(int64_t M, int64_t N, int64_t K, int transpose_A, int transpose_B) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const int s = slice_count(M, N, K, transpose_A, transpose_B);
+    return s > 1 ? (size_t)s * (size_t)M * (size_t)N * 4 : 0;
+}
+
+extern "C" int seraph_gemm_scaled(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
+                                  int transpose_A, int transpose_B, int accumulate, float alpha,
+                                  void* ws, size_t ws_bytes, seraph_stream_t s) {
+    if (M == 0 || N == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(A && B && C, "gemm_scaled: NULL pointer");
+    SERAPH_REQUIRE(M > 0 && N > 0 && K >= 0, "gemm_scaled: bad shape %lld x %lld x %lld", (long long)M, (long long)N, (long long)K);
+    const int64_t lda = transpose_A ? M : K, ldb = transpose_B ? K : N;
+    const bool vec = (lda % 4 == 0) && (ldb % 4 == 0) && aligned16(A) && aligned16(B);
+    const int slices = vec ? slice_count(M, N, K, transpose_A, transpose_B) : 1;
+    hipStream_t st = as_stream(s);
+    if (slices > 1 && ws && aligned16(ws) && ws_bytes >= (size_t)slices * (size_t)M * (size_t)N * 4) {
+        const int64_t nbm = ceil_div(M, 32), nbn = ceil_div(N, 32);
+        const dim3 grid((unsigned)(nbm * nbn), (unsigned)slices), block(kGemmThreads);
+        float* part = (float*)ws;
+#define GOSK(AKC, BKC) \
+    hipLaunchKernelGGL((gemm_f32_mfma_splitk_kernel<AKC, BKC>), grid, block, 0, st, A, B, C, M, N, K, 0, (int)nbm, (int)nbn, slices, part)
+        if (!transpose_A && !transpose_B) GOSK(true, false);
+        else if (!transpose_A && transpose_B) GOSK(true, true);
+        else if (transpose_A && !transpose_B) GOSK(false, false);
+        else GOSK(false, true);
+#undef GOSK
+        SERAPH_LAUNCH_CHECK();
+        const int64_t n = M * N;
+        hipLaunchKernelGGL(gemm_slices_sum_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, st, part, C, n, slices, alpha, accumulate);
+        SERAPH_LAUNCH_CHECK();
+        return SERAPH_OK;
+    }
+    // one pass; a scale that cannot be folded in follows as its own sweep
+    SERAPH_REQUIRE(!accumulate || alpha == 1.0f, "gemm_scaled: scratch of %zu bytes needed to accumulate a scaled product of this shape",
+                   seraph_gemm_scaled_ws_bytes(M, N, K, transpose_A, transpose_B));
+    int rc = seraph_gemm(A, B, C, M, N, K, transpose_A, transpose_B, accumulate, s);
+    if (rc != SERAPH_OK || alpha == 1.0f) return rc;
+    return seraph_scale(C, (size_t)(M * N), alpha, s);
 }

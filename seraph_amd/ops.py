@@ -92,6 +92,19 @@ def gemm(A, B, M, N, K, tA=0, tB=0, out=None, accumulate=False):
     return out
 
 
+def gemm_scaled(A, B, M, N, K, tA=0, tB=0, out=None, accumulate=False, alpha=1.0, scratch=True):
+    """out (+)= alpha * op(A) op(B); with scratch, small outputs with a long K are computed in runs of K."""
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=A.device)
+    k = kernels()
+    nbytes = k.seraph_gemm_scaled_ws_bytes(i64(M), i64(N), i64(K), C.c_int(tA), C.c_int(tB)) if scratch else 0
+    ws = torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=A.device) if scratch else None
+    check(k.seraph_gemm_scaled(_p(A), _p(B), _p(out), i64(M), i64(N), i64(K), C.c_int(tA), C.c_int(tB),
+                               C.c_int(1 if accumulate else 0), f32(alpha), _p(ws), C.c_size_t(int(nbytes)), _stream()),
+          "gemm_scaled")
+    return out
+
+
 def attention_forward(Q, K, V, heads, kv_heads, head_dim, seq_starts=None, scale=None, want_lse=True):
     T = Q.shape[0]
     out = torch.empty_like(Q)

@@ -137,6 +137,11 @@ static void op_fold(hip_trainer_t* t) {
     OP(seraph_gemm_kernel_name((M_), (N_), (K_), (tA_), (tB_)), 2.0 * (double)(M_) * (double)(N_) * (double)(K_), 0.0, \
        seraph_gemm((A_), (B_), (C_), (M_), (N_), (K_), (tA_), (tB_), (acc_), t->stream))
 
+/* C (+)= alpha * product; K cut into runs through the trainer's scratch when the shape gains from it */
+#define GEMM_SCALED(A_, B_, C_, M_, N_, K_, tA_, tB_, acc_, alpha_)                                    \
+    OP("gemm_scaled", 2.0 * (double)(M_) * (double)(N_) * (double)(K_), 0.0,                           \
+       seraph_gemm_scaled((A_), (B_), (C_), (M_), (N_), (K_), (tA_), (tB_), (acc_), (alpha_), t->ws, t->ws_bytes, t->stream))
+
 
 /* ------------------------------------------------------------------ layouts */
 static void make_layouts(hip_trainer_t* t) {
@@ -305,6 +310,16 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
     }
     t->ws_bytes = max_sz(seraph_rmsnorm_backward_ws_bytes(max_tokens, cfg->hidden),
                          seraph_embedding_backward_ws_bytes(max_tokens, cfg->vocab));
+    if (cfg->lora_rank > 0) {                               /* the rank-sized products, K cut into runs */
+        const int64_t Tm = max_tokens, r = cfg->lora_rank, wide = (int64_t)cfg->heads * cfg->head_dim;
+        const int64_t dims[3] = {cfg->hidden, wide, cfg->ffn};
+        for (int i = 0; i < 3; i++) {
+            t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(Tm, r, dims[i], 0, 1));
+            t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(Tm, r, dims[i], 0, 0));
+            t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(dims[i], r, Tm, 1, 0));
+            t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(r, dims[i], Tm, 1, 0));
+        }
+    }
     if (dev_alloc(t, &t->ws, t->ws_bytes)) goto fail;
     if (seraph_hip_host_alloc((void**)&t->h_stage, ((size_t)2 * max_tokens + max_batch + 1) * 4) != SERAPH_OK) goto fail;
     if (seraph_hip_stream_sync(t->stream) != SERAPH_OK) goto fail;
@@ -417,8 +432,7 @@ static int lora_forward_add(hip_trainer_t* t, const float* x, float* out, const 
                             int64_t T, int64_t in, int64_t outd) {
     const int r = t->cfg.lora_rank;
     const float s = t->cfg.lora_alpha / (float)r;
-    GEMM(x, A, t->lora_tmp, T, r, in, 0, 1, 0);
-    OP("scale", 0.0, 8.0 * (double)(T * r), seraph_scale(t->lora_tmp, (size_t)(T * r), s, t->stream));
+    GEMM_SCALED(x, A, t->lora_tmp, T, r, in, 0, 1, 0, s);
     GEMM(t->lora_tmp, B, out, T, outd, r, 0, 1, 1);
     return 0;
 }
@@ -428,12 +442,10 @@ static int lora_backward(hip_trainer_t* t, const float* dY, const float* x, cons
                          float* gA, float* gB, int64_t T, int64_t in, int64_t outd) {
     const int r = t->cfg.lora_rank;
     const float s = t->cfg.lora_alpha / (float)r;
-    GEMM(x, A, t->lora_tmp, T, r, in, 0, 1, 0);
-    OP("scale", 0.0, 8.0 * (double)(T * r), seraph_scale(t->lora_tmp, (size_t)(T * r), s, t->stream));
-    GEMM(dY, t->lora_tmp, gB, outd, r, T, 1, 0, 1);
-    GEMM(dY, B, t->lora_tmp, T, r, outd, 0, 0, 0);
-    OP("scale", 0.0, 8.0 * (double)(T * r), seraph_scale(t->lora_tmp, (size_t)(T * r), s, t->stream));
-    GEMM(t->lora_tmp, x, gA, r, in, T, 1, 0, 1);
+    GEMM_SCALED(x, A, t->lora_tmp, T, r, in, 0, 1, 0, s);
+    GEMM_SCALED(dY, t->lora_tmp, gB, outd, r, T, 1, 0, 1, 1.0f);
+    GEMM_SCALED(dY, B, t->lora_tmp, T, r, outd, 0, 0, 0, s);
+    GEMM_SCALED(t->lora_tmp, x, gA, r, in, T, 1, 0, 1, 1.0f);
     return 0;
 }
 

@@ -145,6 +145,39 @@ def test_gemm_forms(ops, orc, tA, tB, M, N, K):
     parity(out, orc.matmul(A, B, M, N, K, tA, tB, C0), "gemm accumulate", atol=1e-4)
 
 
+@pytest.mark.parametrize("tA,tB,M,N,K", [(0, 1, 2048, 16, 2048), (0, 0, 2048, 16, 1024), (1, 0, 2048, 16, 2048),
+                                          (1, 0, 16, 2048, 2048), (1, 0, 8, 1024, 4096), (0, 1, 300, 20, 1000),
+                                          (0, 1, 64, 64, 64)])
+@pytest.mark.parametrize("scratch", [True, False])
+def test_gemm_scaled(ops, orc, tA, tB, M, N, K, scratch):
+    """alpha * product, also accumulated, with K cut into runs (scratch) and as product + scale (no scratch)."""
+    r = rng(M + 3 * N + 5 * K + tA)
+    A = r.standard_normal((K, M) if tA else (M, K)).astype(np.float32)
+    B = r.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+    C0 = r.standard_normal((M, N)).astype(np.float32)
+    ref = orc.matmul(A, B, M, N, K, tA, tB)
+    got = ops.gemm_scaled(dev(A), dev(B), M, N, K, tA, tB, alpha=2.0, scratch=scratch)
+    parity(got, 2.0 * ref, "gemm_scaled", atol=2e-4)
+    again = ops.gemm_scaled(dev(A), dev(B), M, N, K, tA, tB, alpha=2.0, scratch=scratch)
+    assert torch.equal(got, again)                                        # fixed summation order
+    out = dev(C0)
+    ops.gemm_scaled(dev(A), dev(B), M, N, K, tA, tB, out=out, accumulate=True, alpha=1.0, scratch=scratch)
+    parity(out, orc.matmul(A, B, M, N, K, tA, tB, C0), "gemm_scaled accumulate", atol=1e-4)
+
+
+@pytest.mark.parametrize("M,N,K", [(2048, 2048, 16), (2048, 1024, 16), (333, 512, 8), (4100, 260, 32), (64, 1024, 4)])
+def test_gemm_small_k(ops, orc, M, N, K):
+    """C (+)= A B^T with a rank-sized K: the kernel without matrix instructions."""
+    r = rng(M + N + K)
+    A = r.standard_normal((M, K)).astype(np.float32)
+    B = r.standard_normal((N, K)).astype(np.float32)
+    C0 = r.standard_normal((M, N)).astype(np.float32)
+    parity(ops.gemm(dev(A), dev(B), M, N, K, 0, 1), orc.matmul(A, B, M, N, K, 0, 1), "small-K gemm")
+    out = dev(C0)
+    ops.gemm(dev(A), dev(B), M, N, K, 0, 1, out=out, accumulate=True)
+    parity(out, orc.matmul(A, B, M, N, K, 0, 1, C0), "small-K gemm accumulate")
+
+
 def test_gemm_reference_recipe_is_exact(ops):
     # tests/test_matmul.c:47-49 of the reference: 64^3, integers in [-5, 4]; exact in FP32
     r = rng(64)
