@@ -135,7 +135,7 @@ static void op_fold(hip_trainer_t* t) {
 /* GEMM through the kernel library, classed by the kernel instantiation that will run */
 #define GEMM(A_, B_, C_, M_, N_, K_, tA_, tB_, acc_)                                                   \
     OP(seraph_gemm_kernel_name((M_), (N_), (K_), (tA_), (tB_)), 2.0 * (double)(M_) * (double)(N_) * (double)(K_), 0.0, \
-       seraph_gemm((A_), (B_), (C_), (M_), (N_), (K_), (tA_), (tB_), (acc_), t->stream))
+       seraph_gemm_scaled((A_), (B_), (C_), (M_), (N_), (K_), (tA_), (tB_), (acc_), 1.0f, t->ws, t->ws_bytes, t->stream))
 
 /* C (+)= alpha * product; K cut into runs through the trainer's scratch when the shape gains from it */
 #define GEMM_SCALED(A_, B_, C_, M_, N_, K_, tA_, tB_, acc_, alpha_)                                    \
@@ -310,14 +310,21 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
     }
     t->ws_bytes = max_sz(seraph_rmsnorm_backward_ws_bytes(max_tokens, cfg->hidden),
                          seraph_embedding_backward_ws_bytes(max_tokens, cfg->vocab));
-    if (cfg->lora_rank > 0) {                               /* the rank-sized products, K cut into runs */
+    {
+        /* products with a small output and K = tokens (narrow weight gradients, the rank-sized LoRA products) run
+         * with K cut into runs through the same scratch; a call whose scratch is too small falls back by itself */
         const int64_t Tm = max_tokens, r = cfg->lora_rank, wide = (int64_t)cfg->heads * cfg->head_dim;
-        const int64_t dims[3] = {cfg->hidden, wide, cfg->ffn};
-        for (int i = 0; i < 3; i++) {
-            t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(Tm, r, dims[i], 0, 1));
-            t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(Tm, r, dims[i], 0, 0));
-            t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(dims[i], r, Tm, 1, 0));
-            t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(r, dims[i], Tm, 1, 0));
+        const int64_t kvw = (int64_t)cfg->kv_heads * cfg->head_dim;
+        const int64_t dims[4] = {cfg->hidden, wide, cfg->ffn, kvw};
+        for (int i = 0; i < 4; i++) {
+            if (r > 0) {
+                t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(Tm, r, dims[i], 0, 1));
+                t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(Tm, r, dims[i], 0, 0));
+                t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(dims[i], r, Tm, 1, 0));
+                t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(r, dims[i], Tm, 1, 0));
+            } else {
+                for (int j = 0; j < 4; j++) t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(dims[i], dims[j], Tm, 1, 0));
+            }
         }
     }
     if (dev_alloc(t, &t->ws, t->ws_bytes)) goto fail;
