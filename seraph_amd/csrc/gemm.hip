@@ -228,11 +228,11 @@ __device__ __forceinline__ T* scalar_ptr(T* p) {
     return reinterpret_cast<T*>(((uint64_t)hi << 32) | lo);
 }
 
-template <int TILE, bool KC>
+template <int TILE, bool KC, int NSET = 2>
 struct FastLoader {
     static constexpr int kSlots = TILE * kBK / 4 / kGemmThreads;
     uint32_t off[kSlots];                                  // byte offsets
-    float4 r[2][kSlots];                                   // two tiles in flight
+    float4 r[NSET][kSlots];                                // NSET tiles in flight
 
     // offsets relative to the tile origin (KC: P + mn0*ld + k0, else P + k0*ld + mn0)
     __device__ __forceinline__ void init(int64_t ld, int64_t mn0, int64_t mn_total) {
@@ -491,8 +491,11 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_kernel(c
 #pragma unroll
     for (int v = 0; v < 16; v++) acc[v] = 0.0f;
 
-    FastLoader<BT, A_KC> la;
-    FastLoader<BT, B_KC> lb;
+    // Four stages of both operands in flight (two float4 per lane and stage): with one or two workgroups per
+    // CU nothing else hides the memory latency, and two stages ahead is less than one round trip.
+    constexpr int R = 4;
+    FastLoader<BT, A_KC, R> la;
+    FastLoader<BT, B_KC, R> lb;
     la.init(lda, m0, M);
     lb.init(ldb, n0, N);
     const int64_t k_run = K / slices, k0 = (int64_t)blockIdx.y * k_run;          // whole stages: the launcher sees to it
@@ -504,21 +507,24 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_kernel(c
     const int fa_off = A_KC ? r * (kBK + kPadK) + 8 * wave + 4 * h : (8 * wave + 4 * h) * (BT + kPadM) + r;
     const int fb_off = B_KC ? r * (kBK + kPadK) + 8 * wave + 4 * h : (8 * wave + 4 * h) * (BT + kPadM) + r;
 
-    la.template load<0>(ta);
-    lb.template load<0>(tb);
+    // stage i of the run sits in register set i % R; past the last stage the last one is simply requested again
+    la.template load<0>(ta); lb.template load<0>(tb);
     if (nk > 1) { ta += step_a; tb += step_b; }
-    la.template load<1>(ta);
-    lb.template load<1>(tb);
+    la.template load<1>(ta); lb.template load<1>(tb);
     if (nk > 2) { ta += step_a; tb += step_b; }
+    la.template load<2>(ta); lb.template load<2>(tb);
+    if (nk > 3) { ta += step_a; tb += step_b; }
+    la.template load<3>(ta); lb.template load<3>(tb);
+    if (nk > 4) { ta += step_a; tb += step_b; }
     la.template store<0>(lds_a[0]);
     lb.template store<0>(lds_b[0]);
     __syncthreads();
 
-    auto stage = [&](auto parity, int kt) {
-        constexpr int CUR = decltype(parity)::value;
-        la.template load<CUR>(ta);
-        lb.template load<CUR>(tb);
-        const bool adv = kt + 3 < nk;
+    auto stage = [&](auto set, int kt) {
+        constexpr int SET = decltype(set)::value, CUR = SET & 1;       // R is even: the LDS buffer follows the set's parity
+        la.template load<SET>(ta);                                     // stage kt + R; set SET went to LDS a stage ago
+        lb.template load<SET>(tb);
+        const bool adv = kt + R + 1 < nk;
         ta += adv ? step_a : 0;
         tb += adv ? step_b : 0;
         float fa[4], fb[4];
@@ -538,16 +544,20 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_kernel(c
         }
 #pragma unroll
         for (int q = 0; q < 4; q++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[q], fb[q], acc, 0, 0, 0);
-        la.template store<CUR ^ 1>(lds_a[CUR ^ 1]);
-        lb.template store<CUR ^ 1>(lds_b[CUR ^ 1]);
+        la.template store<(SET + 1) % R>(lds_a[CUR ^ 1]);
+        lb.template store<(SET + 1) % R>(lds_b[CUR ^ 1]);
         __syncthreads();
     };
     int kt = 0;
-    for (; kt + 1 < nk; kt += 2) {
+    for (; kt + 3 < nk; kt += 4) {
         stage(std::integral_constant<int, 0>{}, kt);
         stage(std::integral_constant<int, 1>{}, kt + 1);
+        stage(std::integral_constant<int, 2>{}, kt + 2);
+        stage(std::integral_constant<int, 3>{}, kt + 3);
     }
     if (kt < nk) stage(std::integral_constant<int, 0>{}, kt);
+    if (kt + 1 < nk) stage(std::integral_constant<int, 1>{}, kt + 1);
+    if (kt + 2 < nk) stage(std::integral_constant<int, 2>{}, kt + 2);
 
     // fixed-order sum of the four partial tiles
 #pragma unroll
