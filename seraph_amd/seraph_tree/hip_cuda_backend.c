@@ -387,7 +387,11 @@ static void gemm_op(cuda_train_context_t* ctx, const char* label, const float* A
     if (!st) return;
     char name[80];
     snprintf(name, sizeof(name), "%s [%dx%d K=%d]%s", label, M, N, K, acc ? " +=" : "");
-    RUN(st, name, (size_t)2 * (size_t)M * (size_t)N * (size_t)K, 0, seraph_gemm(A, B, C, M, N, K, tA, tB, acc, st->stream));
+    /* a small output with a long K runs in slices of K through the scratch; other shapes are the plain product */
+    const size_t need = seraph_gemm_scaled_ws_bytes(M, N, K, tA, tB);
+    void* ws = need ? scratch(st, need) : NULL;
+    RUN(st, name, (size_t)2 * (size_t)M * (size_t)N * (size_t)K, 0,
+        seraph_gemm_scaled(A, B, C, M, N, K, tA, tB, acc, 1.0f, ws, ws ? need : 0, st->stream));
 }
 
 void cuda_train_matmul(cuda_train_context_t* ctx, cuda_buffer_t* A, cuda_buffer_t* B, cuda_buffer_t* C, int M, int N, int K) {

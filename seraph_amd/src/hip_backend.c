@@ -272,17 +272,26 @@ void vulkan_nan_check(vulkan_context_t* ctx, vulkan_buffer_t* input, size_t coun
 }
 
 /* ------------------------------------------------------------------ forward ops */
+/* A small output with a long K (narrow weight gradients, rank-sized LoRA products) is computed in runs of K
+ * through the context's scratch; every other shape is the plain product. */
+static void backend_gemm(vulkan_context_t* ctx, hip_state_t* st, const char* what, const float* A, const float* B, float* C,
+                         int M, int N, int K, int tA, int tB, int accumulate) {
+    const size_t need = seraph_gemm_scaled_ws_bytes(M, N, K, tA, tB);
+    void* ws = need ? hip_backend_scratch(ctx, need) : NULL;
+    HIP_OP(ctx, what, seraph_gemm_scaled(A, B, C, M, N, K, tA, tB, accumulate, 1.0f, ws, ws ? need : 0, st->stream));
+}
+
 void vulkan_matmul(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C, int M, int N, int K) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !A || !B || !C) return;
-    HIP_OP(ctx, "matmul", seraph_gemm(FPTR(A), FPTR(B), FPTR(C), M, N, K, 0, 0, 0, st->stream));
+    backend_gemm(ctx, st, "matmul", FPTR(A), FPTR(B), FPTR(C), M, N, K, 0, 0, 0);
 }
 
 void vulkan_matmul_transpose(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C,
                              int M, int N, int K, int transpose_A, int transpose_B, int accumulate) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !A || !B || !C) return;
-    HIP_OP(ctx, "matmul_transpose", seraph_gemm(FPTR(A), FPTR(B), FPTR(C), M, N, K, transpose_A, transpose_B, accumulate, st->stream));
+    backend_gemm(ctx, st, "matmul_transpose", FPTR(A), FPTR(B), FPTR(C), M, N, K, transpose_A, transpose_B, accumulate);
 }
 
 void vulkan_add(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C, size_t count) {
