@@ -307,7 +307,8 @@ def test_adamw(ops, orc, n, clip):
 
 # ------------------------------------------------------------------ attention
 ATTN_CASES = [([0, 200], 4, 4, 64), ([0, 5, 6, 133, 300], 4, 2, 32), ([0, 257], 4, 2, 128), ([0, 128, 256], 2, 1, 64),
-              ([0, 1], 2, 2, 64), ([0, 31, 64, 97, 161], 8, 2, 128)]
+              ([0, 1], 2, 2, 64), ([0, 31, 64, 97, 161], 8, 2, 128),
+              ([0, 40, 40, 100, 100], 4, 2, 64)]          # empty sequences in the middle and at the end
 
 
 def _attn_inputs(seed, starts, H, KVH, D):
