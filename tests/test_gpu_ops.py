@@ -115,15 +115,17 @@ def test_cross_entropy_grad(ops, orc, rows, cols):
     assert (host(g0) == 0).all()
 
 
-def test_cross_entropy_grad_packed(ops, orc):
+@pytest.mark.parametrize("starts,dead", [([0, 3, 4, 20], (2, 3, 19)), ([0, 3, 3, 4, 20, 20], (2, 3, 19))])
+def test_cross_entropy_grad_packed(ops, orc, starts, dead):
+    """The last token of every sequence has no target; empty sequences change nothing."""
     r = rng(11)
-    starts = np.array([0, 3, 4, 20], np.uint32)
+    starts = np.array(starts, np.uint32)
     x = r.standard_normal((20, 8192)).astype(np.float32)
     t = r.integers(0, 8192, 20).astype(np.uint32)
     rg, rl = orc.cross_entropy_grad_packed(x, t, starts, 17)
     g, l = ops.cross_entropy_grad(dev(x), dev(t.view(np.int32)), 17, seq_starts=dev(starts.view(np.int32)))
     parity(g, rg, "packed grad", atol=1e-7); parity(l, rl, "packed loss")
-    for last in (2, 3, 19):
+    for last in dead:
         assert (host(g)[last] == 0).all() and host(l)[last] == 0
 
 
@@ -238,7 +240,7 @@ def test_qk_norm(ops, orc):
 
 # ------------------------------------------------------------------ rope
 @pytest.mark.parametrize("heads,D,theta,starts", [(8, 64, 10000.0, [0, 256, 300]), (16, 128, 1e6, [0, 4096]),
-                                                  (3, 16, 10000.0, [0, 1, 2, 50])])
+                                                  (3, 16, 10000.0, [0, 1, 2, 50]), (4, 64, 10000.0, [0, 7, 7, 40, 40])])
 def test_rope_forward_backward(ops, orc, heads, D, theta, starts):
     r = rng(heads * D)
     T = starts[-1]
