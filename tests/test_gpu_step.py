@@ -67,6 +67,8 @@ CASES = [
     dict(hidden=64, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=96, vocab=101, starts=[0, 33, 34, 70]),
     dict(hidden=128, layers=1, heads=2, kv_heads=2, head_dim=64, ffn=256, vocab=300, starts=[0, 150]),
     dict(hidden=256, layers=2, heads=2, kv_heads=1, head_dim=128, ffn=128, vocab=64, starts=[0, 40, 100, 129]),
+    # 512 tokens: the weight gradients are small outputs with a long K and run as sums over runs of K
+    dict(hidden=128, layers=1, heads=2, kv_heads=2, head_dim=64, ffn=256, vocab=300, starts=[0, 200, 512]),
 ]
 
 
