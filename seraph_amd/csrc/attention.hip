@@ -528,7 +528,8 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
     // written twice: with the per-wave test for those, and as straight-line code for the rest, where
     // every wave works.  (A conditional around the accumulating matrix instructions in the main
     // loop makes the compiler shuttle the 128 dK/dV accumulator registers in and out of the
-    // accumulation register file on every iteration.)
+    // accumulation register file on every iteration.)  `iteration` below is the copy with the test; the
+    // straight-line iterations run `iteration1` (one sub-tile) or `iteration2` (two), which are pipelined.
     const bool wave_has_keys = jw0 < T;
     auto iteration = [&](int hg, int n, int li, int hg2, int n2, auto may_skip) {
         const int cur = li & 1;
