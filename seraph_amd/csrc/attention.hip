@@ -531,7 +531,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
     // accumulation register file on every iteration.)  `iteration` below is the copy with the test; the
     // straight-line iterations run `iteration1` (one sub-tile) or `iteration2` (two), which are pipelined.
     const bool wave_has_keys = jw0 < T;
-    auto iteration = [&](int hg, int n, int li, int hg2, int n2, auto may_skip) {
+    auto iteration = [&](int hg, int n, int li, int hg2, int n2) {
         const int cur = li & 1;
         // No branch around the loads and the LDS staging: past the last tile the same tile is simply
         // fetched and staged again.  (Loads and stores share one in-order counter; behind a branch the
@@ -542,7 +542,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
         for (int qb = 0; qb < QB; qb++) {
         const int64_t i0 = j0 + QR * (int64_t)n + 32 * qb;
         const int ro = 32 * qb;                                              // this sub-tile's first row in the staged tiles
-        if (!decltype(may_skip)::value || (i0 + 31 >= jw0 && wave_has_keys)) {   // some query of the tile can see this wave's keys
+        if (i0 + 31 >= jw0 && wave_has_keys) {                               // some query of the tile can see this wave's keys
             v16f s, dp;
 #pragma unroll
             for (int v = 0; v < 16; v++) { s[v] = 0.0f; dp[v] = 0.0f; }
@@ -609,13 +609,6 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
                     }
                 }
             }
-            if (!decltype(may_skip)::value && qb == 0) {
-                // Straight-line copy: stage the next tile now, ahead of the dS stores.  Loads and stores share
-                // one completion counter that the compiler must treat as unordered once both kinds are
-                // pending, so waiting for the tile's loads after the stores were issued would also wait
-                // for the stores.
-                tiles_store(cur ^ 1); stats_store(cur ^ 1);
-            }
             if (WRITE_DS) {
                 // dS tile (32 queries x 32 keys, row-major) for the dQ pass: band slot = query tile - key tile.
                 // A tile outside the band (it is all zeros: another sequence) goes to a spare tile behind the band.
@@ -668,7 +661,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
             }
         }
         }   // sub-tiles
-        if (decltype(may_skip)::value) { tiles_store(cur ^ 1); stats_store(cur ^ 1); }
+        tiles_store(cur ^ 1); stats_store(cur ^ 1);
         __syncthreads();
     };
     // The straight-line iteration for one sub-tile (head_dim 128), in four runs of matrix instructions that carry
@@ -969,7 +962,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
         for (int g = 0; g < G; g++) {
             int n = ((sub - g * nq) % split + split) % split;      // this item's first query tile of head g
             int g2, n2;
-            for (; n < ndiag; n += split, li++) { successor(g, n, g2, n2); iteration(g, n, li, g2, n2, std::true_type{}); }
+            for (; n < ndiag; n += split, li++) { successor(g, n, g2, n2); iteration(g, n, li, g2, n2); }
             for (; n < nq; n += split, li++) {
                 successor(g, n, g2, n2);
                 if constexpr (QB == 2) iteration2(g, n, li, g2, n2); else iteration1(g, n, li, g2, n2);
