@@ -197,6 +197,12 @@ void hip_qk_norm_backward(vulkan_context_t* ctx, vulkan_buffer_t* qk_pre, vulkan
 void hip_adamw_update_clipped(vulkan_context_t* ctx, vulkan_buffer_t* weight, vulkan_buffer_t* grad, vulkan_buffer_t* m,
                               vulkan_buffer_t* v, float lr, float beta1, float beta2, float weight_decay, float eps,
                               int step, size_t size, float clip);
+/* C (+)= alpha * op(A) op(B): vulkan_matmul_transpose followed by vulkan_scale of the product, the pair the
+ * LoRA path issues (src/train.c:5785-5792, :5815-5841), as one op.  accumulate with alpha != 1 is only possible
+ * for the shapes the library computes through its scratch (small output, long K); otherwise the op reports an
+ * error and leaves C untouched. */
+void hip_matmul_scaled(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C,
+                       int M, int N, int K, int transpose_A, int transpose_B, int accumulate, float alpha);
 /* number of ops whose kernel library call failed since init (errors are also printed to stderr) */
 int hip_backend_error_count(vulkan_context_t* ctx);
 

@@ -281,6 +281,16 @@ static void backend_gemm(vulkan_context_t* ctx, hip_state_t* st, const char* wha
     HIP_OP(ctx, what, seraph_gemm_scaled(A, B, C, M, N, K, tA, tB, accumulate, 1.0f, ws, ws ? need : 0, st->stream));
 }
 
+void hip_matmul_scaled(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C,
+                       int M, int N, int K, int transpose_A, int transpose_B, int accumulate, float alpha) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !A || !B || !C) return;
+    const size_t need = seraph_gemm_scaled_ws_bytes(M, N, K, transpose_A, transpose_B);
+    void* ws = need ? hip_backend_scratch(ctx, need) : NULL;
+    HIP_OP(ctx, "matmul_scaled", seraph_gemm_scaled(FPTR(A), FPTR(B), FPTR(C), M, N, K, transpose_A, transpose_B, accumulate, alpha,
+                                                    ws, ws ? need : 0, st->stream));
+}
+
 void vulkan_matmul(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C, int M, int N, int K) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !A || !B || !C) return;

@@ -149,3 +149,36 @@ def test_loss_chain_and_adamw(vk, orc):
     rw, rm, rv = orc.adamw(w, g, z, z, 3.14e-4, 0.9, 0.999, 0.01, 1e-8, 3)
     close(down(vk, bw, n), rw, atol=1e-7); close(down(vk, bm, n), rm, atol=1e-9); close(down(vk, bv, n), rv, atol=1e-12)
     assert lib.hip_backend_error_count(ctx) == 0
+
+
+def test_lora_products_through_the_backend(vk, orc):
+    """The LoRA adapter's forward the way src/train.c:5785-5792 issues it (product, scale, product into the
+    output), once with the reference's three ops and once with hip_matmul_scaled in place of the first two."""
+    lib, ctx = vk
+    r = rng(21)
+    T, d_in, d_out, rank, s = 512, 256, 192, 16, 2.0
+    x = r.standard_normal((T, d_in)).astype(np.float32)
+    A = (0.05 * r.standard_normal((rank, d_in))).astype(np.float32)
+    B = (0.05 * r.standard_normal((d_out, rank))).astype(np.float32)
+    y0 = r.standard_normal((T, d_out)).astype(np.float32)
+    tmp_ref = s * orc.matmul(x, A, T, rank, d_in, 0, 1)
+    ref = orc.matmul(tmp_ref.astype(np.float32), B, T, d_out, rank, 0, 1, y0)
+    bx, bA, bB = up(vk, x), up(vk, A), up(vk, B)
+    outs = []
+    for fused in (False, True):
+        btmp, by = up(vk, np.zeros((T, rank), np.float32)), up(vk, y0)
+        assert lib.vulkan_cmd_begin(ctx) == 1
+        if fused:
+            lib.hip_matmul_scaled(ctx, bx, bA, btmp, T, rank, d_in, 0, 1, 0, C.c_float(s))
+        else:
+            lib.vulkan_matmul_transpose(ctx, bx, bA, btmp, T, rank, d_in, 0, 1, 0)
+            lib.vulkan_scale(ctx, btmp, C.c_size_t(T * rank), C.c_float(s))
+        lib.vulkan_matmul_transpose(ctx, btmp, bB, by, T, d_out, rank, 0, 1, 1)
+        assert lib.vulkan_cmd_end_submit(ctx) == 1
+        close(down(vk, btmp, (T, rank)), tmp_ref)
+        outs.append(down(vk, by, (T, d_out)))
+        close(outs[-1], ref)
+        lib.vulkan_buffer_free(ctx, btmp); lib.vulkan_buffer_free(ctx, by)
+    for b in (bx, bA, bB):
+        lib.vulkan_buffer_free(ctx, b)
+    assert lib.hip_backend_error_count(ctx) == 0
