@@ -1186,32 +1186,36 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dq_k
 // query tile, key tile) in a band of ds_slots key tiles below the diagonal.  dQ = scale dS K is
 // then a single product per tile and the backward executes 5 products instead of 7.
 // grid: persistent over (128-query tiles, heads); wave w owns queries i0+32w .. +31.
-template <int D>
+// KSPLIT (short batches, as in the forward kernel): 64-query items; waves 0,1 take the even key tiles, waves 2,3 the
+// odd ones of the same queries, two key tiles are staged per iteration and the two partial dQ meet in LDS.
+template <int D, bool KSPLIT>
 __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const float* __restrict__ K, const float* __restrict__ DS,
                                                                          float* __restrict__ dQ, const uint32_t* __restrict__ seq_starts,
                                                                          int batch, int64_t T, int H, int KVH, float scale, int ds_slots,
                                                                          unsigned int* __restrict__ queue) {
     constexpr int LD = D + 4, DB = D / 32;
-    __shared__ __attribute__((aligned(16))) float sK[2][32 * LD];
+    constexpr int KT = KSPLIT ? 2 : 1, QROWS = KSPLIT ? 64 : 128;
+    __shared__ __attribute__((aligned(16))) float sK[2][KT * 32 * LD];
     __shared__ uint32_t sSeq[kMaxSeqLds];
     __shared__ int sItem;
     const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
-    const int nqt = (int)((T + 127) / 128);
+    const int nqt = (int)((T + QROWS - 1) / QROWS);
     const int64_t nqt32 = (T + 31) >> 5;
     const TileQueue tq_{queue, &sItem, nqt * H};
     __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
     const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, [&](int q) {
-        const int64_t a = (int64_t)q * 128, z = (a + 127 < T - 1) ? a + 127 : T - 1;
+        const int64_t a = (int64_t)q * QROWS, z = (a + QROWS - 1 < T - 1) ? a + QROWS - 1 : T - 1;
         return (int)((z + 1 - (seqs.start_of((int)a) / 32) * 32 + 31) / 32);
     });
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
+    const int wq = KSPLIT ? (w & 1) : w, kp = KSPLIT ? (w >> 1) : 0;  // the wave's 32 queries within the item; its key-tile parity
     for (int item = tq_.next(); item >= 0; item = tq_.next()) {
     const int head = item % H, kvh = head / (H / KVH);
-    const int qt128 = by_len(item / H);
-    const int64_t i0 = (int64_t)qt128 * 128;
-    const int64_t iw0 = i0 + 32 * w;
+    const int qtile = by_len(item / H);
+    const int64_t i0 = (int64_t)qtile * QROWS;
+    const int64_t iw0 = i0 + 32 * wq;
     const int64_t qw = (int64_t)H * D, kw = (int64_t)KVH * D;
-    const int64_t i_last = (i0 + 127 < T - 1) ? i0 + 127 : T - 1;
+    const int64_t i_last = (i0 + QROWS - 1 < T - 1) ? i0 + QROWS - 1 : T - 1;
     const int64_t jbeg = (seqs.start_of((int)i0) / 32) * 32;
     const int ntiles = (int)((i_last + 1 - jbeg + 31) / 32);
     // this wave's own range of key tiles (relative to jbeg): from the tile holding the start of its
@@ -1243,38 +1247,70 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const f
         for (int s8 = 0; s8 < 4; s8++) dsf[buf][s8] = *reinterpret_cast<const float4*>(tile + 8 * s8);
     };
 
-    Tile32<D> tk;
-    tk.gload(K, jbeg, T, kw, kvh * D);
-    ds_load(0, 0);
-    tk.sstore(sK[0]);
+    Tile32<D> tk[KT];
+    auto k_load = [&](int t0) {                                // tiles t0 .. t0+KT-1; rows past the last token read as zeros
+#pragma unroll
+        for (int u = 0; u < KT; u++) tk[u].gload(K, jbeg + 32 * (int64_t)(t0 + u), T, kw, kvh * D);
+    };
+    auto k_store = [&](int buf) {
+#pragma unroll
+        for (int u = 0; u < KT; u++) tk[u].sstore(sK[buf] + u * 32 * LD);
+    };
+    k_load(0);
+    ds_load(kp, 0);
+    k_store(0);
     __syncthreads();
 
-    auto body = [&](auto parity, int t) {
+    // tp = first of the KT staged tiles; this wave's tile is tp + kp
+    auto body = [&](auto parity, int tp) {
         constexpr int CUR = decltype(parity)::value;          // register and LDS buffers by compile-time parity
-        if (t + 1 < ntiles) tk.gload(K, jbeg + 32 * (int64_t)(t + 1), T, kw, kvh * D);
-        ds_load(t + 1 < ntiles ? t + 1 : t, CUR ^ 1);
+        const int t = tp + kp;
+        const float* sKt = sK[CUR] + kp * 32 * LD;
+        if (tp + KT < ntiles) k_load(tp + KT);
+        ds_load(t + KT, CUR ^ 1);                               // clamped into the wave's range inside
         if (t >= tb && t <= te) {
 #pragma unroll
             for (int s8 = 0; s8 < 4; s8++) {
                 const float e[4] = {dsf[CUR][s8].x, dsf[CUR][s8].y, dsf[CUR][s8].z, dsf[CUR][s8].w};
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const DVec<DB> kk = lds_dvec<DB>(&sK[CUR][(8 * s8 + 4 * h + q) * LD], r);
+                    const DVec<DB> kk = lds_dvec<DB>(&sKt[(8 * s8 + 4 * h + q) * LD], r);
 #pragma unroll
                     for (int db = 0; db < DB; db++) dq[db] = mfma(e[q], kk.v[db], dq[db]);
                 }
             }
         }
-        if (t + 1 < ntiles) tk.sstore(sK[CUR ^ 1]);
+        if (tp + KT < ntiles) k_store(CUR ^ 1);
         __syncthreads();
     };
-    int t = 0;
-    for (; t + 1 < ntiles; t += 2) {
-        body(std::integral_constant<int, 0>{}, t);
-        body(std::integral_constant<int, 1>{}, t + 1);
+    int tp = 0;
+    for (; tp + KT < ntiles; tp += 2 * KT) {
+        body(std::integral_constant<int, 0>{}, tp);
+        body(std::integral_constant<int, 1>{}, tp + KT);
     }
-    if (t < ntiles) body(std::integral_constant<int, 0>{}, t);
+    if (tp < ntiles) body(std::integral_constant<int, 0>{}, tp);
 
+    if (KSPLIT) {
+        // waves 2,3 hand their partial dQ to waves 0,1 through the tile buffers (nobody reads them any more; the
+        // next item restages them only behind the queue's barriers)
+        float* xo = &sK[0][0] + (size_t)wq * DB * 16 * 64;
+        static_assert(!KSPLIT || 2 * KT * 32 * LD >= 2 * DB * 16 * 64, "tile buffers too small for the exchange");
+        if (kp == 1) {
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) xo[(db * 16 + v) * 64 + lane] = dq[db][v];
+        }
+        __syncthreads();
+        if (kp == 0) {
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) dq[db][v] += xo[(db * 16 + v) * 64 + lane];
+        }
+    }
+
+    if (kp == 0)
 #pragma unroll
     for (int v = 0; v < 16; v++) {
         const int64_t i = iw0 + acc_row(v, h);
@@ -1403,8 +1439,13 @@ static int run_backward(const float* Q, const float* K, const float* V, const fl
     }
     SERAPH_LAUNCH_CHECK();
     if (ds) {
-        dim3 gds((unsigned)std::min<int64_t>(ceil_div(T, 128) * H, (int64_t)num_compute_units() * 2));
-        hipLaunchKernelGGL(attn_bwd_dq_ds_kernel<D>, gds, dim3(kAttnThreads), 0, st, K, ds, dQ, seq_starts, batch, T, H, KVH, scale, ds_slots, qq);
+        if (ceil_div(T, 128) * H <= 2 * (int64_t)num_compute_units()) {        // short batch: see run_forward
+            dim3 gds((unsigned)std::min<int64_t>(ceil_div(T, 64) * H, (int64_t)num_compute_units() * 2));
+            hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<D, true>), gds, dim3(kAttnThreads), 0, st, K, ds, dQ, seq_starts, batch, T, H, KVH, scale, ds_slots, qq);
+        } else {
+            dim3 gds((unsigned)std::min<int64_t>(ceil_div(T, 128) * H, (int64_t)num_compute_units() * 2));
+            hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<D, false>), gds, dim3(kAttnThreads), 0, st, K, ds, dQ, seq_starts, batch, T, H, KVH, scale, ds_slots, qq);
+        }
     } else {
         hipLaunchKernelGGL(attn_bwd_dq_kernel<D>, gq, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dQ, seq_starts, batch,
                            T, H, KVH, scale, scale * kLog2e, qq);
