@@ -161,6 +161,12 @@ int seraph_rmsnorm(const float* x, const float* scale, float* y, int64_t rows, i
 size_t seraph_rmsnorm_backward_ws_bytes(int64_t rows, int64_t cols);
 int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy, float* dx, float* grad_scale,
                             int64_t rows, int64_t cols, float eps, void* ws, size_t ws_bytes, seraph_stream_t s);
+/* The same with dx = residual + (the RMSNorm input gradient): the vulkan_add that follows every
+ * vulkan_rmsnorm_backward_batch of a layer (src/train.c:5180-5193, :5342-5355) folded into the store.
+ * residual may be dx itself (in place) or NULL (then it is seraph_rmsnorm_backward). */
+int seraph_rmsnorm_backward_residual(const float* x, const float* scale, const float* dy, const float* residual, float* dx,
+                                     float* grad_scale, int64_t rows, int64_t cols, float eps, void* ws, size_t ws_bytes,
+                                     seraph_stream_t s);
 /* vulkan_rope / vulkan_rope_backward, include/vulkan_backend.h:493-495,561-563
  * (shaders/rope.comp, rope_backward.comp:26-59) and the packed forms
  * (include/cuda_train_context.h:275,286).  in and out may alias.  backward != 0 applies

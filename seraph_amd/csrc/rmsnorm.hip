@@ -91,7 +91,8 @@ template <int VPL>
 __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const float* __restrict__ x,
                                                              const float* __restrict__ scale,
                                                              const float* __restrict__ dy,
-                                                             float* __restrict__ dx,
+                                                             const float* res,              // NULL, or added to dx (may be dx itself)
+                                                             float* dx,
                                                              float* __restrict__ partial,   // [gridDim.x, cols]
                                                              int64_t rows, int cols, float eps) {
     extern __shared__ float lds[];                        // [kWavesPerBlock, cols]
@@ -112,12 +113,13 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const float* __rest
     for (int64_t row = wave; row < rows; row += nwaves) {
         const float4* xr = reinterpret_cast<const float4*>(x + row * cols);
         const float4* gr = reinterpret_cast<const float4*>(dy + row * cols);
-        float4 xv[VPL], gv[VPL];
+        float4 xv[VPL], gv[VPL], rv[VPL];
 #pragma unroll
         for (int k = 0; k < VPL; k++) {
             int i4 = lane + 64 * k;
             xv[k] = i4 < n4 ? xr[i4] : make_float4(0, 0, 0, 0);
             gv[k] = i4 < n4 ? gr[i4] : make_float4(0, 0, 0, 0);
+            rv[k] = (res && i4 < n4) ? reinterpret_cast<const float4*>(res + row * cols)[i4] : make_float4(0, 0, 0, 0);
         }
         double ssq = 0.0, cp = 0.0;
 #pragma unroll
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const float* __rest
                 acc[e] += (float)(gd * xd * st.inv);                                 // :90
                 o[e] = (float)(gd * (double)s[e] * st.inv - xd * st.k);              // :98
             }
-            if (i4 < n4) dr[i4] = make_float4(o[0], o[1], o[2], o[3]);
+            if (i4 < n4) dr[i4] = make_float4(rv[k].x + o[0], rv[k].y + o[1], rv[k].z + o[2], rv[k].w + o[3]);
         }
     }
 
@@ -186,7 +188,8 @@ template <int VPL, bool PREFETCH = false, bool NT = true>
 __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_block_kernel(const float* __restrict__ x,
                                                                    const float* __restrict__ scale,
                                                                    const float* __restrict__ dy,
-                                                                   float* __restrict__ dx,
+                                                                   const float* res,              // NULL, or added to dx (may be dx itself)
+                                                                   float* dx,
                                                                    float* __restrict__ partial,   // [gridDim.x, cols]
                                                                    int64_t rows, int cols, float eps) {
     __shared__ double red[2][kWavesPerBlock][2];
@@ -199,23 +202,26 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_block_kernel(const float* 
         sc[k] = i4 < n4 ? reinterpret_cast<const float4*>(scale)[i4] : make_float4(0, 0, 0, 0);
         gs[k] = make_float4(0, 0, 0, 0);
     }
-    auto fetch = [&](int64_t row, float4 (&xv)[VPL], float4 (&gv)[VPL]) {
+    auto fetch = [&](int64_t row, float4 (&xv)[VPL], float4 (&gv)[VPL], float4 (&rv)[VPL]) {
         const float4* xr = reinterpret_cast<const float4*>(x + row * cols);
         const float4* gr = reinterpret_cast<const float4*>(dy + row * cols);
+        const float4* rr = reinterpret_cast<const float4*>(res + row * cols);
 #pragma unroll
         for (int k = 0; k < VPL; k++) {
             int i4 = threadIdx.x + kBlock * k;
             xv[k] = i4 < n4 ? (NT ? ldnt4(xr + i4) : xr[i4]) : make_float4(0, 0, 0, 0);
             gv[k] = i4 < n4 ? (NT ? ldnt4(gr + i4) : gr[i4]) : make_float4(0, 0, 0, 0);
+            rv[k] = (res && i4 < n4) ? (NT ? ldnt4(rr + i4) : rr[i4]) : make_float4(0, 0, 0, 0);
         }
     };
-    float4 xv[VPL], gv[VPL], xn[VPL], gn[VPL];
+    // a row's residual is read with the row (before that row of dx is written: in place is safe)
+    float4 xv[VPL], gv[VPL], rv[VPL], xn[VPL], gn[VPL], rn[VPL];
     int64_t row = blockIdx.x;
-    if (row < rows) fetch(row, xv, gv);
+    if (row < rows) fetch(row, xv, gv, rv);
     int it = 0;
     for (; row < rows; row += gridDim.x, it ^= 1) {
         const int64_t next = row + gridDim.x;
-        if (PREFETCH) { if (next < rows) fetch(next, xn, gn); }
+        if (PREFETCH) { if (next < rows) fetch(next, xn, gn, rn); }
         double ssq = 0.0, cp = 0.0;
 #pragma unroll
         for (int k = 0; k < VPL; k++) {
@@ -246,14 +252,15 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_block_kernel(const float* 
                 acc[e] += (float)(gd * xd * st.inv);                                 // :90
                 o[e] = (float)(gd * (double)s[e] * st.inv - xd * st.k);              // :98
             }
-            if (i4 < n4) { if (NT) stnt4(dr + i4, make_float4(o[0], o[1], o[2], o[3])); else dr[i4] = make_float4(o[0], o[1], o[2], o[3]); }
+            const float4 ov = make_float4(rv[k].x + o[0], rv[k].y + o[1], rv[k].z + o[2], rv[k].w + o[3]);
+            if (i4 < n4) { if (NT) stnt4(dr + i4, ov); else dr[i4] = ov; }
         }
         if (next < rows) {
             if (PREFETCH) {
 #pragma unroll
-                for (int k = 0; k < VPL; k++) { xv[k] = xn[k]; gv[k] = gn[k]; }
+                for (int k = 0; k < VPL; k++) { xv[k] = xn[k]; gv[k] = gn[k]; rv[k] = rn[k]; }
             } else {
-                fetch(next, xv, gv);
+                fetch(next, xv, gv, rv);
             }
         }
     }
@@ -268,7 +275,8 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_block_kernel(const float* 
 __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_generic_kernel(const float* __restrict__ x,
                                                                      const float* __restrict__ scale,
                                                                      const float* __restrict__ dy,
-                                                                     float* __restrict__ dx,
+                                                                     const float* res,              // NULL, or added to dx (may be dx itself)
+                                                                     float* dx,
                                                                      float* __restrict__ partial,   // [nwaves, cols], zeroed
                                                                      int64_t rows, int64_t cols, float eps) {
     const int lane = threadIdx.x & 63;
@@ -290,7 +298,8 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_generic_kernel(const float
         for (int64_t c = lane; c < cols; c += 64) {
             double xd = (double)xr[c], gd = (double)gr[c];
             mine[c] += (float)(gd * xd * st.inv);          // same lane revisits the same column: no race
-            dx[row * cols + c] = (float)(gd * (double)scale[c] * st.inv - xd * st.k);
+            const float o = (float)(gd * (double)scale[c] * st.inv - xd * st.k);
+            dx[row * cols + c] = res ? res[row * cols + c] + o : o;
         }
     }
 }
@@ -438,6 +447,13 @@ size_t seraph_rmsnorm_backward_ws_bytes(int64_t rows, int64_t cols) {
 
 int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy, float* dx, float* grad_scale,
                             int64_t rows, int64_t cols, float eps, void* ws, size_t ws_bytes, seraph_stream_t s) {
+    return seraph_rmsnorm_backward_residual(x, scale, dy, nullptr, dx, grad_scale, rows, cols, eps, ws, ws_bytes, s);
+}
+
+int seraph_rmsnorm_backward_residual(const float* x, const float* scale, const float* dy, const float* residual, float* dx,
+                                     float* grad_scale, int64_t rows, int64_t cols, float eps, void* ws, size_t ws_bytes,
+                                     seraph_stream_t s) {
+    const float* res = residual;
     if (rows == 0 || cols == 0) return SERAPH_OK;
     SERAPH_REQUIRE(x && scale && dy && dx && grad_scale, "rmsnorm_backward: NULL pointer");
     SERAPH_REQUIRE(rows > 0 && cols > 0, "rmsnorm_backward: bad shape");
@@ -447,14 +463,14 @@ int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy,
     }
     hipStream_t st = as_stream(s);
     float* partial = (float*)ws;
-    const bool aligned = aligned16(x) && aligned16(scale) && aligned16(dy) && aligned16(dx) && aligned16(ws);
+    const bool aligned = aligned16(x) && aligned16(scale) && aligned16(dy) && aligned16(dx) && aligned16(ws) && (!res || aligned16(res));
     const int bvpl = aligned ? pick_block_vpl(cols) : 0;
     const int wvpl = (aligned && !bvpl && cols <= 512) ? pick_vpl(cols) : 0;
     int nparts;
     if (bvpl) {
         const int grid = bwd_block_grid(rows);
         nparts = grid;
-#define BBWD(V) hipLaunchKernelGGL(rmsnorm_bwd_block_kernel<V>, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, dx, partial, rows, (int)cols, eps)
+#define BBWD(V) hipLaunchKernelGGL(rmsnorm_bwd_block_kernel<V>, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, res, dx, partial, rows, (int)cols, eps)
         switch (bvpl) {
             case 1: BBWD(1); break;
             case 2: BBWD(2); break;
@@ -466,7 +482,7 @@ int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy,
         const int grid = bwd_grid(rows);
         nparts = grid;
         const size_t lds = (size_t)kWavesPerBlock * cols * sizeof(float);
-#define BWD(V) hipLaunchKernelGGL(rmsnorm_bwd_kernel<V>, dim3(grid), dim3(kBlock), lds, st, x, scale, dy, dx, partial, rows, (int)cols, eps)
+#define BWD(V) hipLaunchKernelGGL(rmsnorm_bwd_kernel<V>, dim3(grid), dim3(kBlock), lds, st, x, scale, dy, res, dx, partial, rows, (int)cols, eps)
         if (wvpl == 1) BWD(1); else BWD(2);
 #undef BWD
     } else {
@@ -474,7 +490,7 @@ int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy,
         nparts = grid * kWavesPerBlock;
         int rc = seraph_fill_u32(partial, 0u, (size_t)nparts * cols, s);
         if (rc != SERAPH_OK) return rc;
-        hipLaunchKernelGGL(rmsnorm_bwd_generic_kernel, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, dx, partial, rows, cols, eps);
+        hipLaunchKernelGGL(rmsnorm_bwd_generic_kernel, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, res, dx, partial, rows, cols, eps);
     }
     SERAPH_LAUNCH_CHECK();
     hipLaunchKernelGGL(colsum_add_kernel, dim3((unsigned)ceil_div(cols, 64)), dim3(1024), 0, st,

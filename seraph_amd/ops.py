@@ -146,14 +146,20 @@ def rmsnorm(x, scale, eps):
     return y
 
 
-def rmsnorm_backward(x, scale, dy, eps, grad_scale=None):
-    dx = torch.empty_like(x)
+def rmsnorm_backward(x, scale, dy, eps, grad_scale=None, residual=None, out=None):
+    """residual: added to the input gradient as it is stored (out may be the residual itself)."""
+    dx = torch.empty_like(x) if out is None else out
     gs = torch.zeros_like(scale) if grad_scale is None else grad_scale
     rows, cols = x.shape
     nbytes = kernels().seraph_rmsnorm_backward_ws_bytes(i64(rows), i64(cols))
     ws = _workspace(nbytes)
-    check(kernels().seraph_rmsnorm_backward(_p(x), _p(scale), _p(dy), _p(dx), _p(gs), i64(rows), i64(cols), f32(eps),
-                                            _p(ws), sz(nbytes), _stream()), "rmsnorm_backward")
+    if residual is None:
+        check(kernels().seraph_rmsnorm_backward(_p(x), _p(scale), _p(dy), _p(dx), _p(gs), i64(rows), i64(cols), f32(eps),
+                                                _p(ws), sz(nbytes), _stream()), "rmsnorm_backward")
+    else:
+        check(kernels().seraph_rmsnorm_backward_residual(_p(x), _p(scale), _p(dy), _p(residual), _p(dx), _p(gs), i64(rows),
+                                                         i64(cols), f32(eps), _p(ws), sz(nbytes), _stream()),
+              "rmsnorm_backward_residual")
     return dx, gs
 
 

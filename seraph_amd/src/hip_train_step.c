@@ -635,9 +635,9 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         }
         GEMM(t->g_gate, W + t->L.gate, t->g_xn, T, h, f, 0, 0, 0);
         GEMM(t->g_up, W + t->L.up, t->g_xn, T, h, f, 0, 0, 1);
-        OP("rmsnorm_backward", 0.0, 12.0 * (double)(T * h), seraph_rmsnorm_backward(a->post_in, W + t->L.post_norm, t->g_xn, t->g_tmp,
+        /* the input gradient is added to the residual stream's gradient as it is stored (src/train.c:5180-5193) */
+        OP("rmsnorm_backward", 0.0, 16.0 * (double)(T * h), seraph_rmsnorm_backward_residual(a->post_in, W + t->L.post_norm, t->g_xn, t->g_hidden, t->g_hidden,
                                    lora ? t->scratch_gs : GW + t->L.post_norm, T, h, eps, t->ws, t->ws_bytes, s));
-        OP("add", 0.0, 12.0 * (double)(T * h), seraph_add(t->g_tmp, t->g_hidden, t->g_hidden, (size_t)(T * h), s));
 
         /* attention */
         if (!lora) GEMM(t->g_hidden, a->attn_out, GW + t->L.o, h, qd, T, 1, 0, 1);
@@ -668,9 +668,8 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         GEMM(t->g_q, W + t->L.q, t->g_xn, T, h, qd, 0, 0, 0);
         GEMM(t->g_k, W + t->L.k, t->g_xn, T, h, kv, 0, 0, 1);
         GEMM(t->g_v, W + t->L.v, t->g_xn, T, h, kv, 0, 0, 1);
-        OP("rmsnorm_backward", 0.0, 12.0 * (double)(T * h), seraph_rmsnorm_backward(a->layer_in, W + t->L.in_norm, t->g_xn, t->g_tmp,
-                                   lora ? t->scratch_gs : GW + t->L.in_norm, T, h, eps, t->ws, t->ws_bytes, s));
-        OP("add", 0.0, 12.0 * (double)(T * h), seraph_add(t->g_tmp, t->g_hidden, t->g_hidden, (size_t)(T * h), s));
+        OP("rmsnorm_backward", 0.0, 16.0 * (double)(T * h), seraph_rmsnorm_backward_residual(a->layer_in, W + t->L.in_norm, t->g_xn, t->g_hidden, t->g_hidden,
+                                   lora ? t->scratch_gs : GW + t->L.in_norm, T, h, eps, t->ws, t->ws_bytes, s));       /* src/train.c:5342-5355 */
         NANCHK(t->g_hidden, T * h, nan_gh + (uint32_t)l);
     }
     NANCHK(t->g_hidden, T * h, 8u);

@@ -217,6 +217,24 @@ def test_rmsnorm_forward_backward(ops, orc, rows, cols):
         parity(dx, rdx, "rmsnorm dx", atol=1e-7); parity(gs, rgs, "rmsnorm grad_scale")
 
 
+@pytest.mark.parametrize("rows,cols", [(33, 512), (300, 2048), (5, 4096), (9, 100), (700, 8192)])
+def test_rmsnorm_backward_with_residual(ops, rows, cols):
+    """dx = residual + input gradient in one pass: bit-identical to the separate add, also in place."""
+    r = rng(rows * 3 + cols)
+    x = dev(r.standard_normal((rows, cols)).astype(np.float32))
+    s = dev((1 + 0.02 * r.standard_normal(cols)).astype(np.float32))
+    dy = dev((1e-2 * r.standard_normal((rows, cols))).astype(np.float32))
+    res = dev(r.standard_normal((rows, cols)).astype(np.float32))
+    g0 = r.standard_normal(cols).astype(np.float32)
+    dx, gs = ops.rmsnorm_backward(x, s, dy, 1e-5, grad_scale=dev(g0))
+    want = ops.add(dx, res, torch.empty_like(dx))
+    got, gs2 = ops.rmsnorm_backward(x, s, dy, 1e-5, grad_scale=dev(g0), residual=res)
+    assert torch.equal(got, want) and torch.equal(gs, gs2)
+    inplace = res.clone()
+    ops.rmsnorm_backward(x, s, dy, 1e-5, grad_scale=dev(g0), residual=inplace, out=inplace)
+    assert torch.equal(inplace, want)
+
+
 def test_rmsnorm_backward_clamp_branch(ops, orc):
     r = rng(3)
     x = (1e-4 * r.standard_normal((6, 512))).astype(np.float32)       # sqrt(ms + 1e-5) < 0.01
