@@ -155,6 +155,11 @@ int seraph_attention_backward_banded(const float* Q, const float* K, const float
 /* vulkan_rmsnorm, include/vulkan_backend.h:499-503 (shaders/rmsnorm.comp) */
 int seraph_rmsnorm(const float* x, const float* scale, float* y, int64_t rows, int64_t cols, float eps,
                    seraph_stream_t s);
+/* sum = x + addend, y = rmsnorm(sum): the vulkan_add that closes a residual branch and the vulkan_rmsnorm
+ * that opens the next one (src/train.c:4705-4711; :4737 with the next layer's :4668) in one pass.  sum is a
+ * buffer of its own.  addend == NULL and sum == NULL: seraph_rmsnorm. */
+int seraph_add_rmsnorm(const float* x, const float* addend, float* sum, const float* scale, float* y,
+                       int64_t rows, int64_t cols, float eps, seraph_stream_t s);
 /* vulkan_rmsnorm_backward_batch, include/vulkan_backend.h:552-558
  * (shaders/rmsnorm_backward_batch.comp:34-100): FP64 intermediates, rms floor 0.01,
  * grad_scale accumulated (+=) with a deterministic two-stage column reduction. */

@@ -19,6 +19,8 @@ constexpr int kWavesPerBlock = kBlock / kWave;
 // ---------------------------------------------------------------- forward
 template <int VPL>
 __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const float* __restrict__ x,
+                                                             const float* __restrict__ addend,   // NULL, or added to x first
+                                                             float* __restrict__ sum,            // where x + addend goes
                                                              const float* __restrict__ scale,
                                                              float* __restrict__ y,
                                                              int64_t rows, int cols, float eps) {
@@ -40,6 +42,11 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const float* __rest
         for (int k = 0; k < VPL; k++) {
             int i4 = lane + 64 * k;
             v[k] = i4 < n4 ? xr[i4] : make_float4(0, 0, 0, 0);
+            if (addend && i4 < n4) {
+                const float4 b = reinterpret_cast<const float4*>(addend + row * cols)[i4];
+                v[k] = make_float4(v[k].x + b.x, v[k].y + b.y, v[k].z + b.z, v[k].w + b.w);
+                reinterpret_cast<float4*>(sum + row * cols)[i4] = v[k];
+            }
             ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
         }
         ss = wave_sum(ss);
@@ -57,6 +64,8 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const float* __rest
 
 // Any cols / alignment: the row is read twice (the second read is served by cache).
 __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_generic_kernel(const float* __restrict__ x,
+                                                                     const float* __restrict__ addend,
+                                                                     float* __restrict__ sum,
                                                                      const float* __restrict__ scale,
                                                                      float* __restrict__ y,
                                                                      int64_t rows, int64_t cols, float eps) {
@@ -65,6 +74,10 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_generic_kernel(const float
     const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
     for (int64_t row = wave; row < rows; row += nwaves) {
         const float* xr = x + row * cols;
+        if (addend) {                                     // the sum is stored first and then normalised like any input
+            for (int64_t c = lane; c < cols; c += 64) sum[row * cols + c] = xr[c] + addend[row * cols + c];
+            xr = sum + row * cols;                        // each lane rereads only what it wrote
+        }
         float ss = 0.0f;
         for (int64_t c = lane; c < cols; c += 64) ss += xr[c] * xr[c];
         ss = wave_sum(ss);
@@ -414,15 +427,22 @@ extern "C" {
 
 int seraph_rmsnorm(const float* x, const float* scale, float* y, int64_t rows, int64_t cols, float eps,
                    seraph_stream_t s) {
+    return seraph_add_rmsnorm(x, nullptr, nullptr, scale, y, rows, cols, eps, s);
+}
+
+int seraph_add_rmsnorm(const float* x, const float* addend, float* sum, const float* scale, float* y,
+                       int64_t rows, int64_t cols, float eps, seraph_stream_t s) {
     if (rows == 0 || cols == 0) return SERAPH_OK;
     SERAPH_REQUIRE(x && scale && y, "rmsnorm: NULL pointer");
+    SERAPH_REQUIRE(!addend == !sum, "add_rmsnorm: the addend and the place for the sum come together");
+    SERAPH_REQUIRE(!sum || (sum != x && sum != addend && sum != y), "add_rmsnorm: the sum needs a buffer of its own");
     SERAPH_REQUIRE(rows > 0 && cols > 0, "rmsnorm: bad shape %lld x %lld", (long long)rows, (long long)cols);
     int64_t want = ceil_div(rows, kWavesPerBlock);
     int64_t cap = (int64_t)num_compute_units() * 8;
     int grid = (int)(want < cap ? want : cap);
-    int vpl = (aligned16(x) && aligned16(scale) && aligned16(y)) ? pick_vpl(cols) : 0;
+    int vpl = (aligned16(x) && aligned16(scale) && aligned16(y) && (!addend || (aligned16(addend) && aligned16(sum)))) ? pick_vpl(cols) : 0;
     hipStream_t st = as_stream(s);
-#define FWD(V) hipLaunchKernelGGL(rmsnorm_fwd_kernel<V>, dim3(grid), dim3(kBlock), 0, st, x, scale, y, rows, (int)cols, eps)
+#define FWD(V) hipLaunchKernelGGL(rmsnorm_fwd_kernel<V>, dim3(grid), dim3(kBlock), 0, st, x, addend, sum, scale, y, rows, (int)cols, eps)
     switch (vpl) {
         case 1: FWD(1); break;
         case 2: FWD(2); break;
@@ -430,7 +450,7 @@ int seraph_rmsnorm(const float* x, const float* scale, float* y, int64_t rows, i
         case 8: FWD(8); break;
         case 16: FWD(16); break;
         default:
-            hipLaunchKernelGGL(rmsnorm_fwd_generic_kernel, dim3(grid), dim3(kBlock), 0, st, x, scale, y, rows, cols, eps);
+            hipLaunchKernelGGL(rmsnorm_fwd_generic_kernel, dim3(grid), dim3(kBlock), 0, st, x, addend, sum, scale, y, rows, cols, eps);
     }
 #undef FWD
     SERAPH_LAUNCH_CHECK();

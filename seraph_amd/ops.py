@@ -146,6 +146,14 @@ def rmsnorm(x, scale, eps):
     return y
 
 
+def add_rmsnorm(x, addend, scale, eps):
+    """(x + addend, rmsnorm(x + addend)) in one pass."""
+    total, y = torch.empty_like(x), torch.empty_like(x)
+    check(kernels().seraph_add_rmsnorm(_p(x), _p(addend), _p(total), _p(scale), _p(y), i64(x.shape[0]), i64(x.shape[1]),
+                                       f32(eps), _stream()), "add_rmsnorm")
+    return total, y
+
+
 def rmsnorm_backward(x, scale, dy, eps, grad_scale=None, residual=None, out=None):
     """residual: added to the input gradient as it is stored (out may be the residual itself)."""
     dx = torch.empty_like(x) if out is None else out

@@ -554,7 +554,8 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         const float* LW = lora ? t->LP + t->LL.stride * l : NULL;
         layer_act_t* a = &t->act[l];
         float* next = (l + 1 < NL) ? t->act[l + 1].layer_in : t->final_in;
-        OP("rmsnorm", 0.0, 8.0 * (double)(T * h), seraph_rmsnorm(a->layer_in, W + t->L.in_norm, a->xn_attn, T, h, eps, s));
+        /* the input norm of every layer but the first comes out of the add that ended the previous layer */
+        if (l == 0) OP("rmsnorm", 0.0, 8.0 * (double)(T * h), seraph_rmsnorm(a->layer_in, W + t->L.in_norm, a->xn_attn, T, h, eps, s));
         GEMM(a->xn_attn, W + t->L.q, a->q, T, qd, h, 0, 1, 0);
         if (lora && t->LL.A[0] >= 0 && lora_forward_add(t, a->xn_attn, a->q, LW + t->LL.A[0], LW + t->LL.B[0], T, h, qd)) return -1.0f;
         GEMM(a->xn_attn, W + t->L.k, a->k, T, kv, h, 0, 1, 0);
@@ -565,8 +566,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         OP("attention_forward", 4.0 * D * t->attn_pairs * H, 0.0, seraph_attention_forward(a->q, a->k, a->v, a->attn_out, a->lse, starts, batch, T, H, KVH, D, scale, s));
         GEMM(a->attn_out, W + t->L.o, t->tmp_h, T, h, qd, 0, 1, 0);
         if (lora && t->LL.A[3] >= 0 && lora_forward_add(t, a->attn_out, t->tmp_h, LW + t->LL.A[3], LW + t->LL.B[3], T, qd, h)) return -1.0f;
-        OP("add", 0.0, 12.0 * (double)(T * h), seraph_add(a->layer_in, t->tmp_h, a->post_in, (size_t)(T * h), s));
-        OP("rmsnorm", 0.0, 8.0 * (double)(T * h), seraph_rmsnorm(a->post_in, W + t->L.post_norm, a->xn_ffn, T, h, eps, s));
+        OP("add_rmsnorm", 0.0, 16.0 * (double)(T * h), seraph_add_rmsnorm(a->layer_in, t->tmp_h, a->post_in, W + t->L.post_norm, a->xn_ffn, T, h, eps, s));
         GEMM(a->xn_ffn, W + t->L.gate, a->gate, T, f, h, 0, 1, 0);
         if (lora && t->LL.A[4] >= 0 && lora_forward_add(t, a->xn_ffn, a->gate, LW + t->LL.A[4], LW + t->LL.B[4], T, h, f)) return -1.0f;
         GEMM(a->xn_ffn, W + t->L.up, a->up, T, f, h, 0, 1, 0);
@@ -574,10 +574,13 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         OP("swiglu", 0.0, 12.0 * (double)(T * f), seraph_swiglu(a->gate, a->up, a->ffn_h, (size_t)(T * f), s));
         GEMM(a->ffn_h, W + t->L.down, t->tmp_h, T, h, f, 0, 1, 0);
         if (lora && t->LL.A[6] >= 0 && lora_forward_add(t, a->ffn_h, t->tmp_h, LW + t->LL.A[6], LW + t->LL.B[6], T, f, h)) return -1.0f;
-        OP("add", 0.0, 12.0 * (double)(T * h), seraph_add(a->post_in, t->tmp_h, next, (size_t)(T * h), s));
+        /* residual add and the norm that reads its result: the next layer's input norm, or the final norm */
+        const float* next_gain = (l + 1 < NL) ? P + t->off_layer0 + t->L.stride * (l + 1) + t->L.in_norm : P + t->off_final_norm;
+        float* next_xn = (l + 1 < NL) ? t->act[l + 1].xn_attn : t->xn_final;
+        OP("add_rmsnorm", 0.0, 16.0 * (double)(T * h), seraph_add_rmsnorm(a->post_in, t->tmp_h, next, next_gain, next_xn, T, h, eps, s));
         NANCHK(next, T * h, nan_fwd + (uint32_t)l);
     }
-    OP("rmsnorm", 0.0, 8.0 * (double)(T * h), seraph_rmsnorm(t->final_in, P + t->off_final_norm, t->xn_final, T, h, eps, s));
+    if (NL == 0) OP("rmsnorm", 0.0, 8.0 * (double)(T * h), seraph_rmsnorm(t->final_in, P + t->off_final_norm, t->xn_final, T, h, eps, s));
     NANCHK(t->xn_final, T * h, 2u);
     NANCHK(t->final_in, T * h, 6u);
     GEMM(t->xn_final, P + t->off_embed, t->logits, T, V, h, 0, 1, 0);      /* tied head, src/train.c:4869-4872 */

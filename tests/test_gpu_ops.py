@@ -217,6 +217,18 @@ def test_rmsnorm_forward_backward(ops, orc, rows, cols):
         parity(dx, rdx, "rmsnorm dx", atol=1e-7); parity(gs, rgs, "rmsnorm grad_scale")
 
 
+@pytest.mark.parametrize("rows,cols", [(33, 512), (300, 2048), (9, 100), (17, 4096), (1, 4)])
+def test_add_rmsnorm_equals_add_then_rmsnorm(ops, rows, cols):
+    r = rng(rows + 7 * cols)
+    x = dev(r.standard_normal((rows, cols)).astype(np.float32))
+    b = dev(r.standard_normal((rows, cols)).astype(np.float32))
+    s = dev((1 + 0.02 * r.standard_normal(cols)).astype(np.float32))
+    total = ops.add(x, b, torch.empty_like(x))
+    want = ops.rmsnorm(total, s, 1e-5)
+    got_total, got = ops.add_rmsnorm(x, b, s, 1e-5)
+    assert torch.equal(got_total, total) and torch.equal(got, want)
+
+
 @pytest.mark.parametrize("rows,cols", [(33, 512), (300, 2048), (5, 4096), (9, 100), (700, 8192)])
 def test_rmsnorm_backward_with_residual(ops, rows, cols):
     """dx = residual + input gradient in one pass: bit-identical to the separate add, also in place."""
