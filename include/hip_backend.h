@@ -197,6 +197,15 @@ void hip_qk_norm_backward(vulkan_context_t* ctx, vulkan_buffer_t* qk_pre, vulkan
 void hip_adamw_update_clipped(vulkan_context_t* ctx, vulkan_buffer_t* weight, vulkan_buffer_t* grad, vulkan_buffer_t* m,
                               vulkan_buffer_t* v, float lr, float beta1, float beta2, float weight_decay, float eps,
                               int step, size_t size, float clip);
+/* sum = input + addend, output = rmsnorm(sum): the vulkan_add that closes a residual branch and the vulkan_rmsnorm
+ * that reads its result (src/train.c:4705-4711) in one pass; sum is a buffer of its own */
+void hip_add_rmsnorm(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* addend, vulkan_buffer_t* sum,
+                     vulkan_buffer_t* scale, vulkan_buffer_t* output, int rows, int cols, float eps);
+/* vulkan_rmsnorm_backward_batch with the vulkan_add that follows it (src/train.c:5180-5193) folded in:
+ * grad_input = residual + input gradient; residual may be grad_input itself */
+void hip_rmsnorm_backward_residual(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* scale,
+                                   vulkan_buffer_t* grad_output, vulkan_buffer_t* residual, vulkan_buffer_t* grad_input,
+                                   vulkan_buffer_t* grad_scale, int rows, int cols, float eps);
 /* C (+)= alpha * op(A) op(B): vulkan_matmul_transpose followed by vulkan_scale of the product, the pair the
  * LoRA path issues (src/train.c:5785-5792, :5815-5841), as one op.  accumulate with alpha != 1 is only possible
  * for the shapes the library computes through its scratch (small output, long K); otherwise the op reports an

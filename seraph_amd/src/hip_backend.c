@@ -341,6 +341,15 @@ void vulkan_rmsnorm(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer
     HIP_OP(ctx, "rmsnorm", seraph_rmsnorm(FPTR(input), FPTR(scale), FPTR(output), rows, cols, eps, st->stream));
 }
 
+/* vulkan_add of a residual branch and the vulkan_rmsnorm that reads the sum (src/train.c:4705-4711): sum = input + addend,
+ * output = rmsnorm(sum); sum is a buffer of its own. */
+void hip_add_rmsnorm(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* addend, vulkan_buffer_t* sum,
+                     vulkan_buffer_t* scale, vulkan_buffer_t* output, int rows, int cols, float eps) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !input || !addend || !sum || !scale || !output) return;
+    HIP_OP(ctx, "add_rmsnorm", seraph_add_rmsnorm(FPTR(input), FPTR(addend), FPTR(sum), FPTR(scale), FPTR(output), rows, cols, eps, st->stream));
+}
+
 void vulkan_rope(vulkan_context_t* ctx, vulkan_buffer_t* x_in, vulkan_buffer_t* x_out,
                  int seq_len, int num_heads, int head_dim, float rope_theta) {
     hip_state_t* st = hip_state(ctx);

@@ -47,6 +47,21 @@ void vulkan_rmsnorm_backward_batch(vulkan_context_t* ctx, vulkan_buffer_t* input
                                                                   FPTR(grad_scale), rows, cols, eps, ws, st->ws_bytes, st->stream));
 }
 
+/* vulkan_rmsnorm_backward_batch and the vulkan_add of the residual gradient that follows it (src/train.c:5180-5193):
+ * grad_input = residual + input gradient; residual may be grad_input itself. */
+void hip_rmsnorm_backward_residual(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* scale,
+                                   vulkan_buffer_t* grad_output, vulkan_buffer_t* residual, vulkan_buffer_t* grad_input,
+                                   vulkan_buffer_t* grad_scale, int rows, int cols, float eps) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !input || !scale || !grad_output || !residual || !grad_input || !grad_scale) return;
+    size_t need = seraph_rmsnorm_backward_ws_bytes(rows, cols);
+    void* ws = hip_backend_scratch(ctx, need);
+    if (!ws) return;
+    HIP_OP(ctx, "rmsnorm_backward_residual", seraph_rmsnorm_backward_residual(FPTR(input), FPTR(scale), FPTR(grad_output), FPTR(residual),
+                                                                              FPTR(grad_input), FPTR(grad_scale), rows, cols, eps, ws,
+                                                                              st->ws_bytes, st->stream));
+}
+
 /* src/vulkan_backend_backward.c:931-1045 */
 void vulkan_rope_backward(vulkan_context_t* ctx, vulkan_buffer_t* x_in, vulkan_buffer_t* x_out,
                           int seq_len, int num_heads, int head_dim, float rope_theta) {

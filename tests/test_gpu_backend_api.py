@@ -182,3 +182,32 @@ def test_lora_products_through_the_backend(vk, orc):
     for b in (bx, bA, bB):
         lib.vulkan_buffer_free(ctx, b)
     assert lib.hip_backend_error_count(ctx) == 0
+
+
+def test_residual_adds_folded_into_the_norms(vk):
+    """hip_add_rmsnorm and hip_rmsnorm_backward_residual against the reference's op pairs, bit for bit."""
+    lib, ctx = vk
+    r = rng(22)
+    rows, cols, eps = 300, 512, C.c_float(1e-5)
+    x, b, dy = (r.standard_normal((rows, cols)).astype(np.float32) for _ in range(3))
+    s = (1 + 0.02 * r.standard_normal(cols)).astype(np.float32)
+    bx, bb, bdy, bs = up(vk, x), up(vk, b), up(vk, dy), up(vk, s)
+    zeros = lambda shape: up(vk, np.zeros(shape, np.float32))
+    sum1, y1, sum2, y2 = (zeros((rows, cols)) for _ in range(4))
+    dx1, gs1, gs2 = zeros((rows, cols)), zeros(cols), zeros(cols)
+    res2 = up(vk, b)
+    assert lib.vulkan_cmd_begin(ctx) == 1
+    lib.vulkan_add(ctx, bx, bb, sum1, C.c_size_t(rows * cols))
+    lib.vulkan_rmsnorm(ctx, sum1, bs, y1, rows, cols, eps)
+    lib.hip_add_rmsnorm(ctx, bx, bb, sum2, bs, y2, rows, cols, eps)
+    lib.vulkan_rmsnorm_backward_batch(ctx, bx, bs, bdy, dx1, gs1, rows, cols, eps)
+    lib.vulkan_add(ctx, dx1, bb, dx1, C.c_size_t(rows * cols))
+    lib.hip_rmsnorm_backward_residual(ctx, bx, bs, bdy, res2, res2, gs2, rows, cols, eps)      # in place
+    assert lib.vulkan_cmd_end_submit(ctx) == 1
+    assert (down(vk, sum1, (rows, cols)) == down(vk, sum2, (rows, cols))).all()
+    assert (down(vk, y1, (rows, cols)) == down(vk, y2, (rows, cols))).all()
+    assert (down(vk, dx1, (rows, cols)) == down(vk, res2, (rows, cols))).all()
+    assert (down(vk, gs1, cols) == down(vk, gs2, cols)).all()
+    for buf in (bx, bb, bdy, bs, sum1, y1, sum2, y2, dx1, gs1, gs2, res2):
+        lib.vulkan_buffer_free(ctx, buf)
+    assert lib.hip_backend_error_count(ctx) == 0
