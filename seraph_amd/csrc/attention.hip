@@ -832,11 +832,13 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
         }
         __syncthreads();
     };
-    // The straight-line iteration for two sub-tiles, software-pipelined.  A SIMD runs one wave here, and while a
-    // wave's next instruction is a matrix instruction waiting for the matrix pipe nothing else issues, so the
-    // exponentials and masks only overlap with matrix work when they sit between matrix instructions of the
-    // same wave.  The two sub-tiles provide that: S/dP of sub-tile 1 carries the softmax of sub-tile 0, and
-    // dV/dK of sub-tile 0 carries the softmax of sub-tile 1.
+    // The straight-line iteration for two sub-tiles, software-pipelined.  A SIMD runs one wave here (a second wave
+    // brought nothing: while a wave's next instruction is a matrix instruction waiting for the pipe, the other wave's
+    // arithmetic crawls), so everything that is not a matrix instruction is written into the runs of matrix
+    // instructions of the same wave: S/dP of sub-tile 1 carries the softmax of sub-tile 0, dV/dK of sub-tile 0 the
+    // softmax of sub-tile 1, the LDS writes of the next tile and the dS stores.  The memory and LDS instructions stay
+    // where they are written (every step is one scheduling region); the optimiser still gathers most of the
+    // exponentials at the head of the following phase, which measured faster than pinning them to their steps.
     auto iteration2 = [&](int hg, int n, int li, int hg2, int n2) {
         constexpr int NS = D / 8, EPS = 16 / NS;               // S-phase steps, softmax elements per step
         const int cur = li & 1;
