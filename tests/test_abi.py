@@ -77,3 +77,13 @@ def test_param_count_matches_reference_shapes(libs):
     assert n == 151936 * 2048 + 2048 + 28 * (2 * 2048 + 2 * 2048 * 2048 + 2 * 1024 * 2048 + 3 * 2048 * 6144)
     lora = trainer.model_config(2048, 28, 16, 8, 128, 6144, 151936, lora_rank=16, lora_alpha=32.0, lora_mask=15)
     assert trainer.lora_param_count(lora) == 28 * 16 * ((2048 + 2048) + 2 * (2048 + 1024) + (2048 + 2048))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The build is for one GPU: --gpus N > 1 ends with a message, not with a number."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert p.returncode != 0 and "one GPU" in (p.stdout + p.stderr)
+    assert '"metric"' not in p.stdout

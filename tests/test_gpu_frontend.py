@@ -352,3 +352,24 @@ def test_reference_batched_trainer_profile_and_lora(tmp_path, orc):
     assert len(got) == len(batches) and abs(got[0] - base_loss) < 1.5e-4
     assert all(np.isfinite(got))
     assert os.path.exists(tmp_path / "q" / "checkpoint_final.bin")
+
+
+def test_bench_line_contract():
+    """bench.py prints one JSON line with the agreed keys (33M workload, two steps)."""
+    import json
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--workload", "c1", "--steps", "2", "--warmup", "1",
+                        "--no-cpu-baseline"], capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    lines = [l for l in p.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+              "vs_baseline", "dtype", "data", "config", "roofline"):
+        assert k in d, k
+    assert d["n_gpus"] == 1 and d["steps"] == 2 and d["warmup"] == 1 and d["dtype"] == "f32" and d["vs_baseline"] is None
+    assert d["value"] > 0 and abs(d["value"] - d["config"]["tokens_per_step"] / d["ms_per_step"] * 1e3) < 1e-3 * d["value"]
+    rf = d["roofline"]
+    assert rf["bound"] in ("hbm", "mfma") and abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-3
