@@ -366,7 +366,9 @@ ATTN_CASES_BWD = ATTN_CASES + [([0, 700, 731, 1500], 4, 2, 64), ([0, 513, 1030],
                                # enough (key tile, kv head) items to fill the chip: every item keeps all of its iterations
                                ([0, 600, 1111, 1500, 2100, 2650, 3333, 4100], 16, 8, 128),
                                ([0, 600, 1111, 1500, 2100, 2650, 3333, 4100], 8, 8, 64),
-                               ([0, 77, 2000, 4100], 8, 8, 32)]
+                               ([0, 77, 2000, 4100], 8, 8, 32),
+                               # wider query groups per kv head (4 and 8 query heads each)
+                               ([0, 300, 700], 8, 2, 64), ([0, 513, 1030], 8, 1, 128), ([0, 90, 640], 4, 1, 32)]
 
 
 @pytest.mark.parametrize("starts,H,KVH,D", ATTN_CASES_BWD)
