@@ -390,6 +390,26 @@ def test_attention_backward(ops, orc, starts, H, KVH, D, saved, banded):
     parity(dQ, rdQ, "dQ"); parity(dK, rdK, "dK"); parity(dV, rdV, "dV")
 
 
+def test_attention_many_short_sequences(ops, orc):
+    """More sequences than the kernels keep offsets for in LDS, and more 128-token tiles than they rank by length:
+    the offsets are searched in global memory and the tiles run in their natural order."""
+    n_seq, H, KVH, D = 2800, 2, 1, 32
+    r = rng(77)
+    lens = r.integers(1, 100, n_seq)
+    starts = np.concatenate([[0], np.cumsum(lens)]).astype(np.uint32)
+    T = int(starts[-1])
+    assert T > 1024 * 128 and n_seq + 1 > 1024
+    Q, K, V, dO = _attn_inputs(5, [0, T], H, KVH, D)
+    sd = dev(starts.view(np.int32))
+    ro, rl = orc.attention_forward(Q, K, V, H, KVH, D, starts)
+    o, l = ops.attention_forward(dev(Q), dev(K), dev(V), H, KVH, D, sd)
+    parity(o, ro, "out"); parity(l, rl, "lse")
+    rdQ, rdK, rdV = orc.attention_backward(Q, K, V, dO, H, KVH, D, starts)
+    for msl in (None, int(lens.max())):
+        dQ, dK, dV = ops.attention_backward(dev(Q), dev(K), dev(V), dev(dO), H, KVH, D, sd, out=o, lse=l, max_seq_len=msl)
+        parity(dQ, rdQ, "dQ"); parity(dK, rdK, "dK"); parity(dV, rdV, "dV")
+
+
 def test_attention_backward_is_deterministic(ops):
     Q, K, V, dO = _attn_inputs(4, [0, 300, 700], 4, 2, 64)
     sd = dev(np.array([0, 300, 700], np.int32))
