@@ -390,6 +390,26 @@ def test_attention_backward(ops, orc, starts, H, KVH, D, saved, banded):
     parity(dQ, rdQ, "dQ"); parity(dK, rdK, "dK"); parity(dV, rdV, "dV")
 
 
+def test_rope_and_cross_entropy_many_short_sequences(ops, orc):
+    """Thousands of packed sequences: positions restart and the last token of each has no target."""
+    n_seq = 3000
+    r = rng(78)
+    lens = r.integers(1, 12, n_seq)
+    starts = np.concatenate([[0], np.cumsum(lens)]).astype(np.uint32)
+    T = int(starts[-1])
+    sd = dev(starts.view(np.int32))
+    x = r.standard_normal((T, 2 * 64)).astype(np.float32)
+    parity(ops.rope(dev(x), 2, 64, 10000.0, sd), orc.rope(x, 2, 64, 10000.0, starts), "rope", atol=2e-5)
+    parity(ops.rope(dev(x), 2, 64, 10000.0, sd, backward=True), orc.rope(x, 2, 64, 10000.0, starts, backward=True), "rope bwd", atol=2e-5)
+    V = 1000
+    logits = r.standard_normal((T, V)).astype(np.float32)
+    t = r.integers(0, V, T).astype(np.uint32)
+    valid = T - n_seq
+    rg, rl = orc.cross_entropy_grad_packed(logits, t, starts, valid)
+    g, l = ops.cross_entropy_grad(dev(logits), dev(t.view(np.int32)), valid, seq_starts=sd)
+    parity(g, rg, "packed grad", atol=1e-7); parity(l, rl, "packed loss")
+
+
 def test_attention_many_short_sequences(ops, orc):
     """More sequences than the kernels keep offsets for in LDS, and more 128-token tiles than they rank by length:
     the offsets are searched in global memory and the tiles run in their natural order."""
