@@ -172,6 +172,17 @@ int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy,
 int seraph_rmsnorm_backward_residual(const float* x, const float* scale, const float* dy, const float* residual, float* dx,
                                      float* grad_scale, int64_t rows, int64_t cols, float eps, void* ws, size_t ws_bytes,
                                      seraph_stream_t s);
+/* seraph_rmsnorm_backward_residual for callers that cannot allocate device memory or bring a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The partial rows of the column reduction live in an array built into the
+ * library (seraph_rmsnorm_backward_static_max_bytes() = 16 MiB on every GPU the library runs on, held until
+ * the process ends); the call allocates nothing.  Shapes whose seraph_rmsnorm_backward_ws_bytes exceeds
+ * that size are refused with SERAPH_ERR_WORKSPACE (16384 x 2048 needs 4 MiB; rows of up to 8192 columns
+ * fit at any row count when 16-byte aligned).  Results are bit-identical to the workspace form.  Every
+ * call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race. */
+size_t seraph_rmsnorm_backward_static_max_bytes(void);
+int seraph_rmsnorm_backward_static(const float* x, const float* scale, const float* dy, const float* residual, float* dx,
+                                   float* grad_scale, int64_t rows, int64_t cols, float eps, seraph_stream_t s);
 /* vulkan_rope / vulkan_rope_backward, include/vulkan_backend.h:493-495,561-563
  * (shaders/rope.comp, rope_backward.comp:26-59) and the packed forms
  * (include/cuda_train_context.h:275,286).  in and out may alias.  backward != 0 applies

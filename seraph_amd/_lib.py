@@ -25,7 +25,7 @@ def kernels():
         lib.seraph_hip_last_error.restype = C.c_char_p
         for name in ("seraph_attention_backward_ws_bytes", "seraph_attention_backward_ws_bytes_banded",
                      "seraph_rmsnorm_backward_ws_bytes", "seraph_embedding_backward_ws_bytes",
-                     "seraph_gemm_scaled_ws_bytes"):
+                     "seraph_gemm_scaled_ws_bytes", "seraph_rmsnorm_backward_static_max_bytes"):
             getattr(lib, name).restype = C.c_size_t
         _kernels = lib
     return _kernels

@@ -39,6 +39,7 @@ static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 int num_compute_units();           // cached after seraph_hip_init / first use
+int rmsnorm_static_scratch_setup(); // rmsnorm.hip: looks up its built-in scratch array on the current device
 
 // ---------------------------------------------------------------- device helpers
 __device__ __forceinline__ float wave_sum(float v) {

@@ -9,6 +9,8 @@
 // The column reduction for grad_scale is deterministic: a lane keeps per-column partial sums
 // over the rows it visits, each workgroup writes one partial row to scratch, and a second
 // small kernel adds the partial rows in a fixed order.
+#include <mutex>
+
 #include "common.hpp"
 
 namespace seraph {
@@ -388,6 +390,37 @@ __global__ __launch_bounds__(kBlock) void qk_norm_bwd_kernel(const float* __rest
     }
 }
 
+// ---------------------------------------------------------------- static scratch
+// Partial rows for callers that can neither allocate nor bring a workspace (code under graph capture,
+// serving loops).  One array per GPU, held until the process ends.  `scratch` is a host-side stand-in
+// in host code: only the address hipGetSymbolAddress returns for the current device may reach a kernel.
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
+constexpr int kMaxDevices = 64;
+static float* g_scratch_ptr[kMaxDevices];              // device address of `scratch` on each GPU
+static std::mutex g_scratch_mutex;
+
+// Address of this file's scratch array on the current device (looked up once per device).
+static int static_scratch(float** out) {
+    int dev = -1;
+    SERAPH_HIP_CHECK(hipGetDevice(&dev));
+    SERAPH_REQUIRE(dev >= 0 && dev < kMaxDevices, "rmsnorm_backward_static: device index %d not supported", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        float* ptr = nullptr;
+        SERAPH_HIP_CHECK(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+        SERAPH_REQUIRE(ptr != nullptr, "rmsnorm_backward_static: no device address for the scratch array");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return SERAPH_OK;
+}
+
+int rmsnorm_static_scratch_setup() {
+    float* p = nullptr;
+    return static_scratch(&p);
+}
+
 // ---------------------------------------------------------------- host side
 static int pick_vpl(int64_t cols) {
     if (cols % 4 != 0) return 0;
@@ -470,20 +503,12 @@ int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy,
     return seraph_rmsnorm_backward_residual(x, scale, dy, nullptr, dx, grad_scale, rows, cols, eps, ws, ws_bytes, s);
 }
 
-int seraph_rmsnorm_backward_residual(const float* x, const float* scale, const float* dy, const float* residual, float* dx,
-                                     float* grad_scale, int64_t rows, int64_t cols, float eps, void* ws, size_t ws_bytes,
-                                     seraph_stream_t s) {
-    const float* res = residual;
-    if (rows == 0 || cols == 0) return SERAPH_OK;
-    SERAPH_REQUIRE(x && scale && dy && dx && grad_scale, "rmsnorm_backward: NULL pointer");
-    SERAPH_REQUIRE(rows > 0 && cols > 0, "rmsnorm_backward: bad shape");
-    if (!ws || ws_bytes < seraph_rmsnorm_backward_ws_bytes(rows, cols)) {
-        set_error("rmsnorm_backward: scratch of %zu bytes required", seraph_rmsnorm_backward_ws_bytes(rows, cols));
-        return SERAPH_ERR_WORKSPACE;
-    }
+// Launches of the backward on checked arguments; `partial` holds seraph_rmsnorm_backward_ws_bytes(rows, cols).
+static int rmsnorm_backward_launch(const float* x, const float* scale, const float* dy, const float* res, float* dx,
+                                   float* grad_scale, int64_t rows, int64_t cols, float eps, float* partial,
+                                   seraph_stream_t s) {
     hipStream_t st = as_stream(s);
-    float* partial = (float*)ws;
-    const bool aligned = aligned16(x) && aligned16(scale) && aligned16(dy) && aligned16(dx) && aligned16(ws) && (!res || aligned16(res));
+    const bool aligned = aligned16(x) && aligned16(scale) && aligned16(dy) && aligned16(dx) && aligned16(partial) && (!res || aligned16(res));
     const int bvpl = aligned ? pick_block_vpl(cols) : 0;
     const int wvpl = (aligned && !bvpl && cols <= 512) ? pick_vpl(cols) : 0;
     int nparts;
@@ -517,6 +542,39 @@ int seraph_rmsnorm_backward_residual(const float* x, const float* scale, const f
                        partial, nparts, cols, grad_scale);
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
+}
+
+int seraph_rmsnorm_backward_residual(const float* x, const float* scale, const float* dy, const float* residual, float* dx,
+                                     float* grad_scale, int64_t rows, int64_t cols, float eps, void* ws, size_t ws_bytes,
+                                     seraph_stream_t s) {
+    if (rows == 0 || cols == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(x && scale && dy && dx && grad_scale, "rmsnorm_backward: NULL pointer");
+    SERAPH_REQUIRE(rows > 0 && cols > 0, "rmsnorm_backward: bad shape");
+    if (!ws || ws_bytes < seraph_rmsnorm_backward_ws_bytes(rows, cols)) {
+        set_error("rmsnorm_backward: scratch of %zu bytes required", seraph_rmsnorm_backward_ws_bytes(rows, cols));
+        return SERAPH_ERR_WORKSPACE;
+    }
+    return rmsnorm_backward_launch(x, scale, dy, residual, dx, grad_scale, rows, cols, eps, (float*)ws, s);
+}
+
+size_t seraph_rmsnorm_backward_static_max_bytes(void) { return kStaticScratchBytes; }
+
+int seraph_rmsnorm_backward_static(const float* x, const float* scale, const float* dy, const float* residual, float* dx,
+                                   float* grad_scale, int64_t rows, int64_t cols, float eps, seraph_stream_t s) {
+    if (rows == 0 || cols == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(x && scale && dy && dx && grad_scale, "rmsnorm_backward_static: NULL pointer");
+    SERAPH_REQUIRE(rows > 0 && cols > 0, "rmsnorm_backward_static: bad shape");
+    const size_t need = seraph_rmsnorm_backward_ws_bytes(rows, cols);
+    if (need > kStaticScratchBytes) {
+        set_error("rmsnorm_backward_static: %lld x %lld needs %zu bytes of scratch, the built-in array holds %zu; "
+                  "use seraph_rmsnorm_backward_residual with a workspace", (long long)rows, (long long)cols, need,
+                  kStaticScratchBytes);
+        return SERAPH_ERR_WORKSPACE;
+    }
+    float* partial = nullptr;
+    int rc = static_scratch(&partial);
+    if (rc != SERAPH_OK) return rc;
+    return rmsnorm_backward_launch(x, scale, dy, residual, dx, grad_scale, rows, cols, eps, partial, s);
 }
 
 int seraph_qk_norm(float* qk, int64_t T, int heads, int head_dim, int use_qk_norm, float eps, seraph_stream_t s) {

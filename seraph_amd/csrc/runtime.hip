@@ -52,7 +52,7 @@ int seraph_hip_init(int device_index) {
         return SERAPH_ERR_NODEVICE;
     }
     g_cu_count = prop.multiProcessorCount;
-    return SERAPH_OK;
+    return rmsnorm_static_scratch_setup();     // per-device address of the built-in scratch array
 }
 
 int seraph_hip_device_info(seraph_device_info_t* out) {

@@ -171,6 +171,14 @@ def rmsnorm_backward(x, scale, dy, eps, grad_scale=None, residual=None, out=None
     return dx, gs
 
 
+def rmsnorm_backward_static(x, scale, dy, eps, grad_scale, dx, residual=None):
+    """The backward over the library's built-in scratch array: every buffer is the caller's, nothing is allocated."""
+    rows, cols = x.shape
+    check(kernels().seraph_rmsnorm_backward_static(_p(x), _p(scale), _p(dy), _p(residual), _p(dx), _p(grad_scale), i64(rows),
+                                                   i64(cols), f32(eps), _stream()), "rmsnorm_backward_static")
+    return dx, grad_scale
+
+
 def rope(x, heads, head_dim, theta, seq_starts=None, backward=False, out=None):
     out = torch.empty_like(x) if out is None else out
     check(kernels().seraph_rope(_p(x), _p(out), _p(seq_starts), C.c_int(_batch(seq_starts)), i64(x.shape[0]),

@@ -1,0 +1,58 @@
+"""The entry point that allocates nothing: seraph_rmsnorm_backward_static (partial rows in an array
+built into the library) against seraph_rmsnorm_backward_residual (partial rows in a caller workspace),
+through the C ABI.  Same kernels, same reduction order: the results have to be bit-identical.  Two calls
+in a row share the array, the second on a smaller input, so stale partial rows of the first call would
+show in the second call's grad_scale."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from seraph_amd import ops as o
+    o.init(0)
+    return o
+
+
+def _case(ops, rows, cols, seed, residual):
+    r = np.random.default_rng(seed)
+    x = torch.from_numpy(r.standard_normal((rows, cols)).astype(np.float32)).cuda()
+    s = torch.from_numpy((1 + 0.02 * r.standard_normal(cols)).astype(np.float32)).cuda()
+    dy = torch.from_numpy((0.01 * r.standard_normal((rows, cols))).astype(np.float32)).cuda()
+    res = torch.from_numpy(r.standard_normal((rows, cols)).astype(np.float32)).cuda() if residual else None
+    g0 = torch.from_numpy(r.standard_normal(cols).astype(np.float32)).cuda()      # grad_scale accumulates
+    ref_dx, ref_gs = ops.rmsnorm_backward(x, s, dy, 1e-5, grad_scale=g0.clone(), residual=res)
+    dx, gs = torch.full_like(x, float("nan")), g0.clone()
+    ops.rmsnorm_backward_static(x, s, dy, 1e-5, gs, dx, residual=res)
+    torch.cuda.synchronize()
+    assert torch.equal(dx, ref_dx), (rows, cols, "dx")
+    assert torch.equal(gs, ref_gs), (rows, cols, "grad_scale")
+
+
+def test_static_scratch_matches_workspace_form_on_two_calls_in_a_row(ops):
+    # block-per-row kernel (the training shapes), then a smaller input on the same array
+    _case(ops, 4096, 2048, 1, residual=True)
+    _case(ops, 300, 2048, 2, residual=False)
+    # wave-per-row kernel, then the generic kernel (odd width: zero-filled per-wave partial rows), smaller again
+    _case(ops, 1000, 512, 3, residual=False)
+    _case(ops, 77, 333, 4, residual=True)
+    _case(ops, 5, 333, 5, residual=False)
+
+
+def test_static_scratch_refuses_shapes_beyond_its_size(ops):
+    from seraph_amd._lib import kernels
+    k = kernels()
+    cap = k.seraph_rmsnorm_backward_static_max_bytes()
+    assert cap == 16 << 20
+    rows, cols = 4096, 16384 + 4                      # generic path: one partial row per wave -> far beyond 16 MiB
+    assert k.seraph_rmsnorm_backward_ws_bytes(C.c_int64(rows), C.c_int64(cols)) > cap
+    x = torch.zeros(8, device="cuda")                 # never dereferenced: the size check comes first
+    p = C.c_void_p(x.data_ptr())
+    rc = k.seraph_rmsnorm_backward_static(p, p, p, None, p, p, C.c_int64(rows), C.c_int64(cols), C.c_float(1e-5), None)
+    assert rc == -3
+    assert b"built-in array" in k.seraph_hip_last_error()
