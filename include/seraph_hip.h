@@ -140,8 +140,9 @@ int seraph_attention_backward(const float* Q, const float* K, const float* V, co
  * seraph_attention_backward_ws_bytes_banded(...) bytes, the dK/dV pass leaves dS behind in a band of
  * 32x32 tiles (heads x ceil(T/32) x (ceil(max_seq_len/32)+1) x 4 KiB) and dQ is one product over it:
  * 5 matrix products instead of 7.  With the smaller scratch of seraph_attention_backward_ws_bytes the
- * call is identical to seraph_attention_backward.  max_seq_len <= 0 means T.  A sequence longer than
- * max_seq_len is a caller error (its far-off-diagonal contributions to dQ would be dropped).
+ * call is identical to seraph_attention_backward.  max_seq_len <= 0 means T.  The bound is checked on the
+ * device against seq_starts: when some sequence is longer than max_seq_len the band is left unread and dQ
+ * comes from the recomputing kernel, so the results stay correct and only the saving is lost.
  * Same reference ops as seraph_attention_backward. */
 size_t seraph_attention_backward_ws_bytes_banded(int64_t T, int heads, int kv_heads, int head_dim, int64_t max_seq_len);
 int seraph_attention_backward_banded(const float* Q, const float* K, const float* V, const float* dO,

@@ -29,6 +29,7 @@
 #include <limits.h>
 #include <type_traits>
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 
 #include "common.hpp"
@@ -402,9 +403,14 @@ __global__ __launch_bounds__(kAttnThreads, (KSPLIT ? 1 : 2)) void attn_fwd_kerne
 template <int D>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const float* __restrict__ dO, const float* __restrict__ O,
                                                          float* __restrict__ delta, int64_t T, int H,
-                                                         const uint32_t* __restrict__ seq_starts, int batch, int* __restrict__ row_start) {
+                                                         const uint32_t* __restrict__ seq_starts, int batch, int* __restrict__ row_start,
+                                                         int ds_slots, int epoch, int* __restrict__ band_overflow,
+                                                         unsigned int* __restrict__ queue_a, unsigned int* __restrict__ queue_b) {
     const int lane = threadIdx.x & 63;
     const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    // The two persistent kernels that follow on this stream start from counter pairs this launch has zeroed:
+    // a pair left non-zero by a launch that never finished cannot make them skip tiles.
+    if (blockIdx.x == 0 && threadIdx.x < 4) (threadIdx.x < 2 ? queue_a : queue_b)[threadIdx.x & 1] = 0u;
     if (t >= T) return;
     if (lane == 0) {
         int start = 0;
@@ -417,6 +423,10 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const float* __restrict
             start = (int)seq_starts[lo];
         }
         row_start[t] = start;
+        // A query whose sequence starts more key tiles back than the dS band holds (the caller's bound on the
+        // sequence length was too small): the launch is marked, the banded dQ kernel stands down and the
+        // recomputing one runs instead.  Every marking lane stores the same value.
+        if (ds_slots > 0 && (int)(t >> 5) - (start >> 5) >= ds_slots) *band_overflow = epoch;
     }
     const int64_t qw = (int64_t)H * D;
     constexpr int LPH = D / 4;                                  // lanes per head
@@ -1079,8 +1089,11 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dq_k
                                                                    const float* __restrict__ LSE, const float* __restrict__ DELTA,
                                                                    float* __restrict__ dQ, const uint32_t* __restrict__ seq_starts, int batch,
                                                                    int64_t T, int H, int KVH, float scale, float scale_log2e,
-                                                                   unsigned int* __restrict__ queue) {
+                                                                   unsigned int* __restrict__ queue,
+                                                                   const int* __restrict__ band_overflow, int epoch) {
     constexpr int LD = D + 4, DB = D / 32;
+    // As the stand-in of the banded kernel this launch only works when the delta kernel marked the launch.
+    if (band_overflow && *band_overflow != epoch) return;
     __shared__ __attribute__((aligned(16))) float sK[2][32 * LD];
     __shared__ __attribute__((aligned(16))) float sV[2][32 * LD];
     __shared__ uint32_t sSeq[kMaxSeqLds];
@@ -1194,9 +1207,12 @@ template <int D, bool KSPLIT>
 __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const float* __restrict__ K, const float* __restrict__ DS,
                                                                          float* __restrict__ dQ, const uint32_t* __restrict__ seq_starts,
                                                                          int batch, int64_t T, int H, int KVH, float scale, int ds_slots,
-                                                                         unsigned int* __restrict__ queue) {
+                                                                         unsigned int* __restrict__ queue,
+                                                                         const int* __restrict__ band_overflow, int epoch) {
     constexpr int LD = D + 4, DB = D / 32;
     constexpr int KT = KSPLIT ? 2 : 1, QROWS = KSPLIT ? 64 : 128;
+    // Some sequence is longer than the band was sized for: dQ comes from the recomputing kernel launched next.
+    if (*band_overflow == epoch) return;
     __shared__ __attribute__((aligned(16))) float sK[2][KT * 32 * LD];
     __shared__ uint32_t sSeq[kMaxSeqLds];
     __shared__ int sItem;
@@ -1228,6 +1244,10 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const f
     if (wave_ok) {
         tb = (int)(((int64_t)(seqs.start_of((int)iw0) / 32) * 32 - jbeg) / 32);
         te = (int)((iw0 - jbeg) / 32);
+        // never read a slot the band does not have (only possible in a launch that is marked as overflowing,
+        // which returns above; the clamp keeps every address inside the scratch regardless)
+        const int tmin = qt - (int)(jbeg >> 5) - (ds_slots - 1);
+        tb = tb < tmin ? tmin : tb;
     }
     const float* band = DS + ((((int64_t)head * nqt32 + (wave_ok ? qt : 0)) * ds_slots) << 10);   // slot 0 = diagonal tile
     const int kt0 = (int)(jbeg >> 5);
@@ -1328,7 +1348,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const f
 }
 
 // ---------------------------------------------------------------- host side
-struct AttnWs { float* lse; float* delta; float* out; float* partK; float* partV; int* row_start; float* ds; };
+struct AttnWs { float* lse; float* delta; float* out; float* partK; float* partV; int* row_start; int* overflow; float* ds; };
 constexpr int kMaxSplit = 4;
 
 // Band of dS tiles: for every head and 32-query tile, the key tiles from the diagonal down to the
@@ -1347,7 +1367,9 @@ static size_t attn_ws_layout(int64_t T, int H, int KVH, int D, char* base, AttnW
     char* e = take((size_t)T * H * D * 4);
     char* pk = take((size_t)kMaxSplit * T * KVH * D * 4); char* pv = take((size_t)kMaxSplit * T * KVH * D * 4);
     char* rs = take((size_t)T * 4);
+    char* ov = take(4);
     if (w) {
+        w->overflow = (int*)ov;
         w->lse = (float*)c; w->delta = (float*)d; w->out = (float*)e; w->partK = (float*)pk; w->partV = (float*)pv;
         w->row_start = (int*)rs;
         w->ds = base ? (float*)(base + o) : nullptr;
@@ -1405,15 +1427,21 @@ static int run_forward(const float* Q, const float* K, const float* V, float* O,
 
 template <int D>
 static int run_backward(const float* Q, const float* K, const float* V, const float* dO, const float* O, const float* lse,
-                        float* delta, int* row_start, float* dQ, float* dK, float* dV, const uint32_t* seq_starts, int batch,
+                        float* delta, int* row_start, int* overflow, float* dQ, float* dK, float* dV, const uint32_t* seq_starts, int batch,
                         int64_t T, int H, int KVH, float scale, int64_t longest_seq, float* ds, int ds_slots, float* partK, float* partV,
                         hipStream_t st) {
-    hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)ceil_div(T, 4)), dim3(256), 0, st, dO, O, delta, T, H, seq_starts, batch, row_start);
-    SERAPH_LAUNCH_CHECK();
     unsigned int *qkv = nullptr, *qq = nullptr;
     int rc = acquire_tile_queue(&qkv);
     if (rc == SERAPH_OK) rc = acquire_tile_queue(&qq);
     if (rc != SERAPH_OK) return rc;
+    // The bound on the sequence length is the caller's word; the device checks it against the real offsets.  A
+    // launch number that the scratch cannot hold by accident marks "this launch overflowed its band".
+    static std::atomic<int> launch_counter{0};
+    const int epoch = (launch_counter.fetch_add(1) & 0x3fffffff) + 1;
+    const bool bound_can_fail = ds && (int64_t)ds_slots < ceil_div(T, 32) + 1;
+    hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)ceil_div(T, 4)), dim3(256), 0, st, dO, O, delta, T, H, seq_starts, batch, row_start,
+                       ds ? ds_slots : 0, epoch, overflow, qkv, qq);
+    SERAPH_LAUNCH_CHECK();
     const int per_cu = D <= 64 ? 2 : 1;
     constexpr int kv_per_cu = 1;                               // the dK/dV kernel's registers and LDS tiles leave room for one workgroup
     const int64_t kv_items = ceil_div(T, 128) * KVH;
@@ -1443,14 +1471,19 @@ static int run_backward(const float* Q, const float* K, const float* V, const fl
     if (ds) {
         if (ceil_div(T, 128) * H <= 2 * (int64_t)num_compute_units()) {        // short batch: see run_forward
             dim3 gds((unsigned)std::min<int64_t>(ceil_div(T, 64) * H, (int64_t)num_compute_units() * 2));
-            hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<D, true>), gds, dim3(kAttnThreads), 0, st, K, ds, dQ, seq_starts, batch, T, H, KVH, scale, ds_slots, qq);
+            hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<D, true>), gds, dim3(kAttnThreads), 0, st, K, ds, dQ, seq_starts, batch, T, H, KVH, scale, ds_slots, qq, overflow, epoch);
         } else {
             dim3 gds((unsigned)std::min<int64_t>(ceil_div(T, 128) * H, (int64_t)num_compute_units() * 2));
-            hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<D, false>), gds, dim3(kAttnThreads), 0, st, K, ds, dQ, seq_starts, batch, T, H, KVH, scale, ds_slots, qq);
+            hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<D, false>), gds, dim3(kAttnThreads), 0, st, K, ds, dQ, seq_starts, batch, T, H, KVH, scale, ds_slots, qq, overflow, epoch);
+        }
+        if (bound_can_fail) {                                   // stands down at once unless the delta kernel marked the launch
+            SERAPH_LAUNCH_CHECK();
+            hipLaunchKernelGGL(attn_bwd_dq_kernel<D>, gq, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dQ, seq_starts, batch,
+                               T, H, KVH, scale, scale * kLog2e, qq, (const int*)overflow, epoch);
         }
     } else {
         hipLaunchKernelGGL(attn_bwd_dq_kernel<D>, gq, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, dQ, seq_starts, batch,
-                           T, H, KVH, scale, scale * kLog2e, qq);
+                           T, H, KVH, scale, scale * kLog2e, qq, (const int*)nullptr, 0);
     }
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
@@ -1541,9 +1574,9 @@ int seraph_attention_backward_banded(const float* Q, const float* K, const float
         O = w.out; L = w.lse;
     }
     switch (head_dim) {
-        case 32: return run_backward<32>(Q, K, V, dO, O, L, w.delta, w.row_start, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, max_seq_len, ds, ds_slots, w.partK, w.partV, st);
-        case 64: return run_backward<64>(Q, K, V, dO, O, L, w.delta, w.row_start, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, max_seq_len, ds, ds_slots, w.partK, w.partV, st);
-        default: return run_backward<128>(Q, K, V, dO, O, L, w.delta, w.row_start, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, max_seq_len, ds, ds_slots, w.partK, w.partV, st);
+        case 32: return run_backward<32>(Q, K, V, dO, O, L, w.delta, w.row_start, w.overflow, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, max_seq_len, ds, ds_slots, w.partK, w.partV, st);
+        case 64: return run_backward<64>(Q, K, V, dO, O, L, w.delta, w.row_start, w.overflow, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, max_seq_len, ds, ds_slots, w.partK, w.partV, st);
+        default: return run_backward<128>(Q, K, V, dO, O, L, w.delta, w.row_start, w.overflow, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, max_seq_len, ds, ds_slots, w.partK, w.partV, st);
     }
 }
 

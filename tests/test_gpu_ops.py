@@ -442,6 +442,23 @@ def test_attention_backward_is_deterministic(ops):
     assert (a[1] == c[1]).all() and (a[2] == c[2]).all()      # dK, dV come from the same kernel either way
 
 
+@pytest.mark.parametrize("starts,H,KVH,D,bound", [([0, 700, 731, 1500], 4, 2, 64, 100), ([0, 513, 1030], 2, 1, 128, 300),
+                                                  ([0, 2100], 8, 8, 32, 64)])
+def test_attention_backward_with_a_bound_that_is_too_small(ops, orc, starts, H, KVH, D, bound):
+    """The caller's bound on the sequence length is shorter than a sequence: the device notices (the band of
+    dS tiles cannot hold the sequence), leaves the band unread and forms dQ with the recomputing kernel."""
+    Q, K, V, dO = _attn_inputs(6, starts, H, KVH, D)
+    su = np.array(starts, np.uint32)
+    sd = dev(su.view(np.int32)) if len(starts) > 2 else None
+    rdQ, rdK, rdV = orc.attention_backward(Q, K, V, dO, H, KVH, D, su)
+    assert bound < int(np.diff(starts).max())
+    for _ in range(2):                                       # twice: the mark of one launch must not leak into the next
+        dQ, dK, dV = ops.attention_backward(dev(Q), dev(K), dev(V), dev(dO), H, KVH, D, sd, max_seq_len=bound)
+        parity(dQ, rdQ, "dQ"); parity(dK, rdK, "dK"); parity(dV, rdV, "dV")
+    ok = ops.attention_backward(dev(Q), dev(K), dev(V), dev(dO), H, KVH, D, sd, max_seq_len=int(np.diff(starts).max()))
+    parity(ok[0], rdQ, "dQ after an overflowing launch")
+
+
 def test_attention_rejects_unsupported_head_dim(ops):
     from seraph_amd._lib import SeraphError
     Q = torch.zeros(8, 48, device="cuda")
