@@ -92,9 +92,11 @@ def reduce_sum(x):
     return out
 
 
-def matmul(A, B, M, N, K, tA=0, tB=0, C_in=None):
+def matmul(A, B, M, N, K, tA=0, tB=0, C_in=None, exact=False):
+    """exact: the plain double-accumulated loop nest whatever the size (orc_matmul switches to a
+    cache-blocked form for large products)."""
     out = np.zeros((M, N), np.float32) if C_in is None else C_in.copy()
-    lib().orc_matmul(_f(A), _f(B), _f(out), i64(M), i64(N), i64(K), C.c_int(tA), C.c_int(tB),
+    (lib().orc_matmul_exact if exact else lib().orc_matmul)(_f(A), _f(B), _f(out), i64(M), i64(N), i64(K), C.c_int(tA), C.c_int(tB),
                      C.c_int(0 if C_in is None else 1))
     return out
 

@@ -98,8 +98,94 @@ void orc_reduce_sum(const float* in, float* out, int64_t count) {
 /* GEMM                                                                   */
 /* ====================================================================== */
 
-void orc_matmul(const float* A, const float* B, float* C,
-                int64_t M, int64_t N, int64_t K, int tA, int tB, int accumulate) {
+/* Large products (the step at the benchmark widths) take a cache-blocked form of the same sum: C is cut into
+ * MB x NB tiles, K into runs of KB; inside a run the partial dot products are accumulated in FP32 with fused
+ * multiply-adds (one rounding per term), and the runs are added up in double, so the result is at least as
+ * accurate as an FP32 accumulation over all of K and far closer to the double sum than the tolerance of the
+ * parity tests.  orc_matmul_exact is the plain double-accumulated loop nest (every test of small shapes, and
+ * the check of the blocked form in tests/test_oracle_pins.py). */
+#include <immintrin.h>
+
+enum { GM_MR = 6, GM_NR = 16, GM_MB = 192, GM_NB = 256, GM_KB = 256 };
+
+/* acc[GM_MR][GM_NR] (double) += ap[k][GM_MR] * bp[k][GM_NR] over kb terms */
+static void gemm_micro(const float* ap, const float* bp, int kb, double* acc, int ldacc) {
+    __m256 c[GM_MR][2];
+    for (int i = 0; i < GM_MR; i++) { c[i][0] = _mm256_setzero_ps(); c[i][1] = _mm256_setzero_ps(); }
+    for (int k = 0; k < kb; k++) {
+        const __m256 b0 = _mm256_loadu_ps(bp + (size_t)k * GM_NR), b1 = _mm256_loadu_ps(bp + (size_t)k * GM_NR + 8);
+        for (int i = 0; i < GM_MR; i++) {
+            const __m256 a = _mm256_broadcast_ss(ap + (size_t)k * GM_MR + i);
+            c[i][0] = _mm256_fmadd_ps(a, b0, c[i][0]);
+            c[i][1] = _mm256_fmadd_ps(a, b1, c[i][1]);
+        }
+    }
+    for (int i = 0; i < GM_MR; i++) {
+        float t[GM_NR];
+        _mm256_storeu_ps(t, c[i][0]); _mm256_storeu_ps(t + 8, c[i][1]);
+        for (int j = 0; j < GM_NR; j++) acc[(size_t)i * ldacc + j] += (double)t[j];
+    }
+}
+
+static void matmul_blocked(const float* A, const float* B, float* C,
+                           int64_t M, int64_t N, int64_t K, int tA, int tB, int accumulate) {
+    const int64_t sai = tA ? 1 : K, sak = tA ? M : 1;      /* A(i,k) = A[i*sai + k*sak] */
+    const int64_t sbk = tB ? 1 : N, sbj = tB ? K : 1;      /* B(k,j) = B[k*sbk + j*sbj] */
+    const int64_t mt = (M + GM_MB - 1) / GM_MB, nt = (N + GM_NB - 1) / GM_NB;
+#pragma omp parallel
+    {
+        float* ap = (float*)aligned_alloc(64, sizeof(float) * GM_MB * GM_KB);
+        float* bp = (float*)aligned_alloc(64, sizeof(float) * GM_NB * GM_KB);
+        double* acc = (double*)malloc(sizeof(double) * GM_MB * GM_NB);
+#pragma omp for collapse(2) schedule(dynamic, 1)
+        for (int64_t ti = 0; ti < mt; ti++)
+            for (int64_t tj = 0; tj < nt; tj++) {
+                const int64_t i0 = ti * GM_MB, j0 = tj * GM_NB;
+                const int mb = (int)(M - i0 < GM_MB ? M - i0 : GM_MB), nb = (int)(N - j0 < GM_NB ? N - j0 : GM_NB);
+                memset(acc, 0, sizeof(double) * GM_MB * GM_NB);
+                for (int64_t k0 = 0; k0 < K; k0 += GM_KB) {
+                    const int kb = (int)(K - k0 < GM_KB ? K - k0 : GM_KB);
+                    /* panels of GM_MR rows of A and GM_NR columns of B, k-major inside a panel, zero padded */
+                    for (int pi = 0; pi < GM_MB / GM_MR; pi++) {
+                        float* dst = ap + (size_t)pi * GM_MR * GM_KB;
+                        if (pi * GM_MR >= mb) break;
+                        for (int k = 0; k < kb; k++)
+                            for (int i = 0; i < GM_MR; i++) {
+                                const int ii = pi * GM_MR + i;
+                                dst[(size_t)k * GM_MR + i] = ii < mb ? A[(i0 + ii) * sai + (k0 + k) * sak] : 0.0f;
+                            }
+                    }
+                    for (int pj = 0; pj < GM_NB / GM_NR; pj++) {
+                        float* dst = bp + (size_t)pj * GM_NR * GM_KB;
+                        if (pj * GM_NR >= nb) break;
+                        if (!tB && (pj + 1) * GM_NR <= nb) {
+                            for (int k = 0; k < kb; k++) memcpy(dst + (size_t)k * GM_NR, B + (k0 + k) * sbk + (j0 + pj * GM_NR), sizeof(float) * GM_NR);
+                        } else {
+                            for (int j = 0; j < GM_NR; j++) {
+                                const int jj = pj * GM_NR + j;
+                                if (jj < nb) { const float* src = B + (j0 + jj) * sbj + k0 * sbk; for (int k = 0; k < kb; k++) dst[(size_t)k * GM_NR + j] = src[(int64_t)k * sbk]; }
+                                else for (int k = 0; k < kb; k++) dst[(size_t)k * GM_NR + j] = 0.0f;
+                            }
+                        }
+                    }
+                    for (int pi = 0; pi * GM_MR < mb; pi++)
+                        for (int pj = 0; pj * GM_NR < nb; pj++)
+                            gemm_micro(ap + (size_t)pi * GM_MR * GM_KB, bp + (size_t)pj * GM_NR * GM_KB, kb,
+                                       acc + (size_t)pi * GM_MR * GM_NB + pj * GM_NR, GM_NB);
+                }
+                for (int i = 0; i < mb; i++) {
+                    float* crow = C + (i0 + i) * N + j0;
+                    const double* arow = acc + (size_t)i * GM_NB;
+                    if (accumulate) for (int j = 0; j < nb; j++) crow[j] = (float)((double)crow[j] + arow[j]);
+                    else            for (int j = 0; j < nb; j++) crow[j] = (float)arow[j];
+                }
+            }
+        free(ap); free(bp); free(acc);
+    }
+}
+
+void orc_matmul_exact(const float* A, const float* B, float* C,
+                      int64_t M, int64_t N, int64_t K, int tA, int tB, int accumulate) {
     /* Index expressions as shaders/matmul_transpose.comp:60-80. The loop nest
      * is arranged so the innermost stream is contiguous where it can be. */
 #pragma omp parallel
@@ -133,6 +219,14 @@ void orc_matmul(const float* A, const float* B, float* C,
         }
         free(acc);
     }
+}
+
+void orc_matmul(const float* A, const float* B, float* C,
+                int64_t M, int64_t N, int64_t K, int tA, int tB, int accumulate) {
+    if (M >= 32 && N >= 32 && (double)M * (double)N * (double)K >= 33554432.0)
+        matmul_blocked(A, B, C, M, N, K, tA, tB, accumulate);
+    else
+        orc_matmul_exact(A, B, C, M, N, K, tA, tB, accumulate);
 }
 
 /* ====================================================================== */
@@ -200,12 +294,17 @@ void orc_attention_backward(const float* Q, const float* K, const float* V,
         double* p  = (double*)malloc((size_t)T * sizeof(double));
         double* dp = (double*)malloc((size_t)T * sizeof(double));
         double* dq = (double*)malloc((size_t)D * sizeof(double));
-#pragma omp for schedule(dynamic, 1)
+        /* one (kv head, packed sequence) pair per task: the pairs touch disjoint rows of aK / aV */
+        const int nseq = seq_starts ? batch : 1;
+#pragma omp for collapse(2) schedule(dynamic, 1)
         for (int kvh = 0; kvh < KVH; kvh++) {
+          for (int sq = 0; sq < nseq; sq++) {
+            const int64_t t_lo = seq_starts ? (int64_t)seq_starts[sq] : 0;
+            const int64_t t_hi = seq_starts ? (int64_t)seq_starts[sq + 1] : T;
             for (int h = 0; h < H; h++) {
                 if (h * KVH / H != kvh) continue;    /* batch_attention_backward.comp:58 */
-                for (int64_t t = 0; t < T; t++) {
-                    int64_t j0 = seq_begin_of(seq_starts, batch, t);
+                for (int64_t t = t_lo; t < t_hi && t < T; t++) {
+                    int64_t j0 = t_lo;
                     const float* q  = Q  + t * qw + (int64_t)h * D;
                     const float* go = dO + t * qw + (int64_t)h * D;
                     double mx = -1e300;
@@ -246,6 +345,7 @@ void orc_attention_backward(const float* Q, const float* K, const float* V,
                     for (int d = 0; d < D; d++) dst[d] = (float)(dq[d] * (double)scale);
                 }
             }
+          }
         }
         free(p); free(dp); free(dq);
     }

@@ -58,6 +58,11 @@ void orc_reduce_sum(const float* in, float* out, int64_t count);
  * op(B) is B[K,N] or, transposed, B stored [N,K]. */
 void orc_matmul(const float* A, const float* B, float* C,
                 int64_t M, int64_t N, int64_t K, int tA, int tB, int accumulate);
+/* The same product as a plain loop nest with every term accumulated in double.  orc_matmul
+ * uses it for small shapes and a cache-blocked form (FP32 fused multiply-adds over runs of
+ * 256 terms, runs added in double) for large ones; the tests compare the two. */
+void orc_matmul_exact(const float* A, const float* B, float* C,
+                      int64_t M, int64_t N, int64_t K, int tA, int tB, int accumulate);
 
 /* ---- attention -------------------------------------------------------- */
 

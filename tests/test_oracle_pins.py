@@ -115,6 +115,39 @@ def test_matmul_all_forms(orc, tA, tB, acc):
     close(out, ref + (C0 if acc else 0), rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("tA", [0, 1])
+@pytest.mark.parametrize("tB", [0, 1])
+@pytest.mark.parametrize("acc", [False, True])
+def test_matmul_blocked_form_of_large_products(orc, tA, tB, acc):
+    """Large products take a cache-blocked loop order (FP32 fused multiply-adds over runs of 256 terms of K, runs added
+    in double).  Ragged against every block size (192 x 256 tiles, 6 x 16 panels, runs of 256); checked against
+    float64 numpy and against the plain double-accumulated loop nest."""
+    r = rng(40 + 4 * tA + 2 * tB + acc)
+    M, N, K = 391, 530, 777
+    assert M * N * K >= 1 << 25                                   # the size from which orc_matmul switches
+    A = r.standard_normal((K, M) if tA else (M, K)).astype(np.float32)
+    B = r.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+    C0 = r.standard_normal((M, N)).astype(np.float32)
+    out = orc.matmul(A, B, M, N, K, tA, tB, C0 if acc else None)
+    exact = orc.matmul(A, B, M, N, K, tA, tB, C0 if acc else None, exact=True)
+    ref = (A.T if tA else A).astype(np.float64) @ (B.T if tB else B).astype(np.float64) + (C0 if acc else 0)
+    close(exact, ref, rtol=1e-6, atol=1e-6)
+    # |sum of 777 products of N(0,1)| ~ 28 (up to ~100): FP32 runs of 256 terms leave errors of a few 1e-5 at most,
+    # 1e-6 of the magnitude, against a parity bar of 1e-4 of it
+    assert np.abs(out - ref).max() < 2e-4
+    assert np.linalg.norm(out - ref) / np.linalg.norm(ref) < 1e-6
+
+
+def test_matmul_blocked_form_integer_inputs_exact(orc):
+    """Integer-valued operands: every partial sum is exact in FP32, so the blocked form must be bit-exact."""
+    r = rng(41)
+    M, N, K = 300, 420, 600
+    A = r.integers(-5, 5, (M, K)).astype(np.float32)
+    B = r.integers(-5, 5, (N, K)).astype(np.float32)
+    out = orc.matmul(A, B, M, N, K, 0, 1)
+    assert (out == (A.astype(np.int64) @ B.astype(np.int64).T)).all()
+
+
 def test_matmul_reference_recipe_64cubed(orc):
     # tests/test_matmul.c:47-49: integers in [-5, 4], 64x64x64, NN
     r = rng(20)
