@@ -96,6 +96,12 @@ int seraph_cross_entropy_grad(const float* logits, const uint32_t* targets, floa
                               const uint32_t* seq_starts, int batch,
                               int64_t rows, int64_t cols, int64_t valid_rows, seraph_stream_t s);
 
+/* Rows beyond 32768 columns are shared out between workgroups that exchange their partial (max, sum) through
+ * device memory.  This bounds the wait for a partner, in polls of about 0.3 us (default 65536).  With 0 every
+ * workgroup computes its partners' statistics itself, which is the path a workgroup takes when a partner has not
+ * been scheduled: tests use it to run that path.  A negative value changes nothing.  No reference counterpart. */
+void seraph_cross_entropy_exchange_spins(int spins);
+
 /* ---------------------------------------------------------------- GEMM family */
 /* vulkan_matmul (include/vulkan_backend.h:431-433, shaders/matmul.comp) and
  * vulkan_matmul_transpose (include/vulkan_backend.h:439-442, shaders/matmul_transpose.comp:35-169):

@@ -1,18 +1,19 @@
-// cross_entropy.hip - fused softmax cross-entropy loss + gradient, one workgroup per row.
+// cross_entropy.hip - fused softmax cross-entropy loss + gradient.
 //
-// Two shapes of the same arithmetic (shaders/cross_entropy_grad.comp:44-98):
-//   * rows that fit the workgroup's registers (cols <= 32768) are read from HBM once;
-//   * longer rows (a 151936-entry vocabulary is 608 KB) are owned by one 512-lane workgroup that
-//     has a CU to itself: the first 77824 columns stay in its registers (38 float4 per lane), the
-//     next 32768 in its LDS (128 KB), and only what is left (27 % of that vocabulary) is read a
-//     second time, last-fetched-first while it is still cache resident.  HBM sees 2.27 passes
-//     instead of 3 (4.5 -> 4.06 ms at 16384 x 151936; a CU still idles while its one row is
-//     reduced, which is what separates this from the 3.5 ms the traffic alone would take);
+// Three shapes of the same arithmetic (shaders/cross_entropy_grad.comp:44-98):
+//   * rows that fit one workgroup's registers (cols <= 32768) are owned by one workgroup and read from HBM once;
+//   * longer rows (a 151936-entry vocabulary is 608 KB) are shared out between P workgroups that each keep their
+//     part in registers and exchange one (max, sum of exponentials) pair per row through device memory: every
+//     logit crosses HBM once in each direction (16384 x 151936: 3.44 ms, 5.8 TB/s; the earlier form that kept a
+//     row in one workgroup's registers and LDS and re-read a quarter of it took 4.05 ms);
 //   * unaligned or odd-length rows take an online max / sum-of-exponentials sweep and a second
 //     sweep in the opposite direction.
 // Rows without supervision (target >= cols, or the last token of a packed sequence)
 // are written as zeros without being read.  All offsets are 64-bit: rows*cols exceeds
 // 2^31 at the shapes this runs on.
+#include <atomic>
+#include <mutex>
+
 #include "common.hpp"
 
 namespace seraph {
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(BLOCK) void ce_small_kernel(const float* __restrict
     }
 }
 
-// ---------------------------------------------------------------- rows resident in registers + LDS
+// ---------------------------------------------------------------- helpers of the long-row kernel
 typedef float f4v __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float4 ld_stream4(const float4* p) {
     const f4v v = __builtin_nontemporal_load(reinterpret_cast<const f4v*>(p));
@@ -131,13 +132,9 @@ __device__ __forceinline__ float4 grad4(float4 a, float m, float inv_sum, float 
                        grad_of(a.z, m, inv_sum, scale, c + 2 == target), grad_of(a.w, m, inv_sum, scale, c + 3 == target));
 }
 
-constexpr int kResBlock = 512;           // 8 waves: two per SIMD, 256 registers each
-constexpr int kResVpt = 38;              // float4 per lane held in registers (152 of the 256 a lane has; 40 would spill)
-constexpr int kResLds4 = 8192;           // float4 held in LDS (128 KB)
-constexpr int kBatch = 8;                // independent loads in flight per lane outside the register part
 constexpr int kStreamAux = 2;            // buffer access cache policy: nontemporal
 
-// One row as a buffer: a scalar descriptor plus one 32-bit byte offset per lane, so the 40 register
+// One row as a buffer: a scalar descriptor plus one 32-bit byte offset per lane, so the register
 // slots need no address registers of their own; reads past the end of the row return zeros and
 // stores past it are dropped by the hardware.
 struct RowBuf {
@@ -192,133 +189,193 @@ __device__ __forceinline__ float block_reduce(float v, float* lds) {
     return r;
 }
 
-// cols % 4 == 0, 16-byte aligned rows of at most 2^29 columns.  Slot i4 of the row lives in registers
-// when i4 < BLOCK*VPT, in LDS when it is one of the next kResLds4, and is read twice otherwise.
-// The row maximum is found first; every resident logit is then turned into exp(x - max) once, in
-// place, and only scaled when it is stored (the overflow keeps the online form and pays a second
-// exponential).  A workgroup walks rows blockIdx.x, blockIdx.x + gridDim.x, ...; while it stores the
-// gradient of one row out of its registers it refills each register, and its LDS slots, with the same
-// slots of its next row, so a CU's loads and stores overlap although it holds one row at a time.
-__global__ __launch_bounds__(kResBlock) void ce_resident_kernel(const float* __restrict__ logits,
-                                                                const uint32_t* __restrict__ targets,
-                                                                float* __restrict__ grad, float* __restrict__ loss_rows,
-                                                                const uint32_t* __restrict__ seq_starts, int batch,
-                                                                int64_t rows, int64_t cols, float scale) {
-    __shared__ float4 stash[kResLds4];
-    __shared__ float red[2][kResBlock / 64];
-    constexpr int kReg4 = kResBlock * kResVpt;
-    constexpr int kSlotBytes = kResBlock * 16;               // distance between a lane's consecutive slots
+// ---------------------------------------------------------------- rows shared out between workgroups
+// A row is cut into chunks of 4 KB (one float4 per lane of a 256-lane workgroup); chunk c belongs to part c % P, and P
+// workgroups with consecutive indices hold one part each entirely in registers (kCoopVpt float4 per lane), so every
+// logit crosses HBM once in each direction and the partners sweep the row side by side.  Four workgroups share a CU
+// (while one reduces or waits for its partners the others stream; two of twice the size measured 3.65 ms against
+// 3.44).  A part's (max, sum of exponentials against that max) is published through a small record in device memory;
+// each workgroup combines its row's P records itself, in part order, so all of them derive the same maximum and total.
+//
+// The grid is persistent (a multiple of P workgroups, at most four per CU); workgroup g takes units g, g + G, ...
+// where unit u = (row u / P, part u % P): the P partners of a row work on it in the same round.  Records are
+// double-buffered by round parity and tagged (launch, round): a workgroup can only be one round ahead of a partner
+// it exchanges with, and a tag from another launch or round never matches.  The wait for a partner is bounded: past
+// the limit (a partner that has not been scheduled yet) the workgroup computes that part's statistics itself from
+// the logits, and takes the published ones instead if they have appeared meanwhile (the partner may by then be
+// overwriting its logits with the gradient when the call is in place; it publishes before it stores).
+constexpr int kCoopBlock = 256;
+constexpr int kCoopVpt = 19;                         // float4 per lane: 76 of the 128 registers a lane has at four workgroups per CU
+constexpr int kCoopWgsPerCu = 4;
+constexpr int kCoopMaxParts = 64;                     // one lane of the first wave per partner
+constexpr int kCoopMaxGrid = 2048;
+constexpr int kCoopLaunchSlots = 16;
+
+// Each word of a record validates itself: (statistic, half of a 64-bit hash of (launch, round)).  No ordering between
+// the two stores or the two loads is needed, hence no release/acquire fence (at device scope those write back and
+// invalidate whole caches on this part); the accesses are relaxed device-scope atomics, which go past the per-XCD L2s.
+struct CoopRec { unsigned long long max_word; unsigned long long sum_word; };
+static __device__ CoopRec g_ce_records[kCoopLaunchSlots][2][kCoopMaxGrid];
+
+__device__ __forceinline__ unsigned long long coop_tag(unsigned launch, unsigned round) {
+    unsigned long long z = (((unsigned long long)launch << 32) | round) + 0x9e3779b97f4a7c15ull;      // splitmix64
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+__device__ __forceinline__ void coop_publish(CoopRec* rec, float m, float sum, unsigned long long tag) {
+    __hip_atomic_store(&rec->max_word, (tag << 32) | __float_as_uint(m), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&rec->sum_word, (tag & 0xffffffff00000000ull) | __float_as_uint(sum), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool coop_try_read(const CoopRec* rec, unsigned long long tag, MaxSum* out) {
+    const unsigned long long a = __hip_atomic_load(&rec->max_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long b = __hip_atomic_load(&rec->sum_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((a >> 32) != (tag & 0xffffffffull) || (b >> 32) != (tag >> 32)) return false;
+    out->m = __uint_as_float((unsigned)a);
+    out->s = __uint_as_float((unsigned)b);
+    return true;
+}
+
+__global__ __launch_bounds__(kCoopBlock, kCoopWgsPerCu) void ce_coop_kernel(const float* __restrict__ logits,
+                                                               const uint32_t* __restrict__ targets,
+                                                               float* __restrict__ grad, float* __restrict__ loss_rows,
+                                                               const uint32_t* __restrict__ seq_starts, int batch,
+                                                               int64_t rows, int64_t cols, float scale, int P,
+                                                               CoopRec* __restrict__ recs, unsigned launch, int spin_limit,
+                                                               int in_place) {
+    __shared__ float red[2][kCoopBlock / 64];
+    __shared__ MaxSum redms[kCoopBlock / 64];
+    __shared__ MaxSum parts[kCoopMaxParts];
+    __shared__ unsigned long long missing;
+    __shared__ float bcast[2];
+    constexpr int kChunkBytes = kCoopBlock * 16;                   // one slot of every lane: 4 KB of the row
+    const int G = gridDim.x;
     const int n4 = (int)(cols >> 2);
-    const int lds_end = n4 < kReg4 + kResLds4 ? n4 : kReg4 + kResLds4;
+    const int nchunks = (n4 + kCoopBlock - 1) / kCoopBlock;
+    const int part = (int)(blockIdx.x % P), base_wg = (int)blockIdx.x - part;
+    // Chunk c of the row belongs to part c % P: the P partners sweep the row side by side, and slot k of this
+    // workgroup is chunk k P + part.  A slot whose chunk lies past the end of the row reads zeros and its store is
+    // dropped (the row is addressed as a buffer), so no slot needs a test of its own.
     const int lane_off = threadIdx.x * 16;
+    const int step_bytes = P * kChunkBytes, first_bytes = part * kChunkBytes;
     const float4 pad = make_float4(kNegBig, kNegBig, kNegBig, kNegBig);
+    const int64_t units = rows * P;
     auto is_live = [&](int64_t r) { return r < rows && (int64_t)targets[r] < cols && row_live(seq_starts, batch, r); };
 
-    // The LDS part travels memory -> LDS without passing through registers: lane l of a wave lands at
-    // the wave's base + 16 l, so a lane finds its own slots at stash[u * BLOCK + threadIdx.x].
-    typedef __attribute__((address_space(3))) void* lds_ptr;
-    auto fetch_stash = [&](const RowBuf& xb) {
-#pragma unroll
-        for (int u = 0; u < kResLds4 / kResBlock; u++) {
-            const int s4 = kReg4 + u * kResBlock;
-            if (s4 < lds_end)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(xb.rsrc, (lds_ptr)&stash[u * kResBlock + (threadIdx.x & ~63u)], 16, lane_off,
-                                                         s4 * 16, 0, kStreamAux);
-        }
-    };
-
-    float4 v[kResVpt];
-    bool loaded = false;                     // v and stash already hold (or are receiving) this row's resident part
-    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    float4 v[kCoopVpt];
+    bool loaded = false;
+    unsigned round = 0;
+    for (int64_t u = blockIdx.x; u < units; u += G, round++) {
+        const int64_t row = u / P;
         const RowBuf x(logits + row * cols, cols), g(grad + row * cols, cols);
         if (!is_live(row)) {
-            for (int b = 0; b * kResBlock < n4; b++) g.store(make_float4(0, 0, 0, 0), lane_off, b * kSlotBytes);
-            if (threadIdx.x == 0) loss_rows[row] = 0.0f;
+            for (int k = 0; k < kCoopVpt; k++) g.store(make_float4(0, 0, 0, 0), lane_off, first_bytes + k * step_bytes);
+            if (part == 0 && threadIdx.x == 0) loss_rows[row] = 0.0f;
             loaded = false;
             continue;
         }
         const uint32_t target = targets[row];
         if (!loaded) {
-#pragma unroll
-            for (int k = 0; k < kResVpt; k++) v[k] = x.load<kStreamAux>(lane_off, k * kSlotBytes);
-            fetch_stash(x);
-        }
-        // sweep 1, overflow: online (max, sum of exponentials), kBatch independent loads in flight per lane;
-        // read again in sweep 2, so kept cacheable
-        MaxSum ms;
-        ms.m = kNegBig;
-        ms.s = 0.0f;
-        for (int b4 = lds_end; b4 < n4; b4 += kBatch * kResBlock) {
-            float4 a[kBatch];
-#pragma unroll
-            for (int u = 0; u < kBatch; u++) a[u] = x.load<0>(lane_off, (b4 + u * kResBlock) * 16);
-            float cm = ms.m;
-#pragma unroll
-            for (int u = 0; u < kBatch; u++) {
-                if (b4 + u * kResBlock + (int)threadIdx.x >= n4) a[u] = pad;
-                cm = fmaxf(cm, max4(a[u]));
+            int off = first_bytes;                                // a running scalar offset, kept opaque so that the
+#pragma unroll                                                    // compiler does not hold one scalar register per slot
+            for (int k = 0; k < kCoopVpt; k++) {
+                v[k] = x.load<kStreamAux>(lane_off, off);
+                off += step_bytes;
+                asm volatile("" : "+s"(off));
             }
-            if (cm > ms.m) { ms.s *= __expf(ms.m - cm); ms.m = cm; }
-            const float mc = ms.m * kLog2e;
-            float acc = 0.0f;
-#pragma unroll
-            for (int u = 0; u < kBatch; u++) acc += sum4(exp4(a[u], mc));       // padding adds exp(-huge) = 0
-            ms.s += acc;
         }
-        // Everything requested has landed: the register part and, written straight into LDS, this lane's
-        // own stash slots.  (Explicit: the wait count the compiler derives for v[] does not include the
-        // LDS-bound loads issued after them.)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // the target's logit, read by the part that owns it before any of this workgroup's stores (grad may alias logits)
+        const bool owns_target = ((int)(target >> 2) / kCoopBlock) % P == part;
+        float xt = 0.0f;
+        if (owns_target && threadIdx.x == 0) xt = logits[row * cols + target];
         float mx = kNegBig;
+        {
+            int room = n4 - part * kCoopBlock;                    // float4 slots from this chunk's start to the end of the row
 #pragma unroll
-        for (int k = 0; k < kResVpt; k++) {
-            if ((int)threadIdx.x + kResBlock * k >= n4) v[k] = pad;
-            mx = fmaxf(mx, max4(v[k]));
+            for (int k = 0; k < kCoopVpt; k++) {
+                if ((int)threadIdx.x >= room) v[k] = pad;         // past the end (read as zeros): out of the maximum and the sum
+                mx = fmaxf(mx, max4(v[k]));
+                room -= P * kCoopBlock;
+                asm volatile("" : "+s"(room));
+            }
         }
-        for (int i4 = kReg4 + threadIdx.x; i4 < lds_end; i4 += kResBlock) mx = fmaxf(mx, max4(stash[i4 - kReg4]));
-        const float m = block_reduce<kResBlock, true>(fmaxf(mx, ms.m), red[0]);
-        const float mc = m * kLog2e;
-        // every resident logit becomes exp(x - m), once
-        float sum = ms.s * __expf(ms.m - m);
+        MaxSum mine;
+        mine.m = block_reduce<kCoopBlock, true>(mx, red[0]);
+        const float mc = mine.m * kLog2e;
+        float sum = 0.0f;
 #pragma unroll
-        for (int k = 0; k < kResVpt; k++) { v[k] = exp4(v[k], mc); sum += sum4(v[k]); }
-        for (int i4 = kReg4 + threadIdx.x; i4 < lds_end; i4 += kResBlock) {
-            const float4 e = exp4(stash[i4 - kReg4], mc);
-            stash[i4 - kReg4] = e;
-            sum += sum4(e);
-        }
-        const float total = block_reduce<kResBlock, false>(sum, red[1]);
-        const float k_out = scale / total;
-        if (threadIdx.x == 0) loss_rows[row] = -((logits[row * cols + target] - m) - __logf(total));
-        __syncthreads();                     // grad may alias logits: the target logit is read before any store
+        for (int k = 0; k < kCoopVpt; k++) { v[k] = exp4(v[k], mc); sum += sum4(v[k]); }    // padding: exp(-huge) = 0
+        mine.s = block_reduce<kCoopBlock, false>(sum, red[1]);
 
-        // sweep 2: the overflow first (most recently fetched first), then LDS, then registers
-        for (int e4 = n4; e4 > lds_end; e4 -= kBatch * kResBlock) {
-            float4 a[kBatch];
-#pragma unroll
-            for (int u = 0; u < kBatch; u++) {
-                const int s4 = e4 - (u + 1) * kResBlock;                      // may reach below lds_end: masked below
-                a[u] = x.load<0>(lane_off, (s4 < 0 ? 0 : s4) * 16);
+        float m = mine.m, total = mine.s;
+        if (P > 1) {
+            const unsigned long long tag = coop_tag(launch, round);
+            CoopRec* mine_rec = recs + (size_t)(round & 1u) * kCoopMaxGrid;
+            if (threadIdx.x == 0) {
+                missing = 0ull;
+                coop_publish(mine_rec + blockIdx.x, mine.m, mine.s, tag);
+                // In place the gradient will overwrite this part's logits: the record has to be out before that, for a
+                // partner that gave up waiting and is reading these logits (it looks at the record again afterwards).
+                if (in_place) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             }
-#pragma unroll
-            for (int u = 0; u < kBatch; u++) {
-                const int s4 = e4 - (u + 1) * kResBlock;
-                const int i4 = s4 + (int)threadIdx.x;
-                if (i4 >= lds_end && i4 < n4) g.store(finish4(exp4(a[u], mc), k_out, scale, i4, target), lane_off, s4 * 16);
+            __syncthreads();
+            if (threadIdx.x < (unsigned)P) {                      // one lane per partner (its own part included)
+                const CoopRec* rec = mine_rec + base_wg + threadIdx.x;
+                MaxSum got;
+                bool ok = coop_try_read(rec, tag, &got);
+                for (int spin = 0; !ok && spin < spin_limit; spin++) {
+                    __builtin_amdgcn_s_sleep(4);
+                    ok = coop_try_read(rec, tag, &got);
+                }
+                if (ok) parts[threadIdx.x] = got;
+                else atomicOr(&missing, 1ull << threadIdx.x);
             }
+            __syncthreads();
+            unsigned long long todo = missing;
+            while (todo) {                                        // uniform across the workgroup
+                const int p = __builtin_ctzll(todo);
+                todo &= todo - 1;
+                // that part's statistics from its logits, with the whole workgroup
+                const float4* src = reinterpret_cast<const float4*>(logits + row * cols);
+                MaxSum ms;
+                ms.m = kNegBig; ms.s = 0.0f;
+                for (int c = p; c < nchunks; c += P) {
+                    const int i4 = c * kCoopBlock + (int)threadIdx.x;
+                    if (i4 < n4) {
+                        const float4 a = src[i4];
+                        const float cm = max4(a);
+                        if (cm > ms.m) { ms.s *= __expf(ms.m - cm); ms.m = cm; }
+                        ms.s += sumexp4(a, ms.m);
+                    }
+                }
+                ms = block_combine<kCoopBlock>(ms, redms);
+                if (threadIdx.x == 0) {                           // (the barrier inside block_combine: every lane's loads have returned)
+                    MaxSum got;
+                    parts[p] = coop_try_read(mine_rec + base_wg + p, tag, &got) ? got : ms;
+                }
+                __syncthreads();
+            }
+            if (threadIdx.x < 64) {                               // first wave: combine in part order
+                MaxSum r = parts[0];
+                for (int p = 1; p < P; p++) r = combine(r, parts[p]);
+                if (threadIdx.x == 0) { bcast[0] = r.m; bcast[1] = r.s; }
+            }
+            __syncthreads();
+            m = bcast[0]; total = bcast[1];
         }
-        for (int i4 = kReg4 + threadIdx.x; i4 < lds_end; i4 += kResBlock)
-            g.store(finish4(stash[i4 - kReg4], k_out, scale, i4, target), lane_off, (i4 - (int)threadIdx.x) * 16);
-        const int64_t next = row + gridDim.x;
-        const bool refill = is_live(next);
-        const RowBuf xn(logits + (refill ? next : row) * cols, cols);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this row's LDS slots have been read: they may be overwritten
-        if (refill) fetch_stash(xn);
+        const float k_out = (scale / total) * __expf(mine.m - m);
+        if (owns_target && threadIdx.x == 0) loss_rows[row] = -((xt - m) - __logf(total));
+
+        const int64_t next = u + G;
+        const bool refill = next < units && is_live(next / P);
+        const RowBuf xn(logits + (refill ? next / P : row) * cols, cols);
+        int off = first_bytes, i4 = part * kCoopBlock + (int)threadIdx.x;
 #pragma unroll
-        for (int k = 0; k < kResVpt; k++) {
-            const int i4 = threadIdx.x + kResBlock * k;
-            g.store(finish4(v[k], k_out, scale, i4, target), lane_off, k * kSlotBytes);   // dropped past the row's end
-            if (refill) v[k] = xn.load<kStreamAux>(lane_off, k * kSlotBytes);
+        for (int k = 0; k < kCoopVpt; k++) {
+            g.store(finish4(v[k], k_out, scale, i4, target), lane_off, off);   // dropped past the row's end
+            if (refill) v[k] = xn.load<kStreamAux>(lane_off, off);
+            off += step_bytes; i4 += P * kCoopBlock;
+            asm volatile("" : "+s"(off));
         }
         loaded = refill;
     }
@@ -413,9 +470,28 @@ __global__ __launch_bounds__(BLOCK) void ce_stream_kernel(const float* __restric
     }
 }
 
+// device address of the exchange records on the current device
+static int coop_records(CoopRec** out) {
+    static std::mutex mu;
+    static CoopRec* base[64] = {nullptr};
+    int dev = 0;
+    SERAPH_HIP_CHECK(hipGetDevice(&dev));
+    SERAPH_REQUIRE(dev >= 0 && dev < 64, "device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lk(mu);
+    if (!base[dev]) SERAPH_HIP_CHECK(hipGetSymbolAddress((void**)&base[dev], HIP_SYMBOL(g_ce_records)));
+    *out = base[dev];
+    return SERAPH_OK;
+}
+
+static int g_ce_spin_limit = 1 << 16;     // waits of ~0.3 us each: several milliseconds before a partner is given up on
+
 }  // namespace seraph
 
 using namespace seraph;
+
+extern "C" void seraph_cross_entropy_exchange_spins(int spins) {
+    if (spins >= 0) g_ce_spin_limit = spins;
+}
 
 extern "C" int seraph_cross_entropy_grad(const float* logits, const uint32_t* targets, float* grad, float* loss_rows,
                                          const uint32_t* seq_starts, int batch,
@@ -439,10 +515,22 @@ extern "C" int seraph_cross_entropy_grad(const float* logits, const uint32_t* ta
         else if (n4 <= 4096) SMALL(16);
         else SMALL(32);
 #undef SMALL
-    } else if (vec && cols <= ((int64_t)1 << 29)) {
-        const int64_t cus = num_compute_units();          // one workgroup fills a CU's registers and LDS
-        hipLaunchKernelGGL(ce_resident_kernel, dim3((unsigned)(rows < cus ? rows : cus)), dim3(kResBlock), 0, st, logits, targets,
-                           grad, loss_rows, seq_starts, batch, rows, cols, scale);
+    } else if (vec && ceil_div(ceil_div(cols / 4, kCoopBlock), kCoopVpt) <= kCoopMaxParts) {
+        // rows cut into P register-resident parts: one pass over HBM
+        const int P = (int)ceil_div(ceil_div(cols / 4, kCoopBlock), kCoopVpt);
+        int64_t G = (int64_t)num_compute_units() * kCoopWgsPerCu;
+        if (G > kCoopMaxGrid) G = kCoopMaxGrid;
+        G = (G / P) * P;
+        if (G > rows * P) G = rows * P;
+        static std::atomic<unsigned> launches{0};
+        unsigned launch = launches.fetch_add(1) + 1;
+        if (launch == 0) launch = launches.fetch_add(1) + 1;      // a zeroed record must never look published
+        CoopRec* recs = nullptr;
+        int rc = coop_records(&recs);
+        if (rc != SERAPH_OK) return rc;
+        recs += (size_t)(launch % kCoopLaunchSlots) * 2 * kCoopMaxGrid;
+        hipLaunchKernelGGL(ce_coop_kernel, dim3((unsigned)G), dim3(kCoopBlock), 0, st, logits, targets, grad, loss_rows,
+                           seq_starts, batch, rows, cols, scale, P, recs, launch, g_ce_spin_limit, grad == logits ? 1 : 0);
     } else if (vec) {
         // Rows in flight are re-read by the second sweep: keep their total under the last-level cache.
         // Two 1024-lane workgroups fit a CU; when that many long rows would overflow the cache, an

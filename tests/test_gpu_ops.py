@@ -94,7 +94,7 @@ def test_fill_nan_reduce(ops, orc):
 
 
 # ------------------------------------------------------------------ cross entropy
-@pytest.mark.parametrize("rows,cols", [(9, 8192), (5, 1000), (4, 40000), (3, 33001), (2, 151936), (6, 4)])
+@pytest.mark.parametrize("rows,cols", [(9, 8192), (5, 1000), (4, 40000), (3, 33001), (2, 151936), (6, 4), (1030, 32772), (3, 1300000)])
 def test_cross_entropy_grad(ops, orc, rows, cols):
     r = rng(rows * 100003 + cols)
     x = (2 * r.standard_normal((rows, cols))).astype(np.float32)
@@ -487,9 +487,34 @@ def test_rope_qk_equals_two_rope_calls(ops, packed, D):
         assert torch.equal(q1, q2) and torch.equal(k1, k2)
 
 
-@pytest.mark.parametrize("rows,cols", [(4, 40000), (3, 151936), (300, 151936)])
+@pytest.mark.parametrize("spins", [0, 3])
+def test_cross_entropy_long_rows_when_partners_are_not_waited_for(ops, orc, spins):
+    """Long rows are shared out between workgroups that exchange (max, sum) through device memory.  With the wait
+    bounded to nothing (or next to nothing) a workgroup computes its partners' statistics itself from the logits, as it
+    would for a partner that has not been scheduled: same results, also in place and with unsupervised rows."""
+    from seraph_amd._lib import kernels
+    r = rng(91)
+    try:
+        kernels().seraph_cross_entropy_exchange_spins(spins)
+        for rows, cols in ((5, 40000), (9, 151936), (1100, 36000)):
+            x = (2 * r.standard_normal((rows, cols))).astype(np.float32)
+            t = r.integers(0, cols, rows).astype(np.uint32)
+            t[1] = cols
+            starts = np.array([0, 3, rows], np.uint32)
+            rg, rl = orc.cross_entropy_grad_packed(x, t, starts, rows - 3)
+            sd = dev(starts.view(np.int32))
+            g, l = ops.cross_entropy_grad(dev(x), dev(t.view(np.int32)), rows - 3, seq_starts=sd)
+            parity(g, rg, "grad", atol=1e-7); parity(l, rl, "loss")
+            X = dev(x)
+            g2, l2 = ops.cross_entropy_grad(X, dev(t.view(np.int32)), rows - 3, seq_starts=sd, grad=X)
+            parity(g2, rg, "grad in place", atol=1e-7); parity(l2, rl, "loss in place")
+    finally:
+        kernels().seraph_cross_entropy_exchange_spins(1 << 16)
+
+
+@pytest.mark.parametrize("rows,cols", [(4, 40000), (3, 151936), (300, 151936), (2100, 77828), (40, 1000000)])
 def test_cross_entropy_long_rows_are_deterministic_and_alias_safe(ops, rows, cols):
-    """Rows kept in registers and LDS: repeated runs and the in-place form (grad over logits) give identical bits."""
+    """Rows shared out between workgroups: repeated runs and the in-place form (grad over logits) give identical bits."""
     torch.manual_seed(rows + cols)
     x = torch.randn(rows, cols, device="cuda") * 2
     t = torch.randint(0, cols, (rows,), device="cuda", dtype=torch.int32)
