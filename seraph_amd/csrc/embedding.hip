@@ -2,11 +2,12 @@
 //
 // shaders/embedding_backward.comp:22-44 adds every element of dH into the table with a
 // compare-and-swap loop, so rows of repeated tokens serialise and the summation order
-// changes from run to run.  Here positions are grouped by token first (count, exclusive
-// scan, fill, in-group rank - all integer work, O(T + vocab)); then one workgroup per
-// touched row adds that row's positions in ascending order and performs a single
-// read-modify-write of the table row.  HBM traffic: dH once, each touched row once in
-// and once out.
+// changes from run to run.  Here every position joins its token's chain with one exchange on a
+// per-token table (integer work; the chain's order is arbitrary), the one position of each token that
+// found the chain empty becomes the token's owner, and one wavefront per owner gathers the token's
+// positions, puts them in ascending order and adds their rows of dH in that order, with a single
+// read-modify-write of the table row.  Three launches; HBM traffic: dH once, each touched row once in and
+// once out.  The sum does not depend on the order in which positions joined, so reruns are bit-identical.
 #include "common.hpp"
 
 namespace seraph {
@@ -30,176 +31,188 @@ __global__ __launch_bounds__(256) void embed_lookup_kernel(const uint32_t* __res
     }
 }
 
-// ---------------------------------------------------------------- backward: grouping
+// ---------------------------------------------------------------- backward
+constexpr uint32_t kNil = 0xffffffffu;
 struct EmbWs {
-    uint32_t* cnt;      // [vocab + 1]  per-token count, then fill cursor
-    uint32_t* off;      // [vocab + 1]  exclusive scan of cnt
-    uint32_t* uniq;     // [T]          tokens that occur, ascending
-    uint32_t* nuniq;    // [1]
-    uint32_t* perm;     // [T]          positions grouped by token, arbitrary order inside a group
-    uint32_t* sorted;   // [T]          the same, ascending inside each group
-    uint32_t* csum;     // [chunks]     per-chunk count totals, then bases
-    uint32_t* cnz;      // [chunks]     per-chunk distinct-token totals, then bases
+    uint2* tab;         // [vocab]  x = most recent position that joined the token's chain (kNil: none), y = positions so far
+    uint32_t* link;     // [T]      the position that had joined the same token's chain before this one; kNil for the first
 };
 
 static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 
 static size_t emb_ws_layout(int64_t T, int64_t vocab, char* base, EmbWs* w) {
     size_t o = 0;
-    auto take = [&](size_t count) { uint32_t* p = (uint32_t*)(base + o); o += align_up(count * 4); return p; };
-    uint32_t* cnt = take((size_t)vocab + 1);
-    uint32_t* off = take((size_t)vocab + 1);
-    uint32_t* uniq = take((size_t)T);
-    uint32_t* nuniq = take(1);
-    uint32_t* perm = take((size_t)T);
-    uint32_t* sorted = take((size_t)T);
-    const size_t chunks = (size_t)((vocab + 4095) / 4096);
-    uint32_t* csum = take(chunks);
-    uint32_t* cnz = take(chunks);
-    if (w) { w->csum = csum; w->cnz = cnz; w->cnt = cnt; w->off = off; w->uniq = uniq; w->nuniq = nuniq; w->perm = perm; w->sorted = sorted; }
+    char* tab = base + o; o += align_up((size_t)vocab * 8);
+    char* link = base + o; o += align_up((size_t)T * 4);
+    if (w) { w->tab = (uint2*)tab; w->link = (uint32_t*)link; }
     return o;
 }
 
-__global__ __launch_bounds__(256) void emb_count_kernel(const uint32_t* __restrict__ tokens, uint32_t* cnt,
-                                                        int64_t T, int64_t vocab) {
-    int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (p < T && (int64_t)tokens[p] < vocab) atomicAdd(&cnt[tokens[p]], 1u);     // integer: order-independent
+__global__ __launch_bounds__(256) void emb_init_kernel(uint2* __restrict__ tab, int64_t vocab) {
+    const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (v < vocab) tab[v] = make_uint2(kNil, 0u);
 }
 
-// Exclusive scan of the per-token counts over the vocabulary in three small launches:
-// per-chunk totals (4096 tokens per workgroup, coalesced 16-byte loads), a serial scan of the
-// few chunk totals, then a rescan of every chunk from its base.  The last pass writes
-// off = exclusive scan(cnt) and uniq = tokens with cnt > 0 in ascending order, and clears cnt
-// so the fill kernel can reuse it as a cursor.
-constexpr int kScanBlock = 1024;
-constexpr int kScanChunk = 4 * kScanBlock;
-
-__device__ __forceinline__ uint4 load_cnt4(const uint32_t* cnt, int64_t v0, int64_t vocab) {
-    uint4 c = make_uint4(0, 0, 0, 0);
-    if (v0 + 3 < vocab && ((v0 & 3) == 0)) return *reinterpret_cast<const uint4*>(cnt + v0);
-    if (v0 < vocab) c.x = cnt[v0];
-    if (v0 + 1 < vocab) c.y = cnt[v0 + 1];
-    if (v0 + 2 < vocab) c.z = cnt[v0 + 2];
-    if (v0 + 3 < vocab) c.w = cnt[v0 + 3];
-    return c;
-}
-
-__global__ __launch_bounds__(kScanBlock) void emb_chunk_sums_kernel(const uint32_t* __restrict__ cnt, int64_t vocab,
-                                                                    uint32_t* __restrict__ csum, uint32_t* __restrict__ cnz) {
-    __shared__ uint32_t s_sum[kScanBlock / 64], s_nz[kScanBlock / 64];
-    const int64_t v0 = (int64_t)blockIdx.x * kScanChunk + 4 * threadIdx.x;
-    const uint4 c = load_cnt4(cnt, v0, vocab);
-    uint32_t sum = c.x + c.y + c.z + c.w;
-    uint32_t nz = (c.x ? 1u : 0u) + (c.y ? 1u : 0u) + (c.z ? 1u : 0u) + (c.w ? 1u : 0u);
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) { sum += __shfl_xor(sum, o, 64); nz += __shfl_xor(nz, o, 64); }
-    if ((threadIdx.x & 63) == 0) { s_sum[threadIdx.x >> 6] = sum; s_nz[threadIdx.x >> 6] = nz; }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t a = 0, b = 0;
-        for (int w = 0; w < kScanBlock / 64; w++) { a += s_sum[w]; b += s_nz[w]; }
-        csum[blockIdx.x] = a;
-        cnz[blockIdx.x] = b;
-    }
-}
-
-// chunk totals -> exclusive chunk bases (in place); also off[vocab] and the number of distinct tokens
-__global__ void emb_chunk_scan_kernel(uint32_t* csum, uint32_t* cnz, int nchunks, uint32_t* off, uint32_t* nuniq, int64_t vocab) {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    uint32_t a = 0, b = 0;
-    for (int i = 0; i < nchunks; i++) {
-        uint32_t x = csum[i], y = cnz[i];
-        csum[i] = a; cnz[i] = b;
-        a += x; b += y;
-    }
-    off[vocab] = a;
-    *nuniq = b;
-}
-
-__global__ __launch_bounds__(kScanBlock) void emb_chunk_write_kernel(uint32_t* __restrict__ cnt, int64_t vocab,
-                                                                     const uint32_t* __restrict__ csum,
-                                                                     const uint32_t* __restrict__ cnz,
-                                                                     uint32_t* __restrict__ off, uint32_t* __restrict__ uniq) {
-    __shared__ uint32_t s_sum[kScanBlock], s_nz[kScanBlock];
-    const int tid = threadIdx.x;
-    const int64_t v0 = (int64_t)blockIdx.x * kScanChunk + 4 * tid;
-    const uint4 c = load_cnt4(cnt, v0, vocab);
-    const uint32_t sum = c.x + c.y + c.z + c.w;
-    const uint32_t nz = (c.x ? 1u : 0u) + (c.y ? 1u : 0u) + (c.z ? 1u : 0u) + (c.w ? 1u : 0u);
-    s_sum[tid] = sum; s_nz[tid] = nz;
-    __syncthreads();
-    for (int d = 1; d < kScanBlock; d <<= 1) {                 // Hillis-Steele inclusive scan
-        uint32_t a = tid >= d ? s_sum[tid - d] : 0u, b = tid >= d ? s_nz[tid - d] : 0u;
-        __syncthreads();
-        s_sum[tid] += a; s_nz[tid] += b;
-        __syncthreads();
-    }
-    uint32_t run = csum[blockIdx.x] + s_sum[tid] - sum;         // exclusive prefix of this lane's four tokens
-    uint32_t urun = cnz[blockIdx.x] + s_nz[tid] - nz;
-    const uint32_t cs[4] = {c.x, c.y, c.z, c.w};
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        const int64_t v = v0 + e;
-        if (v < vocab) {
-            off[v] = run;
-            if (cs[e]) uniq[urun++] = (uint32_t)v;
-            run += cs[e];
-            cnt[v] = 0;
-        }
-    }
-}
-
-__global__ __launch_bounds__(256) void emb_fill_kernel(const uint32_t* __restrict__ tokens, uint32_t* cnt,
-                                                       const uint32_t* __restrict__ off, uint32_t* perm,
+__global__ __launch_bounds__(256) void emb_link_kernel(const uint32_t* __restrict__ tokens, uint2* tab, uint32_t* __restrict__ link,
                                                        int64_t T, int64_t vocab) {
-    int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (p >= T) return;
-    uint32_t tok = tokens[p];
-    if ((int64_t)tok >= vocab) return;
-    perm[off[tok] + atomicAdd(&cnt[tok], 1u)] = (uint32_t)p;
+    const uint32_t tok = tokens[p];
+    if ((int64_t)tok >= vocab) { link[p] = 0u; return; }      // skipped position (embedding_backward.comp:31): owns nothing (its token is checked again)
+    atomicAdd(&tab[tok].y, 1u);
+    link[p] = atomicExch(&tab[tok].x, (uint32_t)p);
 }
 
-// Rank of each position inside its group: makes the order independent of the fill race.
-__global__ __launch_bounds__(256) void emb_rank_kernel(const uint32_t* __restrict__ tokens,
-                                                       const uint32_t* __restrict__ off,
-                                                       const uint32_t* __restrict__ perm, uint32_t* sorted,
-                                                       int64_t vocab) {
-    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= (int64_t)off[vocab]) return;
-    uint32_t p = perm[i], tok = tokens[p];
-    uint32_t lo = off[tok], hi = off[tok + 1], rank = 0;
-    for (uint32_t q = lo; q < hi; q++) rank += perm[q] < p ? 1u : 0u;
-    sorted[lo + rank] = p;
-}
+// One wavefront per position; only a token's owner (the position whose exchange found the chain empty) works.
+// The owner's own row of dH is requested before anything is known about the token, the table row as soon as the
+// token is: for a token that occurs once, which is most of them, two dependent loads precede the payload.
+constexpr int kEmbList = 1024;          // positions gathered per batch
+constexpr int kEmbWalk = 16;            // up to this many positions the chain is walked; longer groups are found by scanning the tokens
+constexpr int kEmbVpl = 8;              // float4 per lane and pass: 2048 floats of a row
 
-__global__ __launch_bounds__(256) void emb_sum_kernel(const uint32_t* __restrict__ uniq,
-                                                      const uint32_t* __restrict__ nuniq,
-                                                      const uint32_t* __restrict__ off,
-                                                      const uint32_t* __restrict__ sorted,
-                                                      const float* __restrict__ dH, float* __restrict__ grad_embed,
-                                                      int64_t hidden, int vec) {
-    if (blockIdx.x >= *nuniq) return;
-    const uint32_t tok = uniq[blockIdx.x];
-    const uint32_t lo = off[tok], hi = off[tok + 1];
-    float* row = grad_embed + (int64_t)tok * hidden;
+__global__ __launch_bounds__(64) void emb_sum_kernel(const uint32_t* __restrict__ tokens, const uint2* __restrict__ tab,
+                                                     const uint32_t* __restrict__ link,
+                                                     const float* __restrict__ dH, float* __restrict__ grad_embed,
+                                                     int64_t T, int64_t hidden, int64_t vocab, int vec) {
+    __shared__ uint32_t list[kEmbList], tmp[kEmbWalk];
+    const int lane = threadIdx.x;
+    const int64_t p = blockIdx.x;
+    const int64_t n4 = hidden >> 2;
+    // speculative: the first pass of this position's own row
+    float4 own[kEmbVpl];
     if (vec) {
-        const int64_t n4 = hidden >> 2;
-        for (int64_t i = threadIdx.x; i < n4; i += 256) {
-            float4 a = make_float4(0, 0, 0, 0);
-            for (uint32_t q = lo; q < hi; q++) {
-                float4 g = reinterpret_cast<const float4*>(dH + (int64_t)sorted[q] * hidden)[i];
-                a.x += g.x; a.y += g.y; a.z += g.z; a.w += g.w;
+#pragma unroll
+        for (int k = 0; k < kEmbVpl; k++) {
+            const int64_t i = lane + 64 * k;
+            own[k] = i < n4 ? reinterpret_cast<const float4*>(dH + p * hidden)[i] : make_float4(0, 0, 0, 0);
+        }
+    }
+    const uint32_t tok = tokens[p];
+    const uint32_t lk = link[p];
+    if ((int64_t)tok >= vocab || lk != kNil) return;
+    float* row = grad_embed + (int64_t)tok * hidden;
+    float4 old[kEmbVpl];
+    if (vec) {
+#pragma unroll
+        for (int k = 0; k < kEmbVpl; k++) {
+            const int64_t i = lane + 64 * k;
+            old[k] = i < n4 ? reinterpret_cast<const float4*>(row)[i] : make_float4(0, 0, 0, 0);
+        }
+    }
+    const uint2 e = tab[tok];
+    const uint32_t count = e.y;
+
+    if (count == 1 && vec) {                                   // the common case: nothing to gather
+#pragma unroll
+        for (int k = 0; k < kEmbVpl; k++) {
+            const int64_t i = lane + 64 * k;
+            if (i < n4) reinterpret_cast<float4*>(row)[i] = make_float4(old[k].x + own[k].x, old[k].y + own[k].y, old[k].z + own[k].z, old[k].w + own[k].w);
+        }
+        for (int64_t i0 = 64 * kEmbVpl; i0 < n4; i0 += 64) {   // rows wider than one pass
+            const int64_t i = i0 + lane;
+            if (i < n4) {
+                const float4 g = reinterpret_cast<const float4*>(dH + p * hidden)[i];
+                float4 r = reinterpret_cast<float4*>(row)[i];
+                r.x += g.x; r.y += g.y; r.z += g.z; r.w += g.w;
+                reinterpret_cast<float4*>(row)[i] = r;
             }
-            float4 r = reinterpret_cast<float4*>(row)[i];
-            r.x += a.x; r.y += a.y; r.z += a.z; r.w += a.w;
-            reinterpret_cast<float4*>(row)[i] = r;
         }
-    } else {
-        for (int64_t i = threadIdx.x; i < hidden; i += 256) {
-            float a = 0.0f;
-            for (uint32_t q = lo; q < hi; q++) a += dH[(int64_t)sorted[q] * hidden + i];
-            row[i] += a;
+        return;
+    }
+
+    // The token's positions in ascending order, a batch of at most kEmbList at a time.  Short chains are walked (one
+    // dependent load per position) and ranked; long ones are found by sweeping the token array from the smallest
+    // position on, which costs T / count loads per position found.
+    int64_t cursor = 0;                                        // scan: next token index to look at
+    uint32_t found = 0;
+    bool first_batch = true;
+    while (found < count) {
+        int len = 0;
+        if (count <= (uint32_t)kEmbWalk) {
+            if (lane == 0) {
+                uint32_t q = e.x;
+                for (uint32_t i = 0; i < count; i++) { tmp[i] = q; q = link[q]; }
+            }
+            __syncthreads();
+            if (lane < (int)count) {
+                const uint32_t mine = tmp[lane];
+                int rank = 0;
+                for (uint32_t j = 0; j < count; j++) rank += tmp[j] < mine ? 1 : 0;
+                list[rank] = mine;
+            }
+            len = (int)count;
+        } else {
+            constexpr int U = 8;                               // token loads in flight per lane
+            while (len + 64 * U <= kEmbList && cursor < T && found + (uint32_t)len < count) {
+                uint32_t tk[U];
+#pragma unroll
+                for (int j = 0; j < U; j++) {
+                    const int64_t q = cursor + 64 * j + lane;
+                    tk[j] = q < T ? tokens[q] : kNil;          // kNil is no token (tok < vocab < 2^32 - 1)
+                }
+#pragma unroll
+                for (int j = 0; j < U; j++) {
+                    const bool hit = tk[j] == tok;
+                    const unsigned long long mask = __ballot(hit);
+                    if (hit) list[len + __popcll(mask & ((1ull << lane) - 1ull))] = (uint32_t)(cursor + 64 * j + lane);
+                    len += __popcll(mask);
+                }
+                cursor += 64 * U;
+            }
         }
+        __syncthreads();
+        found += (uint32_t)len;
+        if (len == 0) break;                                   // cannot happen while the counts are consistent; never spin
+        // add the batch's rows in list order, pass by pass over the row's width
+        if (vec) {
+            for (int64_t i0 = 0; i0 < n4; i0 += 64 * kEmbVpl) {
+                float4 acc[kEmbVpl];
+#pragma unroll
+                for (int k = 0; k < kEmbVpl; k++) acc[k] = make_float4(0, 0, 0, 0);
+                int m = 0;
+                for (; m + 4 <= len; m += 4) {                 // four rows' loads in flight, added in list order
+                    float4 g[4][kEmbVpl];
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        const float4* src = reinterpret_cast<const float4*>(dH + (int64_t)list[m + u] * hidden);
+#pragma unroll
+                        for (int k = 0; k < kEmbVpl; k++) {
+                            const int64_t i = i0 + lane + 64 * k;
+                            g[u][k] = i < n4 ? src[i] : make_float4(0, 0, 0, 0);
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; u++)
+#pragma unroll
+                        for (int k = 0; k < kEmbVpl; k++) { acc[k].x += g[u][k].x; acc[k].y += g[u][k].y; acc[k].z += g[u][k].z; acc[k].w += g[u][k].w; }
+                }
+                for (; m < len; m++) {
+                    const float4* src = reinterpret_cast<const float4*>(dH + (int64_t)list[m] * hidden);
+#pragma unroll
+                    for (int k = 0; k < kEmbVpl; k++) {
+                        const int64_t i = i0 + lane + 64 * k;
+                        if (i < n4) { const float4 g = src[i]; acc[k].x += g.x; acc[k].y += g.y; acc[k].z += g.z; acc[k].w += g.w; }
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < kEmbVpl; k++) {
+                    const int64_t i = i0 + lane + 64 * k;
+                    if (i < n4) {
+                        float4 r = (first_batch && i0 == 0) ? old[k] : reinterpret_cast<float4*>(row)[i];
+                        r.x += acc[k].x; r.y += acc[k].y; r.z += acc[k].z; r.w += acc[k].w;
+                        reinterpret_cast<float4*>(row)[i] = r;
+                    }
+                }
+            }
+        } else {
+            for (int64_t i = lane; i < hidden; i += 64) {
+                float a = 0.0f;
+                for (int m = 0; m < len; m++) a += dH[(int64_t)list[m] * hidden + i];
+                row[i] += a;
+            }
+        }
+        first_batch = false;
+        __syncthreads();
     }
 }
 
@@ -238,26 +251,12 @@ int seraph_embedding_backward(const uint32_t* tokens, const float* dH, float* gr
     EmbWs w;
     emb_ws_layout(T, vocab, (char*)ws, &w);
     hipStream_t st = as_stream(s);
-    int rc = seraph_fill_u32(w.cnt, 0u, (size_t)vocab + 1, s);
-    if (rc != SERAPH_OK) return rc;
-    const dim3 tgrid((unsigned)ceil_div(T, 256));
-    hipLaunchKernelGGL(emb_count_kernel, tgrid, dim3(256), 0, st, tokens, w.cnt, T, vocab);
+    hipLaunchKernelGGL(emb_init_kernel, dim3((unsigned)ceil_div(vocab, 256)), dim3(256), 0, st, w.tab, vocab);
     SERAPH_LAUNCH_CHECK();
-    const int nchunks = (int)ceil_div(vocab, kScanChunk);
-    hipLaunchKernelGGL(emb_chunk_sums_kernel, dim3(nchunks), dim3(kScanBlock), 0, st, w.cnt, vocab, w.csum, w.cnz);
-    SERAPH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(emb_chunk_scan_kernel, dim3(1), dim3(64), 0, st, w.csum, w.cnz, nchunks, w.off, w.nuniq, vocab);
-    SERAPH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(emb_chunk_write_kernel, dim3(nchunks), dim3(kScanBlock), 0, st, w.cnt, vocab, w.csum, w.cnz, w.off, w.uniq);
-    SERAPH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(emb_fill_kernel, tgrid, dim3(256), 0, st, tokens, w.cnt, w.off, w.perm, T, vocab);
-    SERAPH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(emb_rank_kernel, tgrid, dim3(256), 0, st, tokens, w.off, w.perm, w.sorted, vocab);
+    hipLaunchKernelGGL(emb_link_kernel, dim3((unsigned)ceil_div(T, 256)), dim3(256), 0, st, tokens, w.tab, w.link, T, vocab);
     SERAPH_LAUNCH_CHECK();
     int vec = (hidden % 4 == 0) && aligned16(dH) && aligned16(grad_embed);
-    int64_t nblocks = T < vocab ? T : vocab;                  // upper bound on the number of touched rows
-    hipLaunchKernelGGL(emb_sum_kernel, dim3((unsigned)nblocks), dim3(256), 0, st, w.uniq, w.nuniq, w.off, w.sorted,
-                       dH, grad_embed, hidden, vec);
+    hipLaunchKernelGGL(emb_sum_kernel, dim3((unsigned)T), dim3(64), 0, st, tokens, w.tab, w.link, dH, grad_embed, T, hidden, vocab, vec);
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }

@@ -199,7 +199,7 @@ __device__ __forceinline__ void stnt4(float4* p, float4 v) {
     __builtin_nontemporal_store(r, reinterpret_cast<f4v*>(p));
 }
 
-template <int VPL, bool PREFETCH = false, bool NT = true>
+template <int VPL, int AHEAD>
 __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_block_kernel(const float* __restrict__ x,
                                                                    const float* __restrict__ scale,
                                                                    const float* __restrict__ dy,
@@ -210,42 +210,44 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_block_kernel(const float* 
     __shared__ double red[2][kWavesPerBlock][2];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int n4 = cols >> 2;
-    float4 sc[VPL], gs[VPL];
+    float4 gs[VPL];
+    double sd[VPL][4];                                            // the gains, widened once
 #pragma unroll
     for (int k = 0; k < VPL; k++) {
         int i4 = threadIdx.x + kBlock * k;
-        sc[k] = i4 < n4 ? reinterpret_cast<const float4*>(scale)[i4] : make_float4(0, 0, 0, 0);
+        const float4 sc = i4 < n4 ? reinterpret_cast<const float4*>(scale)[i4] : make_float4(0, 0, 0, 0);
+        sd[k][0] = (double)sc.x; sd[k][1] = (double)sc.y; sd[k][2] = (double)sc.z; sd[k][3] = (double)sc.w;
         gs[k] = make_float4(0, 0, 0, 0);
     }
-    auto fetch = [&](int64_t row, float4 (&xv)[VPL], float4 (&gv)[VPL], float4 (&rv)[VPL]) {
+    struct Row { float4 x[VPL], g[VPL], r[VPL]; };
+    auto fetch = [&](Row& b, int64_t row) {
         const float4* xr = reinterpret_cast<const float4*>(x + row * cols);
         const float4* gr = reinterpret_cast<const float4*>(dy + row * cols);
         const float4* rr = reinterpret_cast<const float4*>(res + row * cols);
 #pragma unroll
         for (int k = 0; k < VPL; k++) {
             int i4 = threadIdx.x + kBlock * k;
-            xv[k] = i4 < n4 ? (NT ? ldnt4(xr + i4) : xr[i4]) : make_float4(0, 0, 0, 0);
-            gv[k] = i4 < n4 ? (NT ? ldnt4(gr + i4) : gr[i4]) : make_float4(0, 0, 0, 0);
-            rv[k] = (res && i4 < n4) ? (NT ? ldnt4(rr + i4) : rr[i4]) : make_float4(0, 0, 0, 0);
+            b.x[k] = i4 < n4 ? ldnt4(xr + i4) : make_float4(0, 0, 0, 0);
+            b.g[k] = i4 < n4 ? ldnt4(gr + i4) : make_float4(0, 0, 0, 0);
+            b.r[k] = (res && i4 < n4) ? ldnt4(rr + i4) : make_float4(0, 0, 0, 0);
         }
     };
-    // a row's residual is read with the row (before that row of dx is written: in place is safe)
-    float4 xv[VPL], gv[VPL], rv[VPL], xn[VPL], gn[VPL], rn[VPL];
-    int64_t row = blockIdx.x;
-    if (row < rows) fetch(row, xv, gv, rv);
-    int it = 0;
-    for (; row < rows; row += gridDim.x, it ^= 1) {
-        const int64_t next = row + gridDim.x;
-        if (PREFETCH) { if (next < rows) fetch(next, xn, gn, rn); }
+    // a row's residual is read with the row, and a workgroup's rows are fetched in the order it stores them, so dx may be
+    // the residual itself
+    auto process = [&](const Row& b, int64_t row, int it) {
+        // Every value is widened once and kept: x, dy and dy * scale are needed on both sides of the barrier.
+        double xd[VPL][4], gd[VPL][4], td[VPL][4];
         double ssq = 0.0, cp = 0.0;
 #pragma unroll
         for (int k = 0; k < VPL; k++) {
-            const float* xs = &xv[k].x; const float* g = &gv[k].x; const float* s = &sc[k].x;
+            const float* xs = &b.x[k].x; const float* g = &b.g[k].x;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                double xd = (double)xs[e];
-                ssq += xd * xd;
-                cp += (double)g[e] * (double)s[e] * xd;
+                xd[k][e] = (double)xs[e];
+                gd[k][e] = (double)g[e];
+                td[k][e] = gd[k][e] * sd[k][e];
+                ssq += xd[k][e] * xd[k][e];
+                cp += td[k][e] * xd[k][e];                                           // dy * scale * x, :70
             }
         }
         ssq = wave_sum(ssq);
@@ -259,24 +261,39 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_block_kernel(const float* 
 #pragma unroll
         for (int k = 0; k < VPL; k++) {
             int i4 = threadIdx.x + kBlock * k;
-            const float* xs = &xv[k].x; const float* g = &gv[k].x; const float* s = &sc[k].x;
             float o[4]; float* acc = &gs[k].x;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                double xd = (double)xs[e], gd = (double)g[e];
-                acc[e] += (float)(gd * xd * st.inv);                                 // :90
-                o[e] = (float)(gd * (double)s[e] * st.inv - xd * st.k);              // :98
+                acc[e] += (float)(gd[k][e] * xd[k][e] * st.inv);                     // :90
+                o[e] = (float)(td[k][e] * st.inv - xd[k][e] * st.k);                 // :98
             }
-            const float4 ov = make_float4(rv[k].x + o[0], rv[k].y + o[1], rv[k].z + o[2], rv[k].w + o[3]);
-            if (i4 < n4) { if (NT) stnt4(dr + i4, ov); else dr[i4] = ov; }
+            const float4 ov = make_float4(b.r[k].x + o[0], b.r[k].y + o[1], b.r[k].z + o[2], b.r[k].w + o[3]);
+            if (i4 < n4) stnt4(dr + i4, ov);
         }
-        if (next < rows) {
-            if (PREFETCH) {
-#pragma unroll
-                for (int k = 0; k < VPL; k++) { xv[k] = xn[k]; gv[k] = gn[k]; rv[k] = rn[k]; }
-            } else {
-                fetch(next, xv, gv, rv);
-            }
+    };
+    const int64_t G = gridDim.x;
+    int64_t row = blockIdx.x;
+    if (AHEAD == 1) {
+        // the next row's loads are issued before the current row's arithmetic (FP64: a third of the kernel's time if
+        // nothing else ran beside it); two register sets take turns, so no row is ever copied
+        Row a, b;
+        if (row < rows) fetch(a, row);
+        while (row < rows) {
+            if (row + G < rows) fetch(b, row + G);
+            process(a, row, 0);
+            row += G;
+            if (row >= rows) break;
+            if (row + G < rows) fetch(a, row + G);
+            process(b, row, 1);
+            row += G;
+        }
+    } else {
+        Row a;
+        int it = 0;
+        if (row < rows) fetch(a, row);
+        for (; row < rows; row += G, it ^= 1) {
+            process(a, row, it);
+            if (row + G < rows) fetch(a, row + G);
         }
     }
 #pragma unroll
@@ -319,32 +336,61 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_generic_kernel(const float
     }
 }
 
-// grad_scale[c] += sum over partial rows in a fixed order.  64 columns x 16 row groups per
-// workgroup: group g adds rows g, g+16, ... in double, the 16 group sums are combined in order.
+// grad_scale[c] += sum over partial rows in a fixed order.  64 columns x 64 row groups per workgroup when the width
+// allows 16-byte loads (a lane takes four columns of rows g, g + 64, ..., all loads in flight, added in double in row
+// order; the 64 group sums are then combined in group order), else 64 columns x 16 row groups with scalar loads.
+template <bool VEC>
 __global__ __launch_bounds__(1024) void colsum_add_kernel(const float* __restrict__ partial, int nparts,
                                                            int64_t cols, float* __restrict__ grad_scale) {
-    __shared__ double part[16][64];
-    const int cx = threadIdx.x & 63, g = threadIdx.x >> 6;
-    const int64_t c = (int64_t)blockIdx.x * 64 + cx;
-    double s = 0.0;
-    if (c < cols) {
-        int p = g;
-        for (; p + 15 * 16 < nparts; p += 16 * 16) {          // sixteen loads in flight, added in row order
-            float a[16];
+    constexpr int GROUPS = VEC ? 64 : 16;
+    __shared__ double part[GROUPS][64];
+    double t4[4] = {0.0, 0.0, 0.0, 0.0};
+    int g, cx;
+    if (VEC) {
+        cx = (threadIdx.x & 15) * 4; g = threadIdx.x >> 4;
+        const int64_t c = (int64_t)blockIdx.x * 64 + cx;
+        if (c < cols) {
+            int p = g;
+            for (; p + 7 * GROUPS < nparts; p += 8 * GROUPS) {
+                float4 a[8];
 #pragma unroll
-            for (int u = 0; u < 16; u++) a[u] = partial[(size_t)(p + 16 * u) * cols + c];
+                for (int u = 0; u < 8; u++) a[u] = *reinterpret_cast<const float4*>(partial + (size_t)(p + GROUPS * u) * cols + c);
 #pragma unroll
-            for (int u = 0; u < 16; u++) s += (double)a[u];
+                for (int u = 0; u < 8; u++) { t4[0] += (double)a[u].x; t4[1] += (double)a[u].y; t4[2] += (double)a[u].z; t4[3] += (double)a[u].w; }
+            }
+            for (; p < nparts; p += GROUPS) {
+                const float4 a = *reinterpret_cast<const float4*>(partial + (size_t)p * cols + c);
+                t4[0] += (double)a.x; t4[1] += (double)a.y; t4[2] += (double)a.z; t4[3] += (double)a.w;
+            }
         }
-        for (; p < nparts; p += 16) s += (double)partial[(size_t)p * cols + c];
-    }
-    part[g][cx] = s;
-    __syncthreads();
-    if (g == 0 && c < cols) {
-        double t = 0.0;
 #pragma unroll
-        for (int k = 0; k < 16; k++) t += part[k][cx];
-        grad_scale[c] = (float)((double)grad_scale[c] + t);
+        for (int e = 0; e < 4; e++) part[g][cx + e] = t4[e];
+    } else {
+        cx = threadIdx.x & 63; g = threadIdx.x >> 6;
+        const int64_t c = (int64_t)blockIdx.x * 64 + cx;
+        double s = 0.0;
+        if (c < cols) {
+            int p = g;
+            for (; p + 15 * 16 < nparts; p += 16 * 16) {          // sixteen loads in flight, added in row order
+                float a[16];
+#pragma unroll
+                for (int u = 0; u < 16; u++) a[u] = partial[(size_t)(p + 16 * u) * cols + c];
+#pragma unroll
+                for (int u = 0; u < 16; u++) s += (double)a[u];
+            }
+            for (; p < nparts; p += 16) s += (double)partial[(size_t)p * cols + c];
+        }
+        part[g][cx] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        const int64_t c = (int64_t)blockIdx.x * 64 + threadIdx.x;
+        if (c < cols) {
+            double t = 0.0;
+#pragma unroll
+            for (int k = 0; k < GROUPS; k++) t += part[k][threadIdx.x];
+            grad_scale[c] = (float)((double)grad_scale[c] + t);
+        }
     }
 }
 
@@ -515,7 +561,7 @@ static int rmsnorm_backward_launch(const float* x, const float* scale, const flo
     if (bvpl) {
         const int grid = bwd_block_grid(rows);
         nparts = grid;
-#define BBWD(V) hipLaunchKernelGGL(rmsnorm_bwd_block_kernel<V>, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, res, dx, partial, rows, (int)cols, eps)
+#define BBWD(V) hipLaunchKernelGGL((rmsnorm_bwd_block_kernel<V, 0>), dim3(grid), dim3(kBlock), 0, st, x, scale, dy, res, dx, partial, rows, (int)cols, eps)
         switch (bvpl) {
             case 1: BBWD(1); break;
             case 2: BBWD(2); break;
@@ -538,8 +584,10 @@ static int rmsnorm_backward_launch(const float* x, const float* scale, const flo
         hipLaunchKernelGGL(rmsnorm_bwd_generic_kernel, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, res, dx, partial, rows, cols, eps);
     }
     SERAPH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(colsum_add_kernel, dim3((unsigned)ceil_div(cols, 64)), dim3(1024), 0, st,
-                       partial, nparts, cols, grad_scale);
+    if (cols % 4 == 0 && aligned16(partial))
+        hipLaunchKernelGGL(colsum_add_kernel<true>, dim3((unsigned)ceil_div(cols, 64)), dim3(1024), 0, st, partial, nparts, cols, grad_scale);
+    else
+        hipLaunchKernelGGL(colsum_add_kernel<false>, dim3((unsigned)ceil_div(cols, 64)), dim3(1024), 0, st, partial, nparts, cols, grad_scale);
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }

@@ -533,3 +533,35 @@ def test_cross_entropy_long_rows_are_deterministic_and_alias_safe(ops, rows, col
         live[1] = False
     assert float(g_ref[live].double().sum(dim=1).abs().max()) < 1e-6
     assert float(g_ref[~live].abs().max()) == 0 if (~live).any() else True
+
+
+@pytest.mark.parametrize("case", ["one token", "few tokens", "pairs", "mixed"])
+def test_embedding_backward_repeated_tokens(ops, orc, case):
+    """Groups of every size: a batch that is one token repeated (a padding-dominated batch), a handful of tokens, every
+    token twice, and a mixture whose groups straddle the lengths at which the gathering changes method (16) and the
+    batch size of the gather list (1024).  Integer-valued gradients: the sums are exact, so the check is bit-exact."""
+    r = rng(15)
+    T, h, V = 5000, 256, 3000
+    if case == "one token":
+        tok = np.full(T, 7, np.uint32)
+    elif case == "few tokens":
+        tok = r.integers(0, 3, T).astype(np.uint32) * 1000
+    elif case == "pairs":
+        tok = np.concatenate([r.permutation(T // 2), r.permutation(T // 2)]).astype(np.uint32)
+    else:
+        sizes = [1, 2, 15, 16, 17, 63, 64, 65, 1023, 1024, 1025]
+        tok = np.concatenate([np.full(n, 10 + i, np.uint32) for i, n in enumerate(sizes)] +
+                             [np.arange(100, 100 + T - sum(sizes), dtype=np.uint32)])
+        tok = tok[r.permutation(T)]
+        tok[::97] = V + 5                                      # skipped positions in between
+    dH = r.integers(-8, 9, (T, h)).astype(np.float32)
+    base = r.integers(-3, 4, (V, h)).astype(np.float32)
+    ref = orc.embedding_backward(tok, dH, base)
+    got = host(ops.embedding_backward(dev(tok.view(np.int32)), dev(dH), dev(base)))
+    assert (got == ref).all()
+    # float gradients: deterministic and within tolerance
+    dF = r.standard_normal((T, h)).astype(np.float32)
+    a = ops.embedding_backward(dev(tok.view(np.int32)), dev(dF), dev(base))
+    b = ops.embedding_backward(dev(tok.view(np.int32)), dev(dF), dev(base))
+    assert torch.equal(a, b)
+    parity(a, orc.embedding_backward(tok, dF, base), "embedding backward", atol=1e-4)
