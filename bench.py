@@ -3,12 +3,17 @@
 training step on ONE MI355X, with the dominant kernel's roofline fraction measured live and
 the CPU oracle timed beside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c1] [--pmc-calibration]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c1] [--headline-only] [--pmc-calibration]
 
 Workloads (BASELINE.json configs): c5 = Qwen3-1.7B-shape full-weight FP32 training,
 4 x 4096 tokens (default); c4 = the same model, LoRA r16 on q/k/v/o, 1 x 2048; c1 = the
 33M Seraph-native model, 8 x 256.  Synthetic data: uniform token ids, N(0, 0.02) weights,
-norm gains 1, fixed seeds.  Prints ONE JSON line.
+norm gains 1, fixed seeds.  Prints ONE JSON line.  The headline keys (value, ms_per_step, roofline,
+cpu_baseline ...) are the named workload's.  The default run (c5) then also measures the rest of the
+metric and adds it under extra keys: `workloads` (c1 and c4 as whole steps, each with its own roofline),
+`ops` (the single-op configurations alone: attention backward at B8 H16 S1024 D64, and cross entropy,
+RMSNorm backward, SwiGLU backward, AdamW, RoPE, qk_norm and embedding backward at 16384 tokens), and
+`drop_in_path` (the reference's unmodified step driver over this backend's vulkan_* symbols).
 
 --pmc-calibration launches the library's in-place scale kernel three times over 1 GiB before
 the steps (reads 1 GiB, writes 1 GiB per launch): under `rocprofv3 --pmc FETCH_SIZE` /
@@ -143,30 +148,11 @@ def gemm_table(w):
     print(f"GEMM time per step: this library {tot[0]:.1f} ms, hipBLASLt {tot[1]:.1f} ms")
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=3)
-    ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--pmc-calibration", action="store_true")
-    ap.add_argument("--no-op-timing", action="store_true",
-                    help="do not bracket every kernel-library call with an event pair (no roofline / kernels objects)")
-    ap.add_argument("--gemm-table", action="store_true",
-                    help="instead of the benchmark, time every GEMM shape of the workload's step beside hipBLASLt")
-    args = ap.parse_args()
-    if args.gemm_table:
-        gemm_table(WORKLOADS[args.workload])
-        return
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
-                 "(value is the one GPU's throughput)")
-
+def run_workload(w, key, steps, warmup, op_timing=True, pmc_calibration=False):
+    """`warmup` untimed steps, then `steps` timed ones of workload `w`; returns the fields of the bench line."""
     import torch
     from seraph_amd import trainer as tr
 
-    w = WORKLOADS[args.workload]
     T = w["batch"] * w["seq"]
     lora = w["lora"] or dict(rank=0, alpha=0.0, mask=0)
     cfg = tr.model_config(w["hidden"], w["layers"], w["heads"], w["kv_heads"], w["head_dim"], w["ffn"], w["vocab"],
@@ -198,7 +184,7 @@ def main():
                 o += oo * r
         t.upload(tr.LORA_PARAMS, lo)
 
-    if args.pmc_calibration:
+    if pmc_calibration:
         from seraph_amd import ops
         cal = torch.ones(1 << 28, dtype=torch.float32, device=dev)
         for _ in range(3):
@@ -208,35 +194,35 @@ def main():
 
     rng = np.random.default_rng(99)
     starts = np.arange(0, T + 1, w["seq"], dtype=np.int32)
-    batches = [rng.integers(0, w["vocab"], T).astype(np.int32) for _ in range(args.warmup + args.steps)]
+    batches = [rng.integers(0, w["vocab"], T).astype(np.int32) for _ in range(warmup + steps)]
 
     losses = []
     tw = time.perf_counter()
-    for i in range(args.warmup):
+    for i in range(warmup):
         losses.append(t.step(batches[i], starts))
     torch.cuda.synchronize()
-    warm_ms = 1000.0 * (time.perf_counter() - tw) / max(args.warmup, 1)
+    warm_ms = 1000.0 * (time.perf_counter() - tw) / max(warmup, 1)
 
     # Per-kernel timing brackets every kernel-library call of the step with a HIP event pair on the step's
     # stream.  On a step of hundreds of milliseconds that costs well under 1 % and runs inside the timed
     # region.  On a step of a few milliseconds (c1) the ~1000 event records would take a third of the step,
     # so the timed region runs without them and the same batches are replayed once more with them.
-    in_region = (not args.no_op_timing) and (args.warmup == 0 or warm_ms >= 100.0)
+    in_region = op_timing and (warmup == 0 or warm_ms >= 100.0)
     t.enable_op_timing(in_region)
     t.reset_op_stats()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        losses.append(t.step(batches[args.warmup + i], starts))
+    for i in range(steps):
+        losses.append(t.step(batches[warmup + i], starts))
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     timing = t.last_timing()
     roofline_from = "timed region"
-    if not in_region and not args.no_op_timing:
+    if not in_region and op_timing:
         t.enable_op_timing(True)
         t.reset_op_stats()
-        for i in range(args.steps):
-            t.step(batches[args.warmup + i], starts)
+        for i in range(steps):
+            t.step(batches[warmup + i], starts)
         torch.cuda.synchronize()
         roofline_from = ("second pass over the timed region's batches: per-kernel events inside a step this short "
                          "would dominate it")
@@ -270,16 +256,15 @@ def main():
                         avg_launch_ms=round(dom["ms"] / dom["launches"], 4), bytes_per_launch=dom["bytes"] / dom["launches"])
 
     if roofline is not None:
-        roofline["traffic"] = measured_traffic(dom["name"], args.workload)
+        roofline["traffic"] = measured_traffic(dom["name"], key)
         roofline["measured_over"] = roofline_from
 
     out = {
-        "metric": "train tok/s (fwd+bwd+AdamW)", "value": round(args.steps * T / elapsed, 2), "unit": "tok/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(1000.0 * elapsed / args.steps, 3),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "value": round(steps * T / elapsed, 2), "unit": "tok/s", "steps": steps, "warmup": warmup,
+        "ms_per_step": round(1000.0 * elapsed / steps, 3),
         "config": {"workload": w["name"], "tokens_per_step": T, "batch": w["batch"], "seq_len": w["seq"],
                    "params": n, "device_bytes": t.device_bytes + sum(x.numel() * 4 for x in ext if x is not None),
-                   "rms_eps": w["rms_eps"], "adamw_clip": w["clip"], "seed": 1234},
+                   "rms_eps": w["rms_eps"], "adamw_clip": w["clip"], "qk_norm": False, "seed": 1234},
         "loss_first_last": [round(losses[0], 5), round(losses[-1], 5)],
         "phase_ms_last_step": {k: round(v, 3) for k, v in timing.items()},
         "roofline": roofline,
@@ -288,8 +273,263 @@ def main():
     t.close()
     del params, ext
     torch.cuda.empty_cache()
+    return out
+
+
+def time_op(fn, iters, warm=2, reps=1):
+    """Mean device time of one fn() call in ms.  One event pair brackets `reps` back-to-back calls (a pair costs a few
+    microseconds, which matters for ops of tens of microseconds); the events are recorded on the stream the op is
+    launched on (the ops below run on torch's current stream, which is where torch records its events).  fn gets a
+    running call index so that it can rotate between operand sets."""
+    import torch
+    ms = []
+    call = 0
+    for i in range(warm + iters):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(reps):
+            fn(call)
+            call += 1
+        b.record()
+        torch.cuda.synchronize()
+        if i >= warm:
+            ms.append(a.elapsed_time(b) / reps)
+    return sum(ms) / len(ms), min(ms)
+
+
+def isolated_ops():
+    """The single-op configurations: causal attention backward at B8 H16 S1024 D64 and the bandwidth-bound backward
+    chain over 16384 tokens (hidden 2048, FFN 6144, vocabulary 151936, AdamW over 50 M parameters), each op alone
+    through the C ABI.  Bandwidth-bound ops run on operands too large for the caches or on rotating operand sets,
+    so every call starts cold.  Algorithmic work: each input read once, each output written once."""
+    import torch
+    from seraph_amd import ops
+    ops.init(0)
+    out = {}
+    dev = "cuda"
+
+    def hbm(name, nbytes, fn, iters=6, reps=6, note=None):
+        avg, best = time_op(fn, iters, reps=reps)
+        e = dict(ms=round(avg, 4), min_ms=round(best, 4), bound="hbm", algorithmic_bytes=nbytes,
+                 achieved=round(nbytes / avg / 1e6, 1), unit="GB/s", peak=PEAK_HBM_GBS, frac=round(nbytes / avg / 1e6 / PEAK_HBM_GBS, 4))
+        if note:
+            e["note"] = note
+        out[name] = e
+
+    # ---- attention backward, B8 H16 S1024 D64 (saved O and log-sum-exp from the forward, as the step has them)
+    B, S, H, D = 8, 1024, 16, 64
+    T = B * S
+    g = torch.Generator(device=dev).manual_seed(7)
+    mk = lambda w: torch.randn(T, w, device=dev, generator=g) / 8.0
+    Q, K, V, dO = mk(H * D), mk(H * D), mk(H * D), mk(H * D)
+    ss = torch.arange(0, T + 1, S, device=dev, dtype=torch.int32)
+    O, L = ops.attention_forward(Q, K, V, H, H, D, ss)
+    dQ, dK, dV = torch.empty_like(Q), torch.zeros_like(K), torch.zeros_like(V)
+    flops = 10.0 * D * H * B * S * (S + 1) / 2
+    avg, best = time_op(lambda i: ops.attention_backward(Q, K, V, dO, H, H, D, ss, out=O, lse=L, dK=dK, dV=dV, dQ=dQ, max_seq_len=S), 6, reps=4)
+    out["attention_backward_b8_h16_s1024_d64"] = dict(
+        ms=round(avg, 4), min_ms=round(best, 4), bound="mfma", algorithmic_flops=flops, achieved=round(flops / avg / 1e9, 2),
+        unit="TFLOP/s", peak=PEAK_FP32_MFMA_TFLOPS, frac=round(flops / avg / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4),
+        note="delta + dK/dV (+ dS band) + dQ kernels; dK/dV accumulate into the caller's buffers")
+    avg, best = time_op(lambda i: ops.attention_forward(Q, K, V, H, H, D, ss), 6, reps=4)
+    out["attention_forward_b8_h16_s1024_d64"] = dict(
+        ms=round(avg, 4), min_ms=round(best, 4), bound="mfma", algorithmic_flops=0.4 * flops, achieved=round(0.4 * flops / avg / 1e9, 2),
+        unit="TFLOP/s", peak=PEAK_FP32_MFMA_TFLOPS, frac=round(0.4 * flops / avg / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4))
+    del Q, K, V, dO, O, L, dQ, dK, dV
+
+    # ---- cross entropy 16384 x 151936, logits N(0, 2), gradient written over the logits as in the step
+    rows, cols = 16384, 151936
+    x = torch.randn(rows, cols, device=dev, generator=g) * 2.0
+    tgt = torch.randint(0, cols, (rows,), device=dev, dtype=torch.int32)
+
+    def ce(i):
+        ops.cross_entropy_grad(x, tgt, rows, grad=x)
+    # in place the second call would see gradients as logits: still 2 x rows x cols x 4 bytes of the same traffic
+    hbm("cross_entropy_grad_16384_x_151936", 2 * rows * cols * 4 + 8 * rows, ce, iters=5, reps=1)
+    del x
+
+    # ---- RMSNorm backward 16384 x 2048 (x N(0,1), gains N(1, 0.02), dY N(0, 1e-2)); three operand sets in rotation
+    rows, cols = 16384, 2048
+    sets = [(torch.randn(rows, cols, device=dev, generator=g), torch.randn(rows, cols, device=dev, generator=g) * 1e-2,
+             torch.empty(rows, cols, device=dev)) for _ in range(3)]
+    gains = 1.0 + 0.02 * torch.randn(cols, device=dev, generator=g)
+    gs = torch.zeros(cols, device=dev)
+    hbm("rmsnorm_backward_16384_x_2048", 3 * rows * cols * 4 + 2 * cols * 4,
+        lambda i: ops.rmsnorm_backward(sets[i % 3][0], gains, sets[i % 3][1], 1e-6, grad_scale=gs, out=sets[i % 3][2]),
+        note="row kernel + column sum of the gain gradient")
+    # qk_norm backward as the step runs it (from the normalised output and the saved rms), all 16 heads of a token together
+    rms_tok = torch.rand(rows, device=dev, generator=g) + 0.5
+    hbm("qk_norm_backward_16384_x_16_heads_128", 3 * rows * cols * 4 + 4 * rows,
+        lambda i: ops.qk_norm_backward_saved(sets[i % 3][0], rms_tok, sets[i % 3][1], 16, 128, 1e-6, out=sets[i % 3][2]))
+    # RoPE backward in place over 16 heads of 128
+    hbm("rope_backward_16384_x_16_heads_128", 2 * rows * cols * 4,
+        lambda i: ops.rope(sets[i % 3][0], 16, 128, 1e6, None, backward=True, out=sets[i % 3][0]))
+    # embedding backward: 16384 rows of 2048 into a 151936-row table, uniform tokens
+    V = 151936
+    tok = torch.randint(0, V, (rows,), device=dev, dtype=torch.int32)
+    uniq = int(torch.unique(tok).numel())
+    table = torch.zeros(V, cols, device=dev)
+    hbm("embedding_backward_16384_x_2048_into_151936_rows", rows * cols * 4 + 2 * uniq * cols * 4 + rows * 4,
+        lambda i: ops.embedding_backward(tok, sets[i % 3][0], table), note=f"{uniq} distinct tokens; three launches")
+    del sets, table
+
+    # ---- SwiGLU backward 16384 x 6144
+    n = 16384 * 6144
+    gate, up, dH = (torch.randn(n, device=dev, generator=g) for _ in range(3))
+    outs = (torch.empty(n, device=dev), torch.empty(n, device=dev))
+    hbm("swiglu_backward_16384_x_6144", 5 * n * 4, lambda i: ops.swiglu_backward(gate, up, dH, out=outs))
+    del gate, up, dH, outs
+
+    # ---- AdamW over 50 M parameters, gradients N(0, 1e-3) with 1 % entries of magnitude 10
+    n = 50_000_000
+    wts = [torch.randn(n, device=dev, generator=g) * 0.02 for _ in range(2)]
+    grad = torch.randn(n, device=dev, generator=g) * 1e-3
+    grad[torch.rand(n, device=dev, generator=g) < 0.01] = 10.0
+    m, v = torch.zeros(n, device=dev), torch.zeros(n, device=dev)
+    for clip in (0.0, 1.0):
+        hbm(f"adamw_50m_clip_{clip:g}", 7 * n * 4,
+            lambda i: ops.adamw_(wts[i % 2], grad, m, v, 3.14e-4, 0.9, 0.999, 0.01, 1e-8, 1 + i, clip),
+            note="clip 0 is the reference's formula" if clip == 0.0 else "per-element clamp of the gradient first")
+    del wts, grad, m, v
+    torch.cuda.empty_cache()
+    return out
+
+
+def reference_cpu_step(w, tokens=64):
+    """The reference's own CPU training step (its C code in src/train.c, compiled from the Seraph tree into
+    oracle/_ref/ref_step_hip where that tree was present at build time), one sequence of `tokens` tokens,
+    single-threaded as the reference runs it.  None when the binary is not there."""
+    import struct
+    import subprocess
+    import tempfile
+    exe = os.path.join(ROOT, "oracle", "_ref", "ref_step_hip")
+    if not os.path.exists(exe) or w["lora"]:
+        return None
+    from oracle import oracle as orc
+    cfg = orc.make_config(hidden=w["hidden"], layers=w["layers"], heads=w["heads"], kv_heads=w["kv_heads"], head_dim=w["head_dim"],
+                          ffn=w["ffn"], vocab=w["vocab"], rms_eps=w["rms_eps"], rope_theta=w["rope_theta"])
+    n = orc.param_count(cfg)
+    r = np.random.default_rng(3)
+    with tempfile.TemporaryDirectory() as d:
+        with open(os.path.join(d, "in.bin"), "wb") as f:
+            f.write(struct.pack("11i", w["hidden"], w["layers"], w["heads"], w["kv_heads"], w["head_dim"], w["ffn"], w["vocab"], 1, tokens, 0, 0))
+            f.write(struct.pack("3f", w["lr"], w["rope_theta"], 0.0))
+            f.write((0.02 * r.standard_normal(n)).astype(np.float32).tobytes())
+            f.write(r.integers(0, w["vocab"], tokens).astype(np.int32).tobytes())
+        p = subprocess.run([exe, "--cpu", "--time", os.path.join(d, "in.bin"), os.path.join(d, "out.bin")],
+                           capture_output=True, text=True, timeout=600)
+    for line in p.stdout.splitlines():
+        if line.startswith("seconds_per_step"):
+            sec = float(line.split()[1])
+            return dict(value=round(tokens / sec, 3), unit="tok/s", cores=1, kind="reference",
+                        sample=(f"the reference's CPU training step (train_step with no backend: train_forward_fp32, loss, "
+                                f"train_backward, AdamW; src/train.c) on one sequence of {tokens} tokens of this model, "
+                                f"{sec:.1f} s, single-threaded as the reference runs it; its backward is the reference's "
+                                f"approximate CPU gradient, timed only"))
+    return None
+
+
+def drop_in_step(w, seq, steps=6):
+    """tok/s of the reference's own step driver (train_step -> train_step_gpu_full, unmodified, one sequence per step,
+    its per-tensor AdamW and cache copies) running over this backend's vulkan_* symbols: what `make hip` gives a
+    Seraph user without touching train.c.  None when oracle/_ref/ref_step_hip is not there."""
+    import struct
+    import subprocess
+    import tempfile
+    exe = os.path.join(ROOT, "oracle", "_ref", "ref_step_hip")
+    if not os.path.exists(exe) or w["lora"]:
+        return None
+    from oracle import oracle as orc
+    cfg = orc.make_config(hidden=w["hidden"], layers=w["layers"], heads=w["heads"], kv_heads=w["kv_heads"], head_dim=w["head_dim"],
+                          ffn=w["ffn"], vocab=w["vocab"])
+    n = orc.param_count(cfg)
+    r = np.random.default_rng(4)
+    with tempfile.TemporaryDirectory() as d:
+        with open(os.path.join(d, "in.bin"), "wb") as f:
+            f.write(struct.pack("11i", w["hidden"], w["layers"], w["heads"], w["kv_heads"], w["head_dim"], w["ffn"], w["vocab"], steps, seq, 0, 0))
+            f.write(struct.pack("3f", w["lr"], w["rope_theta"], 0.0))
+            f.write((0.02 * r.standard_normal(n)).astype(np.float32).tobytes())
+            f.write(r.integers(0, w["vocab"], steps * seq).astype(np.int32).tobytes())
+        p = subprocess.run([exe, "--time", os.path.join(d, "in.bin"), os.path.join(d, "out.bin")], capture_output=True, text=True, timeout=600)
+    for line in p.stdout.splitlines():
+        if line.startswith("seconds_per_step"):
+            sec = float(line.split()[1])
+            return dict(value=round(seq / sec, 1), unit="tok/s", ms_per_step=round(1000 * sec, 3), tokens_per_step=seq,
+                        what="reference train_step_gpu_full, unmodified, over this backend; one sequence per step")
+    return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true")
+    ap.add_argument("--no-op-timing", action="store_true",
+                    help="do not bracket every kernel-library call with an event pair (no roofline / kernels objects)")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="only the headline workload: no other workloads, isolated ops or drop-in path in the line")
+    ap.add_argument("--gemm-table", action="store_true",
+                    help="instead of the benchmark, time every GEMM shape of the workload's step beside hipBLASLt")
+    args = ap.parse_args()
+    if args.gemm_table:
+        gemm_table(WORKLOADS[args.workload])
+        return
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
+                 "(value is the one GPU's throughput)")
+
+    w = WORKLOADS[args.workload]
+    head = run_workload(w, args.workload, args.steps, args.warmup, op_timing=not args.no_op_timing,
+                        pmc_calibration=args.pmc_calibration)
+    out = {
+        "metric": "train tok/s (fwd+bwd+AdamW)", "value": head["value"], "unit": "tok/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": head["config"], "loss_first_last": head["loss_first_last"], "phase_ms_last_step": head["phase_ms_last_step"],
+        "roofline": head["roofline"], "kernels": head["kernels"],
+    }
+    full = args.workload == "c5" and not args.headline_only
+    if full:
+        # the rest of the metric: the 33M model and the LoRA configuration as whole steps, the single-op
+        # configurations alone, and the unmodified reference step driver over the vulkan_* symbols
+        others = {}
+        for key, steps, warmup in (("c1", 30, 5), ("c4", 8, 2)):
+            r = run_workload(WORKLOADS[key], key, steps, warmup, op_timing=not args.no_op_timing)
+            others[key] = {k: r[k] for k in ("value", "unit", "ms_per_step", "steps", "warmup", "config", "loss_first_last", "roofline")}
+            top = sorted(r["kernels"].items(), key=lambda kv: -kv[1]["share"])[:6]
+            others[key]["kernels"] = dict(top)
+        out["workloads"] = others
+        out["ops"] = isolated_ops()
+        c1 = WORKLOADS["c1"]
+        di = {f"c1_shape_1x{seq}": drop_in_step(c1, seq) for seq in (256, 2048)}
+        if any(v is not None for v in di.values()):
+            out["drop_in_path"] = di
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)
+        if full:
+            c1 = WORKLOADS["c1"]
+            from oracle import oracle as orc
+            tok = np.random.default_rng(0).integers(0, c1["vocab"], 2048).astype(np.int32)
+            cfg = orc.make_config(hidden=c1["hidden"], layers=c1["layers"], heads=c1["heads"], kv_heads=c1["kv_heads"],
+                                  head_dim=c1["head_dim"], ffn=c1["ffn"], vocab=c1["vocab"], rms_eps=c1["rms_eps"], rope_theta=c1["rope_theta"])
+            p = np.full(orc.param_count(cfg), 0.01, np.float32)
+            best = 1e9
+            for _ in range(2):
+                t0 = time.perf_counter()
+                _, g = orc.step_full(cfg, p, tok, np.arange(0, 2049, 256, dtype=np.int32))
+                z = np.zeros_like(p)
+                orc.adamw(p, g, z, z, 3.14e-6, 0.9, 0.999, 0.01, 1e-8, 1, clip=1.0)
+                best = min(best, time.perf_counter() - t0)
+            out["workloads"]["c1"]["cpu_baseline"] = dict(
+                value=round(2048 / best, 2), unit="tok/s", cores=orc.num_threads(), kind="port",
+                sample=f"one full step of the 33M configuration (8 x 256 tokens: forward, loss, backward, AdamW) with the oracle, {best:.2f} s (best of 2)")
+            ref = reference_cpu_step(c1)
+            if ref is not None:
+                out["workloads"]["c1"]["cpu_baseline_reference"] = ref
     print(json.dumps(out))
 
 

@@ -39,6 +39,10 @@ typedef struct {
     int32_t lora_rank;      /* 0 = full-weight training */
     float   lora_alpha;
     int32_t lora_mask;      /* bit0 q, 1 k, 2 v, 3 o, 4 gate, 5 up, 6 down (src/lora.c:372-396) */
+    int32_t use_qk_norm;    /* 0 (the reference's language-model mode, src/model_config.c:282): off.  1: q and k are divided by
+                               their root mean square over all heads of a token after RoPE (shaders/qk_norm.comp, called at
+                               src/train.c:4688-4689 with the step's eps) and, unlike the reference, whose backward treats the
+                               op as the identity, the backward applies its derivative before the RoPE backward */
 } hip_model_config_t;
 
 typedef struct {

@@ -206,6 +206,14 @@ int seraph_rope_qk(const float* q_in, float* q_out, int q_heads, const float* k_
 int seraph_qk_norm(float* qk, int64_t T, int heads, int head_dim, int use_qk_norm, float eps, seraph_stream_t s);
 int seraph_qk_norm_backward(const float* x_pre, const float* dy, float* dx, int64_t T, int heads, int head_dim,
                             float eps, seraph_stream_t s);
+/* The pair a training step uses: the forward (always applied) also leaves each token's unclamped root mean square in
+ * rms_out [T] (NULL: not wanted), and the backward works from the normalised output y, which the step keeps for the
+ * attention anyway, and that rms: dx = (dy - y (dy.y)/n) / rms, or dy/eps where the forward clamped.  dx may be dy.
+ * Same derivative as seraph_qk_norm_backward; no reference counterpart (the reference treats qk_norm as the identity
+ * in its backward, src/train.c:5224-5266). */
+int seraph_qk_norm_saved(float* qk, float* rms_out, int64_t T, int heads, int head_dim, float eps, seraph_stream_t s);
+int seraph_qk_norm_backward_saved(const float* y, const float* rms, const float* dy, float* dx, int64_t T, int heads,
+                                  int head_dim, float eps, seraph_stream_t s);
 
 /* ---------------------------------------------------------------- element-wise */
 /* vulkan_silu, include/vulkan_backend.h:476-478 (shaders/silu.comp) */

@@ -23,7 +23,8 @@ class Config(C.Structure):
     _fields_ = [("hidden", C.c_int32), ("layers", C.c_int32), ("heads", C.c_int32),
                 ("kv_heads", C.c_int32), ("head_dim", C.c_int32), ("ffn", C.c_int32),
                 ("vocab", C.c_int32), ("rms_eps", C.c_float), ("rope_theta", C.c_float),
-                ("lora_rank", C.c_int32), ("lora_alpha", C.c_float), ("lora_mask", C.c_int32)]
+                ("lora_rank", C.c_int32), ("lora_alpha", C.c_float), ("lora_mask", C.c_int32),
+                ("use_qk_norm", C.c_int32)]
 
 
 _lib = None
@@ -216,9 +217,9 @@ def lr_schedule(base_lr, optimizer_step, accum_steps=1):
 
 
 def make_config(hidden, layers, heads, kv_heads, head_dim, ffn, vocab, rms_eps=1e-5, rope_theta=10000.0,
-                lora_rank=0, lora_alpha=0.0, lora_mask=0):
+                lora_rank=0, lora_alpha=0.0, lora_mask=0, use_qk_norm=0):
     return Config(hidden, layers, heads, kv_heads, head_dim, ffn, vocab, rms_eps, rope_theta,
-                  lora_rank, lora_alpha, lora_mask)
+                  lora_rank, lora_alpha, lora_mask, use_qk_norm)
 
 
 def param_count(cfg):

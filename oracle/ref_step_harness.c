@@ -11,7 +11,12 @@
  * for the ops (those are this build's kernels); it cross-checks the op ORDER of the
  * oracle's step against the reference's own driver.
  *
- * usage: ref_step_hip <in.bin> <out.bin>
+ * usage: ref_step_hip [--cpu] [--time] <in.bin> <out.bin>
+ *   --cpu  : no backend is created, so train_step takes the reference's CPU path (src/train.c:6842-6983:
+ *            train_forward_fp32, the scalar loss loops, train_backward, the CPU AdamW); full-weight mode only.
+ *            This is the timed "reference" CPU baseline; its gradients are NOT those of the GPU path
+ *            (the CPU backward is an approximation) and nothing is compared with them.
+ *   --time : prints "seconds_per_step <mean over all steps but the first>" (all steps when there is only one)
  *   in : int32 hidden, layers, heads, kv_heads, head_dim, ffn, vocab, steps, T, lora_rank, lora_mask
  *        float32 lr, rope_theta, lora_alpha
  *        float32 params[...] in this build's arena order
@@ -24,6 +29,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 #include "model_config.h"
 #include "lora.h"
@@ -34,8 +40,21 @@ static int rd(void* p, size_t n, FILE* f) { return fread(p, 1, n, f) == n ? 0 : 
 
 typedef struct { weight_tensor_t* t; vulkan_buffer_t* w; vulkan_buffer_t* g; } slot_t;
 
+static double now_s(void) {
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
+}
+
 int main(int argc, char** argv) {
-    if (argc != 3) { fprintf(stderr, "usage: %s in.bin out.bin\n", argv[0]); return 2; }
+    int cpu_only = 0, timed = 0;
+    while (argc > 1 && argv[1][0] == '-' && argv[1][1] == '-') {
+        if (!strcmp(argv[1], "--cpu")) cpu_only = 1;
+        else if (!strcmp(argv[1], "--time")) timed = 1;
+        else { fprintf(stderr, "unknown option %s\n", argv[1]); return 2; }
+        argv++; argc--;
+    }
+    if (argc != 3) { fprintf(stderr, "usage: %s [--cpu] [--time] in.bin out.bin\n", argv[0]); return 2; }
     FILE* f = fopen(argv[1], "rb");
     if (!f) { perror("in.bin"); return 2; }
     int hdr[11]; float fl[3];
@@ -101,6 +120,25 @@ int main(int argc, char** argv) {
     if (rd(tokens, (size_t)steps * T * sizeof(int), f)) { fprintf(stderr, "short tokens\n"); return 2; }
     fclose(f);
 
+    if (cpu_only) {
+        if (rank > 0) { fprintf(stderr, "--cpu: full-weight mode only\n"); return 2; }
+        /* what train_init leaves behind for the CPU path (src/train.c:7927-7934); vulkan_ctx stays NULL */
+        st.act_cache = activation_cache_alloc(layers, hidden, ffn, heads * hd, kvh * hd, T);
+        float* closs = malloc((size_t)steps * sizeof(float));
+        double t_first = 0.0, t_rest = 0.0;
+        for (int s = 0; s < steps; s++) {
+            const double t0 = now_s();
+            closs[s] = train_step(&st, tokens + (size_t)s * T, T);
+            const double dt = now_s() - t0;
+            if (s == 0) t_first = dt; else t_rest += dt;
+        }
+        printf("ref_step_hip: CPU path, %d steps of %d tokens, %zu parameters, optimizer_step=%d, last loss %.6f\n",
+               steps, T, total, st.optimizer_step, closs[steps - 1]);
+        if (timed) printf("seconds_per_step %.6f\n", steps > 1 ? t_rest / (steps - 1) : t_first);
+        FILE* o = fopen(argv[2], "wb");
+        if (o) { fwrite(closs, sizeof(float), (size_t)steps, o); fclose(o); }
+        return 0;
+    }
     vulkan_context_t* ctx = vulkan_init_ex(0, -1);
     if (!ctx) { fprintf(stderr, "backend init failed\n"); return 4; }
     st.vulkan_ctx = ctx;
@@ -131,7 +169,14 @@ int main(int argc, char** argv) {
     }
 
     float* loss = malloc((size_t)steps * sizeof(float));
-    for (int s = 0; s < steps; s++) loss[s] = train_step(&st, tokens + (size_t)s * T, T);
+    double t_first = 0.0, t_rest = 0.0;
+    for (int s = 0; s < steps; s++) {                    /* train_step returns after its submit-and-wait and loss download */
+        const double t0 = now_s();
+        loss[s] = train_step(&st, tokens + (size_t)s * T, T);
+        const double dt = now_s() - t0;
+        if (s == 0) t_first = dt; else t_rest += dt;
+    }
+    if (timed) printf("seconds_per_step %.6f\n", steps > 1 ? t_rest / (steps - 1) : t_first);
 
     if (rank > 0) {
         if (save_checkpoint(&st, argv[2]) != 0) return 5;      /* pulls A, B, m, v back into st.lora */

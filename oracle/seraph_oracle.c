@@ -705,7 +705,7 @@ static float step_impl(const orc_config_t* c, const float* P, float* G,
           **attn_out = calloc(NL, sizeof(float*)), **post_in = calloc(NL, sizeof(float*)),
           **xn_ffn = calloc(NL, sizeof(float*)), **gate = calloc(NL, sizeof(float*)),
           **up = calloc(NL, sizeof(float*)), **silu_out = calloc(NL, sizeof(float*)),
-          **ffn_h = calloc(NL, sizeof(float*));
+          **ffn_h = calloc(NL, sizeof(float*)), **pq = calloc(NL, sizeof(float*)), **pk = calloc(NL, sizeof(float*));
     float* hidden = fnew(T * h);
     float* tmp_h = fnew(T * h);
     float* ltmp = fnew(T * (r > 0 ? r : 1));
@@ -726,6 +726,12 @@ static float step_impl(const orc_config_t* c, const float* P, float* G,
         if (lora && LL.A[2] >= 0) lora_forward_add(xn_attn[l], cv[l], LW + LL.A[2], LW + LL.B[2], ltmp, T, h, kv, r, ls);
         orc_rope(cq[l], cq[l], starts, batch, T, H, D, c->rope_theta, 0);
         orc_rope(ck[l], ck[l], starts, batch, T, KVH, D, c->rope_theta, 0);
+        if (c->use_qk_norm) {                                    /* src/train.c:4687-4689; the inputs are kept for the derivative */
+            pq[l] = fnew(T * qd); memcpy(pq[l], cq[l], (size_t)(T * qd) * 4);
+            pk[l] = fnew(T * kv); memcpy(pk[l], ck[l], (size_t)(T * kv) * 4);
+            orc_qk_norm(cq[l], T, H, D, eps);
+            orc_qk_norm(ck[l], T, KVH, D, eps);
+        }
         attn_out[l] = fnew(T * qd);
         orc_attention_forward(cq[l], ck[l], cv[l], attn_out[l], NULL, starts, batch, T, H, KVH, D, scale);
         orc_matmul(attn_out[l], W + L.rel.o, tmp_h, T, h, qd, 0, 1, 0);
@@ -807,6 +813,13 @@ static float step_impl(const orc_config_t* c, const float* P, float* G,
             lora_backward(g_hidden, attn_out[l], LW + LL.A[3], LW + LL.B[3], LGW + LL.A[3], LGW + LL.B[3], ltmp, T, qd, h, r, ls);
         memset(g_k, 0, (size_t)(T * kv) * 4); memset(g_v, 0, (size_t)(T * kv) * 4);
         orc_attention_backward(cq[l], ck[l], cv[l], g_attn, g_q, g_k, g_v, starts, batch, T, H, KVH, D, scale);
+        if (c->use_qk_norm) {
+            float* tq = fnew(T * qd); float* tk = fnew(T * kv);
+            orc_qk_norm_backward(pq[l], g_q, tq, T, H, D, eps);
+            orc_qk_norm_backward(pk[l], g_k, tk, T, KVH, D, eps);
+            memcpy(g_q, tq, (size_t)(T * qd) * 4); memcpy(g_k, tk, (size_t)(T * kv) * 4);
+            free(tq); free(tk);
+        }
         orc_rope(g_q, g_q, starts, batch, T, H, D, c->rope_theta, 1);
         orc_rope(g_k, g_k, starts, batch, T, KVH, D, c->rope_theta, 1);
         if (!lora) {
@@ -832,7 +845,9 @@ static float step_impl(const orc_config_t* c, const float* P, float* G,
     for (int l = 0; l < NL; l++) {
         free(layer_in[l]); free(xn_attn[l]); free(cq[l]); free(ck[l]); free(cv[l]); free(attn_out[l]);
         free(post_in[l]); free(xn_ffn[l]); free(gate[l]); free(up[l]); free(silu_out[l]); free(ffn_h[l]);
+        free(pq[l]); free(pk[l]);
     }
+    free(pq); free(pk);
     free(layer_in); free(xn_attn); free(cq); free(ck); free(cv); free(attn_out); free(post_in);
     free(xn_ffn); free(gate); free(up); free(silu_out); free(ffn_h);
     free(hidden); free(tmp_h); free(ltmp); free(final_in); free(xn_final); free(loss_rows);

@@ -160,6 +160,11 @@ typedef struct {
     int32_t lora_rank;
     float   lora_alpha;
     int32_t lora_mask;    /* bit0 q, 1 k, 2 v, 3 o, 4 gate, 5 up, 6 down */
+    /* 1: shaders/qk_norm.comp on q and k after RoPE, as src/train.c:4688-4689 calls it (eps = the step's rms eps),
+     * and its exact derivative in the backward.  The reference's backward has no counterpart (it treats the op as
+     * the identity, src/train.c:5224-5266) and its language-model mode never enables it (src/model_config.c:282):
+     * PARITY UNPINNED by the reference; pinned by float64 autograd of the forward definition only. */
+    int32_t use_qk_norm;
 } orc_config_t;
 
 /* Element offsets of every tensor inside one flat parameter vector:

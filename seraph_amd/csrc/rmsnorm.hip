@@ -395,8 +395,37 @@ __global__ __launch_bounds__(1024) void colsum_add_kernel(const float* __restric
 }
 
 // ---------------------------------------------------------------- qk_norm
-// shaders/qk_norm.comp:38-75: y = x / max(sqrt(mean(x^2)), eps) over all heads of a token.
-__global__ __launch_bounds__(kBlock) void qk_norm_kernel(float* __restrict__ qk, int64_t T, int64_t n, float eps) {
+// shaders/qk_norm.comp:38-75: y = x / max(sqrt(mean(x^2)), eps) over all heads of a token, in place.  One wavefront
+// per token holds the token's n = heads * head_dim values in registers (16-byte streamed accesses, no LDS); rms_out,
+// when given, receives the unclamped root mean square for the backward.
+template <int VPL>
+__global__ __launch_bounds__(kBlock) void qk_norm_vec_kernel(float* __restrict__ qk, float* __restrict__ rms_out,
+                                                             int64_t T, int n, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (t >= T) return;
+    const int n4 = n >> 2;
+    float4* row = reinterpret_cast<float4*>(qk + t * n);
+    float4 v[VPL];
+    float ss = 0.0f;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+        const int i4 = lane + 64 * k;
+        v[k] = i4 < n4 ? ldnt4(row + i4) : make_float4(0, 0, 0, 0);
+        ss += (v[k].x * v[k].x + v[k].y * v[k].y) + (v[k].z * v[k].z + v[k].w * v[k].w);
+    }
+    ss = wave_sum(ss);
+    const float rms = sqrtf(ss / (float)n);
+    const float inv = 1.0f / fmaxf(rms, eps);
+    if (rms_out && lane == 0) rms_out[t] = rms;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+        const int i4 = lane + 64 * k;
+        if (i4 < n4) stnt4(row + i4, make_float4(v[k].x * inv, v[k].y * inv, v[k].z * inv, v[k].w * inv));
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void qk_norm_kernel(float* __restrict__ qk, float* __restrict__ rms_out, int64_t T, int64_t n, float eps) {
     const int lane = threadIdx.x & 63;
     const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
     const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
@@ -405,13 +434,14 @@ __global__ __launch_bounds__(kBlock) void qk_norm_kernel(float* __restrict__ qk,
         float ss = 0.0f;
         for (int64_t c = lane; c < n; c += 64) ss += xr[c] * xr[c];
         ss = wave_sum(ss);
-        float rms = fmaxf(sqrtf(ss / (float)n), eps);
-        float inv = 1.0f / rms;
+        const float rms = sqrtf(ss / (float)n);
+        if (rms_out && lane == 0) rms_out[t] = rms;
+        float inv = 1.0f / fmaxf(rms, eps);
         for (int64_t c = lane; c < n; c += 64) xr[c] *= inv;
     }
 }
 
-// d/dx of the above: dx = dy/r - x (dy.x)/(n r^3) while r = rms > eps; dx = dy/eps when clamped.
+// d/dx of the above from the input: dx = dy/r - x (dy.x)/(n r^3) while r = rms > eps; dx = dy/eps when clamped.
 __global__ __launch_bounds__(kBlock) void qk_norm_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy,
                                                              float* __restrict__ dx, int64_t T, int64_t n, float eps) {
     const int lane = threadIdx.x & 63;
@@ -433,6 +463,60 @@ __global__ __launch_bounds__(kBlock) void qk_norm_bwd_kernel(const float* __rest
             float k = gx / ((float)n * rms * rms * rms);
             for (int64_t c = lane; c < n; c += 64) dx[t * n + c] = gr[c] * inv - xr[c] * k;
         }
+    }
+}
+
+// The same derivative from what the training step has at hand: the normalised output y (which the attention reads
+// and the step keeps) and the saved rms.  With x = r y:  dx = (dy - y (dy.y)/n) / r  while r = rms >= eps, and
+// dx = dy/eps when the forward clamped.  dx may be dy.
+template <int VPL>
+__global__ __launch_bounds__(kBlock) void qk_norm_bwd_saved_vec_kernel(const float* __restrict__ y, const float* __restrict__ rms,
+                                                                       const float* dy, float* dx, int64_t T, int n, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (t >= T) return;
+    const int n4 = n >> 2;
+    const float4* yr = reinterpret_cast<const float4*>(y + t * n);
+    const float4* gr = reinterpret_cast<const float4*>(dy + t * n);
+    float4 yv[VPL], gv[VPL];
+    float gy = 0.0f;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+        const int i4 = lane + 64 * k;
+        yv[k] = i4 < n4 ? ldnt4(yr + i4) : make_float4(0, 0, 0, 0);
+        gv[k] = i4 < n4 ? ldnt4(gr + i4) : make_float4(0, 0, 0, 0);
+        gy += (gv[k].x * yv[k].x + gv[k].y * yv[k].y) + (gv[k].z * yv[k].z + gv[k].w * yv[k].w);
+    }
+    gy = wave_sum(gy);
+    const float r = rms[t];
+    const bool clamped = r < eps;
+    const float inv = 1.0f / (clamped ? eps : r);
+    const float c = clamped ? 0.0f : gy / (float)n;
+    float4* dr = reinterpret_cast<float4*>(dx + t * n);
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+        const int i4 = lane + 64 * k;
+        if (i4 < n4) stnt4(dr + i4, make_float4((gv[k].x - yv[k].x * c) * inv, (gv[k].y - yv[k].y * c) * inv,
+                                                (gv[k].z - yv[k].z * c) * inv, (gv[k].w - yv[k].w * c) * inv));
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void qk_norm_bwd_saved_kernel(const float* __restrict__ y, const float* __restrict__ rms,
+                                                                   const float* dy, float* dx, int64_t T, int64_t n, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+    for (int64_t t = wave; t < T; t += nwaves) {
+        const float* yr = y + t * n;
+        const float* gr = dy + t * n;
+        float gy = 0.0f;
+        for (int64_t c = lane; c < n; c += 64) gy += gr[c] * yr[c];
+        gy = wave_sum(gy);                                     // every lane has read its dy before any lane writes dx
+        const float r = rms[t];
+        const bool clamped = r < eps;
+        const float inv = 1.0f / (clamped ? eps : r);
+        const float k = clamped ? 0.0f : gy / (float)n;
+        for (int64_t c = lane; c < n; c += 64) dx[t * n + c] = (gr[c] - yr[c] * k) * inv;
     }
 }
 
@@ -626,11 +710,55 @@ int seraph_rmsnorm_backward_static(const float* x, const float* scale, const flo
 }
 
 int seraph_qk_norm(float* qk, int64_t T, int heads, int head_dim, int use_qk_norm, float eps, seraph_stream_t s) {
-    if (!use_qk_norm || T == 0) return SERAPH_OK;                 // shaders/qk_norm.comp:32
-    SERAPH_REQUIRE(qk && heads > 0 && head_dim > 0, "qk_norm: bad argument");
-    int64_t want = ceil_div(T, kWavesPerBlock), cap = (int64_t)num_compute_units() * 8;
-    hipLaunchKernelGGL(qk_norm_kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(kBlock), 0, as_stream(s),
-                       qk, T, (int64_t)heads * head_dim, eps);
+    if (!use_qk_norm) return SERAPH_OK;                           // shaders/qk_norm.comp:32
+    return seraph_qk_norm_saved(qk, nullptr, T, heads, head_dim, eps, s);
+}
+
+int seraph_qk_norm_saved(float* qk, float* rms_out, int64_t T, int heads, int head_dim, float eps, seraph_stream_t s) {
+    if (T == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(qk && heads > 0 && head_dim > 0 && T > 0, "qk_norm: bad argument");
+    const int64_t n = (int64_t)heads * head_dim;
+    const int vpl = aligned16(qk) ? pick_vpl(n) : 0;
+    hipStream_t st = as_stream(s);
+    const dim3 grid((unsigned)ceil_div(T, kWavesPerBlock));
+#define QKN(V) hipLaunchKernelGGL(qk_norm_vec_kernel<V>, grid, dim3(kBlock), 0, st, qk, rms_out, T, (int)n, eps)
+    switch (vpl) {
+        case 1: QKN(1); break;
+        case 2: QKN(2); break;
+        case 4: QKN(4); break;
+        case 8: QKN(8); break;
+        case 16: QKN(16); break;
+        default: {
+            int64_t want = ceil_div(T, kWavesPerBlock), cap = (int64_t)num_compute_units() * 8;
+            hipLaunchKernelGGL(qk_norm_kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(kBlock), 0, st, qk, rms_out, T, n, eps);
+        }
+    }
+#undef QKN
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
+}
+
+int seraph_qk_norm_backward_saved(const float* y, const float* rms, const float* dy, float* dx, int64_t T, int heads, int head_dim,
+                                  float eps, seraph_stream_t s) {
+    if (T == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(y && rms && dy && dx && heads > 0 && head_dim > 0 && T > 0, "qk_norm_backward_saved: bad argument");
+    const int64_t n = (int64_t)heads * head_dim;
+    const int vpl = (aligned16(y) && aligned16(dy) && aligned16(dx)) ? pick_vpl(n) : 0;
+    hipStream_t st = as_stream(s);
+    const dim3 grid((unsigned)ceil_div(T, kWavesPerBlock));
+#define QKB(V) hipLaunchKernelGGL(qk_norm_bwd_saved_vec_kernel<V>, grid, dim3(kBlock), 0, st, y, rms, dy, dx, T, (int)n, eps)
+    switch (vpl) {
+        case 1: QKB(1); break;
+        case 2: QKB(2); break;
+        case 4: QKB(4); break;
+        case 8: QKB(8); break;
+        case 16: QKB(16); break;
+        default: {
+            int64_t want = ceil_div(T, kWavesPerBlock), cap = (int64_t)num_compute_units() * 8;
+            hipLaunchKernelGGL(qk_norm_bwd_saved_kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(kBlock), 0, st, y, rms, dy, dx, T, n, eps);
+        }
+    }
+#undef QKB
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }

@@ -117,11 +117,11 @@ def attention_forward(Q, K, V, heads, kv_heads, head_dim, seq_starts=None, scale
 
 
 def attention_backward(Q, K, V, dO, heads, kv_heads, head_dim, seq_starts=None, scale=None, out=None, lse=None,
-                       dK=None, dV=None, max_seq_len=None):
+                       dK=None, dV=None, max_seq_len=None, dQ=None):
     """max_seq_len: a bound on the longest packed sequence; when given, the scratch is sized for the
     dS band and the 5-product path runs (seraph_attention_backward_banded)."""
     T = Q.shape[0]
-    dQ = torch.empty_like(Q)
+    dQ = torch.empty_like(Q) if dQ is None else dQ
     dK = torch.zeros_like(K) if dK is None else dK
     dV = torch.zeros_like(V) if dV is None else dV
     scale = head_dim ** -0.5 if scale is None else scale
@@ -193,10 +193,25 @@ def qk_norm_(x, heads, head_dim, eps, use_qk_norm=1):
     return x
 
 
-def qk_norm_backward(x_pre, dy, heads, head_dim, eps):
-    dx = torch.empty_like(x_pre)
+def qk_norm_backward(x_pre, dy, heads, head_dim, eps, out=None):
+    dx = torch.empty_like(x_pre) if out is None else out
     check(kernels().seraph_qk_norm_backward(_p(x_pre), _p(dy), _p(dx), i64(x_pre.shape[0]), C.c_int(heads),
                                             C.c_int(head_dim), f32(eps), _stream()), "qk_norm_backward")
+    return dx
+
+
+def qk_norm_saved_(x, heads, head_dim, eps):
+    """In place; returns (x, rms per token) as the training step keeps them."""
+    rms = torch.empty(x.shape[0], dtype=torch.float32, device=x.device)
+    check(kernels().seraph_qk_norm_saved(_p(x), _p(rms), i64(x.shape[0]), C.c_int(heads), C.c_int(head_dim), f32(eps), _stream()),
+          "qk_norm_saved")
+    return x, rms
+
+
+def qk_norm_backward_saved(y, rms, dy, heads, head_dim, eps, out=None):
+    dx = torch.empty_like(y) if out is None else out
+    check(kernels().seraph_qk_norm_backward_saved(_p(y), _p(rms), _p(dy), _p(dx), i64(y.shape[0]), C.c_int(heads),
+                                                  C.c_int(head_dim), f32(eps), _stream()), "qk_norm_backward_saved")
     return dx
 
 
@@ -218,8 +233,8 @@ def mul_backward(A, B, dC):
     return dA, dB
 
 
-def swiglu_backward(gate, up, dH):
-    dG, dU = torch.empty_like(gate), torch.empty_like(gate)
+def swiglu_backward(gate, up, dH, out=None):
+    dG, dU = (torch.empty_like(gate), torch.empty_like(gate)) if out is None else out
     check(kernels().seraph_swiglu_backward(_p(gate), _p(up), _p(dH), _p(dG), _p(dU), sz(gate.numel()), _stream()),
           "swiglu_backward")
     return dG, dU

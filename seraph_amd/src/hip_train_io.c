@@ -340,6 +340,7 @@ int hip_model_config_load(const char* model_dir, hip_model_config_t* cfg) {
         const jnode_t* rp = j_get(src, "rope_parameters");
         cfg->rope_theta = rp ? j_float(rp, "rope_theta", 10000.0f) : 10000.0f;
     }
+    cfg->use_qk_norm = j_int(src, "use_qk_norm", 0) ? 1 : 0;              /* src/model_config.c:282 */
     json_free(root);
     if (cfg->vocab < 1 || cfg->hidden < 1 || cfg->layers < 1 || cfg->ffn < 1 || cfg->heads < 1 || cfg->kv_heads < 1 || cfg->head_dim < 1) {
         IO_ERR("config.json holds a non-positive model dimension");

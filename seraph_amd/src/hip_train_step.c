@@ -28,6 +28,7 @@ typedef struct { int64_t A[7], B[7], in[7], out[7], stride; } lora_layout_t;   /
 
 typedef struct {
     float *layer_in, *xn_attn, *q, *k, *v, *attn_out, *lse, *post_in, *xn_ffn, *gate, *up, *ffn_h;
+    float *rms_q, *rms_k;        /* per token, with use_qk_norm */
 } layer_act_t;
 
 struct hip_trainer {
@@ -280,7 +281,7 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
         const size_t qd = (size_t)cfg->heads * cfg->head_dim, kv = (size_t)cfg->kv_heads * cfg->head_dim;
         const size_t r = cfg->lora_rank > 0 ? (size_t)cfg->lora_rank : 1;
         const size_t per_layer = 4 * up256(T * h * 4) + 2 * up256(T * qd * 4) + 2 * up256(T * kv * 4) +
-                                 up256(T * cfg->heads * 4) + 3 * up256(T * f * 4);
+                                 up256(T * cfg->heads * 4) + 3 * up256(T * f * 4) + (cfg->use_qk_norm ? 2 * up256(T * 4) : 0);
         const size_t rest = 2 * up256(T * h * 4) + up256(T * Vv * 4) + 3 * up256(T * 4) + up256(T * h * 4) + up256(T * r * 4) +
                             3 * up256(T * h * 4) + 3 * up256(T * f * 4) + 2 * up256(T * qd * 4) + 2 * up256(T * kv * 4) +
                             up256(h * 4) + 2 * up256(T * 4) + up256(((size_t)max_batch + 1) * 4);
@@ -295,6 +296,7 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
             TAKE(a->layer_in, T * h * 4); TAKE(a->xn_attn, T * h * 4); TAKE(a->post_in, T * h * 4); TAKE(a->xn_ffn, T * h * 4);
             TAKE(a->q, T * qd * 4); TAKE(a->attn_out, T * qd * 4); TAKE(a->k, T * kv * 4); TAKE(a->v, T * kv * 4);
             TAKE(a->lse, T * cfg->heads * 4);
+            if (cfg->use_qk_norm) { TAKE(a->rms_q, T * 4); TAKE(a->rms_k, T * 4); }
             TAKE(a->gate, T * f * 4); TAKE(a->up, T * f * 4); TAKE(a->ffn_h, T * f * 4);
         }
         TAKE(t->final_in, T * h * 4); TAKE(t->xn_final, T * h * 4); TAKE(t->logits, T * Vv * 4);
@@ -563,6 +565,10 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         GEMM(a->xn_attn, W + t->L.v, a->v, T, kv, h, 0, 1, 0);
         if (lora && t->LL.A[2] >= 0 && lora_forward_add(t, a->xn_attn, a->v, LW + t->LL.A[2], LW + t->LL.B[2], T, h, kv)) return -1.0f;
         OP("rope", 0.0, 8.0 * (double)(T * (qd + kv)), seraph_rope_qk(a->q, a->q, H, a->k, a->k, KVH, starts, batch, T, D, theta, 0, s));
+        if (c->use_qk_norm) {                                              /* after RoPE, before the attention: src/train.c:4687-4689 */
+            OP("qk_norm", 0.0, 8.0 * (double)(T * qd), seraph_qk_norm_saved(a->q, a->rms_q, T, H, D, eps, s));
+            OP("qk_norm", 0.0, 8.0 * (double)(T * kv), seraph_qk_norm_saved(a->k, a->rms_k, T, KVH, D, eps, s));
+        }
         OP("attention_forward", 4.0 * D * t->attn_pairs * H, 0.0, seraph_attention_forward(a->q, a->k, a->v, a->attn_out, a->lse, starts, batch, T, H, KVH, D, scale, s));
         GEMM(a->attn_out, W + t->L.o, t->tmp_h, T, h, qd, 0, 1, 0);
         if (lora && t->LL.A[3] >= 0 && lora_forward_add(t, a->attn_out, t->tmp_h, LW + t->LL.A[3], LW + t->LL.B[3], T, qd, h)) return -1.0f;
@@ -655,6 +661,10 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         NANCHK(t->g_q, T * qd, nan_bwd + 5u * (uint32_t)l + 1u);
         NANCHK(t->g_k, T * kv, nan_bwd + 5u * (uint32_t)l + 2u);
         NANCHK(t->g_v, T * kv, nan_bwd + 5u * (uint32_t)l + 3u);
+        if (c->use_qk_norm) {                                              /* from the kept outputs and the saved rms, in place */
+            OP("qk_norm_backward", 0.0, 12.0 * (double)(T * qd), seraph_qk_norm_backward_saved(a->q, a->rms_q, t->g_q, t->g_q, T, H, D, eps, s));
+            OP("qk_norm_backward", 0.0, 12.0 * (double)(T * kv), seraph_qk_norm_backward_saved(a->k, a->rms_k, t->g_k, t->g_k, T, KVH, D, eps, s));
+        }
         OP("rope", 0.0, 8.0 * (double)(T * (qd + kv)), seraph_rope_qk(t->g_q, t->g_q, H, t->g_k, t->g_k, KVH, starts, batch, T, D, theta, 1, s));
         NANCHK(t->g_q, T * qd, nan_bwd + 5u * (uint32_t)l + 4u);
         if (!lora) {

@@ -13,7 +13,7 @@ class ModelConfig(C.Structure):
     _fields_ = [("hidden", C.c_int32), ("layers", C.c_int32), ("heads", C.c_int32), ("kv_heads", C.c_int32),
                 ("head_dim", C.c_int32), ("ffn", C.c_int32), ("vocab", C.c_int32), ("rms_eps", C.c_float),
                 ("rope_theta", C.c_float), ("lora_rank", C.c_int32), ("lora_alpha", C.c_float),
-                ("lora_mask", C.c_int32)]
+                ("lora_mask", C.c_int32), ("use_qk_norm", C.c_int32)]
 
 
 class OptimConfig(C.Structure):
@@ -41,9 +41,9 @@ PARAMS, GRADS, ADAM_M, ADAM_V, LORA_PARAMS, LORA_GRADS, LORA_M, LORA_V = range(8
 
 
 def model_config(hidden, layers, heads, kv_heads, head_dim, ffn, vocab, rms_eps=1e-5, rope_theta=10000.0,
-                 lora_rank=0, lora_alpha=0.0, lora_mask=0):
+                 lora_rank=0, lora_alpha=0.0, lora_mask=0, use_qk_norm=0):
     return ModelConfig(hidden, layers, heads, kv_heads, head_dim, ffn, vocab, rms_eps, rope_theta, lora_rank,
-                       lora_alpha, lora_mask)
+                       lora_alpha, lora_mask, use_qk_norm)
 
 
 def optim_config(learning_rate, beta1=0.9, beta2=0.999, weight_decay=0.01, eps=1e-8, clip=0.0, warmup_steps=100,

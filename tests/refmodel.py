@@ -66,6 +66,12 @@ def rope(x, pos, heads, D, theta):
     return torch.stack([x0 * c - x1 * s, x0 * s + x1 * c], -1).reshape(T, heads * D)
 
 
+def qk_norm(x, eps):
+    """shaders/qk_norm.comp:38-75: every token's vector over all heads divided by max(its root mean square, eps)."""
+    rms = torch.sqrt((x * x).mean(-1, keepdim=True))
+    return x / torch.clamp(rms, min=float(eps))
+
+
 def attention(q, k, v, seq_id, H, KVH, D):
     T = q.shape[0]
     q = q.view(T, H, D).transpose(0, 1)
@@ -105,6 +111,8 @@ def loss_fn(cfg, P, tokens, seq_starts, lora=None, drop_adapter_dgrad=True):
         q = rope(proj(xn, W["q"], ad.get("q")), pos, H, D, cfg.rope_theta)
         k = rope(proj(xn, W["k"], ad.get("k")), pos, KVH, D, cfg.rope_theta)
         v = proj(xn, W["v"], ad.get("v"))
+        if getattr(cfg, "use_qk_norm", 0):                   # after RoPE, before the attention (src/train.c:4687-4689)
+            q, k = qk_norm(q, cfg.rms_eps), qk_norm(k, cfg.rms_eps)
         a = attention(q, k, v, seq_id, H, KVH, D)
         x = x + proj(a, W["o"], ad.get("o"))
         xn = rmsnorm(x, W["post_norm"], cfg.rms_eps)

@@ -213,3 +213,20 @@ def test_attention_backward_16384_tokens_gqa_d128(ops, orc):
     parity(seven[0], host(dQ), "dQ, 7-product vs 5-product path", atol=1e-6)
     assert torch.equal(seven[1], dK) and torch.equal(seven[2], dV)
     assert bool(torch.isfinite(dQ).all() and torch.isfinite(dK).all() and torch.isfinite(dV).all())
+
+
+# ------------------------------------------------------------------ qk_norm, 16384 x 16 heads x 128
+def test_qk_norm_pair_16384_x_16_heads_128(ops, orc):
+    """The step's qk_norm pair at the benchmark shape's query width, against the oracle (forward, and the derivative
+    computed from the input), plus the identity sum(y^2) = n for every unclamped token and <dx, x> = 0 (the derivative
+    of a scale-invariant map is orthogonal to its input)."""
+    T, heads, D = 16384, 16, 128
+    r = np.random.default_rng(33)
+    x = r.standard_normal((T, heads * D)).astype(np.float32)
+    dy = r.standard_normal((T, heads * D)).astype(np.float32)
+    y, rms = ops.qk_norm_saved_(dev(x), heads, D, 1e-6)
+    parity(y, orc.qk_norm(x, heads, D, 1e-6), "qk_norm forward")
+    dx = ops.qk_norm_backward_saved(y, rms, dev(dy), heads, D, 1e-6)
+    parity(dx, orc.qk_norm_backward(x, dy, heads, D, 1e-6), "qk_norm backward", atol=2e-5)
+    assert float(((y.double() ** 2).sum(1) - heads * D).abs().max()) < 1e-2
+    assert float((dx.double() * dev(x).double()).sum(1).abs().max()) < 1e-2

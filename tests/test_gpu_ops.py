@@ -268,6 +268,26 @@ def test_qk_norm(ops, orc):
     parity(ops.qk_norm_backward(dev(x), dev(dy), 4, 64, 1e-6), orc.qk_norm_backward(x, dy, 4, 64, 1e-6), "qk_norm bwd")
 
 
+@pytest.mark.parametrize("T,heads,D", [(37, 4, 64), (300, 16, 128), (5, 3, 6), (1000, 8, 128), (64, 2, 32)])
+def test_qk_norm_saved_pair(ops, orc, T, heads, D):
+    """The pair the training step uses: the forward that also leaves each token's rms, and the backward from the
+    normalised output and that rms.  Same derivative as the backward from the input (the oracle's), also in place, also
+    for tokens whose norm is clamped at eps."""
+    r = rng(T + heads)
+    eps = 1e-3
+    x = r.standard_normal((T, heads * D)).astype(np.float32)
+    x[1] *= 1e-5                                                  # rms below eps: clamped
+    x[3] = 0
+    dy = r.standard_normal((T, heads * D)).astype(np.float32)
+    y, rms = ops.qk_norm_saved_(dev(x), heads, D, eps)
+    parity(y, orc.qk_norm(x, heads, D, eps), "qk_norm forward")
+    parity(rms, np.sqrt((x.astype(np.float64) ** 2).mean(1)), "saved rms", atol=1e-7)
+    ref = orc.qk_norm_backward(x, dy, heads, D, eps)
+    parity(ops.qk_norm_backward_saved(y, rms, dev(dy), heads, D, eps), ref, "qk_norm backward from the output", atol=2e-5 if T else ATOL)
+    g = dev(dy)
+    parity(ops.qk_norm_backward_saved(y, rms, g, heads, D, eps, out=g), ref, "in place", atol=2e-5)
+
+
 # ------------------------------------------------------------------ rope
 @pytest.mark.parametrize("heads,D,theta,starts", [(8, 64, 10000.0, [0, 256, 300]), (16, 128, 1e6, [0, 4096]),
                                                   (3, 16, 10000.0, [0, 1, 2, 50]), (4, 64, 10000.0, [0, 7, 7, 40, 40])])

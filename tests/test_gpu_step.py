@@ -172,6 +172,38 @@ def test_lora_step(tr, orc, b_zero, mask):
     t.close()
 
 
+@pytest.mark.parametrize("lora", [False, True])
+def test_step_with_qk_norm(tr, orc, lora):
+    """use_qk_norm = 1 in both step drivers: forward after RoPE, derivative before the RoPE backward (the reference's
+    backward has no such term: parity unpinned by the reference; the oracle's is pinned by float64 autograd)."""
+    case = dict(hidden=128, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=192, vocab=211, rms_eps=1e-5, use_qk_norm=1)
+    if lora:
+        case.update(lora_rank=8, lora_alpha=16.0, lora_mask=0b1111)
+    ocfg, cfg = orc.make_config(**case), tr.model_config(**case)
+    p = init_params(orc, ocfg, 21)
+    starts = np.array([0, 70, 71, 200], np.int32)
+    tok = rng(22).integers(0, 211, 200).astype(np.int32)
+    t = tr.Trainer(cfg, tr.optim_config(1e-3), max_tokens=200, max_batch=3)
+    t.upload(tr.PARAMS, p)
+    if lora:
+        lo = (0.05 * rng(23).standard_normal(orc.lora_param_count(ocfg))).astype(np.float32)
+        t.upload(tr.LORA_PARAMS, lo)
+        ref_loss, ref_g = orc.step_lora(ocfg, p, lo, tok, starts)
+    else:
+        ref_loss, ref_g = orc.step_full(ocfg, p, tok, starts)
+    loss = t.step(tok, starts, run_optimizer=False)
+    assert abs(loss - ref_loss) < 1e-5 * max(1.0, abs(ref_loss))
+    g = t.download(tr.LORA_GRADS if lora else tr.GRADS).astype(np.float64)
+    bad = np.abs(g - ref_g) > ATOL + RTOL * np.abs(ref_g)
+    assert not bad.any(), f"{bad.sum()} gradients outside tolerance, max {np.abs(g - ref_g).max():.3e}"
+    assert np.linalg.norm(g - ref_g) <= 1e-4 * np.linalg.norm(ref_g)
+    # the same model without the switch gives another gradient: the option is live
+    off = dict(case, use_qk_norm=0)
+    g_off = (orc.step_lora(orc.make_config(**off), p, lo, tok, starts) if lora else orc.step_full(orc.make_config(**off), p, tok, starts))[1]
+    assert np.linalg.norm(g_off - ref_g) > 1e-2 * np.linalg.norm(ref_g)
+    t.close()
+
+
 def test_step_rejects_bad_batches(tr):
     from seraph_amd._lib import SeraphError
     cfg = tr.model_config(64, 1, 2, 2, 32, 64, 50)

@@ -386,6 +386,41 @@ def test_step_full_vs_autograd(orc):
     assert np.linalg.norm(grads2 - 2 * g) <= 4e-6 * np.linalg.norm(g)
 
 
+@pytest.mark.parametrize("lora", [False, True])
+def test_step_with_qk_norm_vs_autograd(orc, lora):
+    """use_qk_norm = 1: q and k divided by their root mean square over all heads of a token after RoPE, and the exact
+    derivative in the backward (the reference's backward has none: parity unpinned by the reference, pinned here by
+    float64 autograd of the forward definition).  One token's q is made tiny so that its norm is clamped at eps."""
+    kw = dict(use_qk_norm=1, rms_eps=1e-3)
+    if lora:
+        kw.update(lora_rank=4, lora_alpha=8.0, lora_mask=0b1111)
+    cfg = _tiny_cfg(orc, **kw)
+    p = _init(orc, cfg, 110)
+    r = rng(111)
+    starts = np.array([0, 9, 26], np.int32)
+    tok = r.integers(0, cfg.vocab, 26).astype(np.int32)
+    P32 = refmodel.split_params(cfg, torch.from_numpy(p))
+    P32["embed"][tok[5]] *= 1e-4                                  # a token whose q and k are far below eps in layer 0
+    if lora:
+        lo = (0.05 * r.standard_normal(orc.lora_param_count(cfg))).astype(np.float32)
+        loss, grads = orc.step_lora(cfg, p, lo, tok, starts)
+        flat = torch.tensor(lo, dtype=torch.float64, requires_grad=True)
+        ref = refmodel.loss_fn(cfg, refmodel.split_params(cfg, torch.tensor(p, dtype=torch.float64)), tok, starts,
+                               lora=refmodel.split_lora(cfg, flat), drop_adapter_dgrad=True)
+    else:
+        loss, grads = orc.step_full(cfg, p, tok, starts)
+        flat = torch.tensor(p, dtype=torch.float64, requires_grad=True)
+        ref = refmodel.loss_fn(cfg, refmodel.split_params(cfg, flat), tok, starts)
+    ref.backward()
+    assert abs(loss - ref.item()) < 1e-5
+    g = flat.grad.numpy()
+    assert np.linalg.norm(grads - g) <= 3e-6 * np.linalg.norm(g)
+    # and the switch matters: without it the gradient is a different one
+    off = _tiny_cfg(orc, **dict(kw, use_qk_norm=0))
+    g_off = orc.step_lora(off, p, lo, tok, starts)[1] if lora else orc.step_full(off, p, tok, starts)[1]
+    assert np.linalg.norm(g_off - g) > 1e-2 * np.linalg.norm(g)
+
+
 def test_step_full_single_sequence_equals_unpacked(orc):
     cfg = _tiny_cfg(orc, kv_heads=4)
     p = _init(orc, cfg, 102)
