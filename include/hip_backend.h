@@ -197,6 +197,13 @@ void hip_qk_norm_backward(vulkan_context_t* ctx, vulkan_buffer_t* qk_pre, vulkan
 void hip_adamw_update_clipped(vulkan_context_t* ctx, vulkan_buffer_t* weight, vulkan_buffer_t* grad, vulkan_buffer_t* m,
                               vulkan_buffer_t* v, float lr, float beta1, float beta2, float weight_decay, float eps,
                               int step, size_t size, float clip);
+/* vulkan_adamw_update over `count` tensors as one recorded op: a maintainer replaces the body of
+ * full_weights_optimizer_step_gpu_resident_record (src/train.c:4225-4284: one vulkan_adamw_update and one barrier per
+ * tensor, 2 + 9 L of them) by filling the four arrays and calling this once.  sizes are element counts; NULL entries
+ * or zero sizes are skipped like the single-tensor op skips them.  Bit-identical to the per-tensor calls. */
+void hip_adamw_update_multi(vulkan_context_t* ctx, int count, vulkan_buffer_t* const* weights, vulkan_buffer_t* const* grads,
+                            vulkan_buffer_t* const* m, vulkan_buffer_t* const* v, const size_t* sizes,
+                            float lr, float beta1, float beta2, float weight_decay, float eps, int step, float clip);
 /* sum = input + addend, output = rmsnorm(sum): the vulkan_add that closes a residual branch and the vulkan_rmsnorm
  * that reads its result (src/train.c:4705-4711) in one pass; sum is a buffer of its own */
 void hip_add_rmsnorm(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* addend, vulkan_buffer_t* sum,

@@ -251,6 +251,15 @@ int seraph_adamw(float* w, const float* g, float* m, float* v, size_t n,
                  float lr, float beta1, float beta2, float weight_decay, float eps, int step, float clip,
                  seraph_stream_t s);
 
+/* The same update for a list of tensors in one launch (48 per launch for longer lists): the reference records one
+ * vulkan_adamw_update and one barrier per tensor, 2 + 9 L of them per optimizer step (src/train.c:4225-4284).
+ * `tensors` is a HOST array; the descriptors travel as kernel arguments.  Every element receives exactly the
+ * arithmetic of seraph_adamw, so the results are bit-identical to per-tensor calls.  Tensors must not overlap. */
+typedef struct { float* w; const float* g; float* m; float* v; size_t n; } seraph_adamw_tensor_t;
+int seraph_adamw_multi(const seraph_adamw_tensor_t* tensors, int count,
+                       float lr, float beta1, float beta2, float weight_decay, float eps, int step, float clip,
+                       seraph_stream_t s);
+
 #ifdef __cplusplus
 }
 #endif

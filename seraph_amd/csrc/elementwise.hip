@@ -168,6 +168,34 @@ struct AdamWOp {
     __device__ void one(size_t i) const { float W = w[i], M = m[i], V = v[i]; elem(W, g[i], M, V); m[i] = M; v[i] = V; w[i] = W; }
 };
 
+// ---------------------------------------------------------------- AdamW over a list of tensors
+// The per-tensor launches of the reference's optimizer step (2 + 9 L of them, src/train.c:4225-4284) as one: the
+// descriptors travel in the kernel arguments (no table in device memory, no copy), a workgroup finds its tensor by
+// the running block counts and then does what stream_kernel<AdamWOp> does for that tensor, so every element gets
+// the same arithmetic in the same order as with seraph_adamw.
+constexpr int kMultiMax = 48;            // tensors per launch: 48 x 40 bytes of arguments
+struct AdamWMultiArgs {
+    float* w[kMultiMax]; const float* g[kMultiMax]; float* m[kMultiMax]; float* v[kMultiMax];
+    unsigned long long n[kMultiMax];     // elements; bit 63: the tensor's pointers allow 16-byte slots
+    unsigned int first_block[kMultiMax + 1];
+    int count;
+    float lr, beta1, beta2, wd, eps, bc1, bc2, clip;
+};
+
+__global__ __launch_bounds__(kStreamBlock) void adamw_multi_kernel(const AdamWMultiArgs a) {
+    int lo = 0, hi = a.count - 1;                              // last tensor whose first block is <= blockIdx.x (uniform)
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (a.first_block[mid] <= blockIdx.x) lo = mid; else hi = mid - 1;
+    }
+    const size_t n = (size_t)(a.n[lo] & 0x7fffffffffffffffull);
+    const size_t n4 = (a.n[lo] >> 63) ? n / 4 : 0;
+    const AdamWOp op{a.w[lo], a.g[lo], a.m[lo], a.v[lo], a.lr, a.beta1, a.beta2, a.wd, a.eps, a.bc1, a.bc2, a.clip};
+    const size_t i = (size_t)(blockIdx.x - a.first_block[lo]) * kStreamBlock + threadIdx.x;
+    if (i < n4) op.vec(i);
+    else if (i - n4 < n - 4 * n4) op.one(4 * n4 + (i - n4));
+}
+
 // ---------------------------------------------------------------- nan check, reduce
 __global__ __launch_bounds__(kBlock) void nan_check_kernel(const float* __restrict__ x, size_t n,
                                                            uint32_t* flags, uint32_t flag_index) {
@@ -267,6 +295,48 @@ int seraph_adamw(float* w, const float* g, float* m, float* v, size_t n,
     float bc2 = 1.0f - powf(beta2, (float)step);
     return launch_stream(AdamWOp{w, g, m, v, lr, beta1, beta2, weight_decay, eps, bc1, bc2, clip}, n,
                          ALL_ALIGNED(w, g, m, v), as_stream(s));
+}
+
+int seraph_adamw_multi(const seraph_adamw_tensor_t* tensors, int count,
+                       float lr, float beta1, float beta2, float weight_decay, float eps, int step, float clip,
+                       seraph_stream_t s) {
+    if (count <= 0) return SERAPH_OK;
+    SERAPH_REQUIRE(tensors, "adamw_multi: NULL tensor list");
+    SERAPH_REQUIRE(step >= 1, "adamw_multi: step must be >= 1 (got %d)", step);
+    for (int i = 0; i < count; i++)
+        SERAPH_REQUIRE(tensors[i].n == 0 || (tensors[i].w && tensors[i].g && tensors[i].m && tensors[i].v),
+                       "adamw_multi: NULL pointer in tensor %d", i);
+    AdamWMultiArgs a;
+    a.lr = lr; a.beta1 = beta1; a.beta2 = beta2; a.wd = weight_decay; a.eps = eps; a.clip = clip;
+    a.bc1 = 1.0f - powf(beta1, (float)step);          // src/vulkan_backend.c:2151-2152
+    a.bc2 = 1.0f - powf(beta2, (float)step);
+    int i = 0;
+    while (i < count) {
+        int k = 0;
+        unsigned long long blocks = 0;
+        for (; i < count && k < kMultiMax; i++) {
+            const seraph_adamw_tensor_t& t = tensors[i];
+            if (t.n == 0) continue;
+            const bool vec = ALL_ALIGNED(t.w, t.g, t.m, t.v);
+            const size_t n4 = vec ? t.n / 4 : 0;
+            const unsigned long long nb = (n4 + (t.n - 4 * n4) + kStreamBlock - 1) / kStreamBlock;
+            if (blocks + nb > 0x7fffffffull) {
+                if (k == 0) { set_error("adamw_multi: tensor %d of %zu elements exceeds the launch limit", i, t.n); return SERAPH_ERR_INVALID; }
+                break;                                 // the rest goes into the next launch
+            }
+            a.w[k] = t.w; a.g[k] = t.g; a.m[k] = t.m; a.v[k] = t.v;
+            a.n[k] = (unsigned long long)t.n | (vec ? 1ull << 63 : 0ull);
+            a.first_block[k] = (unsigned int)blocks;
+            blocks += nb;
+            k++;
+        }
+        if (k == 0) continue;
+        a.first_block[k] = (unsigned int)blocks;
+        a.count = k;
+        hipLaunchKernelGGL(adamw_multi_kernel, dim3((unsigned)blocks), dim3(kStreamBlock), 0, as_stream(s), a);
+        SERAPH_LAUNCH_CHECK();
+    }
+    return SERAPH_OK;
 }
 
 int seraph_nan_check(const float* x, size_t n, uint32_t* flags, uint32_t flag_index, seraph_stream_t s) {

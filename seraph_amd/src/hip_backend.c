@@ -406,6 +406,24 @@ void hip_adamw_update_clipped(vulkan_context_t* ctx, vulkan_buffer_t* weight, vu
     HIP_OP(ctx, "adamw", seraph_adamw(FPTR(weight), FPTR(grad), FPTR(m), FPTR(v), size, lr, beta1, beta2, weight_decay, eps, step, clip, st->stream));
 }
 
+void hip_adamw_update_multi(vulkan_context_t* ctx, int count, vulkan_buffer_t* const* weights, vulkan_buffer_t* const* grads,
+                            vulkan_buffer_t* const* m, vulkan_buffer_t* const* v, const size_t* sizes,
+                            float lr, float beta1, float beta2, float weight_decay, float eps, int step, float clip) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || count <= 0 || !weights || !grads || !m || !v || !sizes) return;
+    seraph_adamw_tensor_t* list = (seraph_adamw_tensor_t*)malloc((size_t)count * sizeof(*list));
+    if (!list) { hip_backend_report(ctx, "adamw", SERAPH_ERR_INVALID); return; }
+    int k = 0;
+    for (int i = 0; i < count; i++) {
+        if (!weights[i] || !grads[i] || !m[i] || !v[i] || sizes[i] == 0) continue;      /* as vulkan_adamw_update: silently */
+        list[k].w = FPTR(weights[i]); list[k].g = FPTR(grads[i]); list[k].m = FPTR(m[i]); list[k].v = FPTR(v[i]);
+        list[k].n = sizes[i];
+        k++;
+    }
+    HIP_OP(ctx, "adamw", seraph_adamw_multi(list, k, lr, beta1, beta2, weight_decay, eps, step, clip, st->stream));
+    free(list);
+}
+
 void vulkan_adamw_update(vulkan_context_t* ctx, vulkan_buffer_t* weight, vulkan_buffer_t* grad, vulkan_buffer_t* m,
                          vulkan_buffer_t* v, float lr, float beta1, float beta2, float weight_decay, float eps,
                          int step, size_t size) {

@@ -211,3 +211,51 @@ def test_residual_adds_folded_into_the_norms(vk):
     for buf in (bx, bb, bdy, bs, sum1, y1, sum2, y2, dx1, gs1, gs2, res2):
         lib.vulkan_buffer_free(ctx, buf)
     assert lib.hip_backend_error_count(ctx) == 0
+
+
+def test_adamw_update_multi_equals_per_tensor_updates(vk, orc):
+    """hip_adamw_update_multi over a tensor list (the 2 + 9 L tensors of a model, src/train.c:4225-4284) in one recorded
+    op: bit-identical to one vulkan_adamw_update per tensor, and within tolerance of the oracle.  More tensors than one
+    launch carries (48), odd sizes, an empty and a missing entry."""
+    lib, ctx = vk
+    r = rng(40)
+    sizes = [8192 * 64, 64] + [64, 64 * 64, 48 * 64, 48 * 64, 64 * 64, 64, 96 * 64, 96 * 64, 64 * 96] * 8 + [1, 3, 1027, 0]
+    n = len(sizes)
+    host = [[(0.1 * r.standard_normal(s)).astype(np.float32) for s in sizes] for _ in range(2)]     # w, g
+    host_m = [(1e-3 * r.standard_normal(s)).astype(np.float32) for s in sizes]
+    host_v = [(1e-6 * r.random(s)).astype(np.float32) for s in sizes]
+    hp = (C.c_float(3e-4), C.c_float(0.9), C.c_float(0.999), C.c_float(0.01), C.c_float(1e-8), C.c_int(7))
+
+    def buffers():
+        return [[up(vk, a) if a.size else None for a in arrs] for arrs in (host[0], host[1], host_m, host_v)]
+
+    one = buffers()
+    lib.vulkan_cmd_begin(ctx)
+    for i in range(n):
+        if sizes[i]:
+            lib.vulkan_adamw_update(ctx, one[0][i], one[1][i], one[2][i], one[3][i], *hp, C.c_size_t(sizes[i]))
+    assert lib.vulkan_cmd_end_submit(ctx) == 1
+
+    many = buffers()
+    many[1][5] = None                                              # a missing gradient: that tensor is skipped
+    arr = lambda bufs: (C.POINTER(Buf) * n)(*[b if b is not None else C.POINTER(Buf)() for b in bufs])
+    lib.vulkan_cmd_begin(ctx)
+    lib.hip_adamw_update_multi(ctx, C.c_int(n), arr(many[0]), arr(many[1]), arr(many[2]), arr(many[3]),
+                               (C.c_size_t * n)(*sizes), *hp, C.c_float(0.0))
+    assert lib.vulkan_cmd_end_submit(ctx) == 1
+    assert lib.hip_backend_error_count(ctx) == 0
+    for i in range(n):
+        if not sizes[i]:
+            continue
+        for which, src in ((0, host[0]), (2, host_m), (3, host_v)):
+            got = down(vk, many[which][i], sizes[i])
+            if i == 5:
+                assert (got == src[i]).all()                       # skipped: untouched
+            else:
+                assert (got == down(vk, one[which][i], sizes[i])).all(), (i, which)
+    rw, rm, rv = orc.adamw(host[0][2], host[1][2], host_m[2], host_v[2], 3e-4, 0.9, 0.999, 0.01, 1e-8, 7)
+    close(down(vk, many[0][2], sizes[2]), rw, atol=1e-7)
+    for bufs in one + many:
+        for b in bufs:
+            if b is not None:
+                lib.vulkan_buffer_free(ctx, b)
