@@ -125,8 +125,13 @@ int   hip_trainer_accumulation_counter(const hip_trainer_t* t);
  *   embedding weight / gradient / m / v before AdamW and weight after it,
  * holds AdamW back until the flags have been read, skips it when any is set and returns NAN
  * (src/train.c:5446-5448, :5486-5660).  hip_trainer_nan_flags copies the last step's flags and
- * returns their count; hip_trainer_nan_report prints the "- buffer: ..." lines. */
+ * returns their count; hip_trainer_nan_report prints the "- buffer: ..." lines.
+ * When a step detects a NaN/Inf it also writes the step's buffers for offline inspection, in the files and layouts
+ * of src/train.c:5562-5653 that tools/nan_dump_inspect.c reads: "<prefix>_<step>_meta.txt", "_tokens.u32",
+ * "_hidden.f32", "_logits.f32", "_grad_logits.f32", ..., "_L0_q.f32", "_grad_v.f32".  The prefix defaults to the
+ * reference's "/tmp/seraph_nan_step"; hip_trainer_set_nan_dump_prefix changes it (NULL or "": no dumps). */
 int   hip_trainer_enable_nan_check(hip_trainer_t* t, int on);
+void  hip_trainer_set_nan_dump_prefix(hip_trainer_t* t, const char* prefix);
 int   hip_trainer_nan_detected(const hip_trainer_t* t);
 int   hip_trainer_nan_flags(const hip_trainer_t* t, uint32_t* out, int max);
 void  hip_trainer_nan_report(const hip_trainer_t* t, FILE* out);

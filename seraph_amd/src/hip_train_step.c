@@ -63,6 +63,8 @@ struct hip_trainer {
     float last_lr;
     /* NaN/Inf flag lattice of src/train.c:4499-4546 (off unless enabled) */
     int nan_check, nan_detected;
+    int step_counter;            /* training steps run (state->current_step of the reference) */
+    char nan_dump_prefix[256];   /* "" = no buffer dumps on detection */
     uint32_t* d_nan_flags;
     uint32_t* h_nan_flags;
     uint32_t nan_flag_count;
@@ -252,6 +254,7 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
     t->cfg = *cfg; t->opt = *opt;
     t->max_tokens = max_tokens; t->max_batch = max_batch;
     t->lora = cfg->lora_rank > 0;
+    snprintf(t->nan_dump_prefix, sizeof(t->nan_dump_prefix), "/tmp/seraph_nan_step");   /* src/train.c:5566 */
     make_layouts(t);
     if (seraph_hip_stream_create(&t->stream) != SERAPH_OK) goto fail;
     for (int i = 0; i < 4; i++) if (seraph_hip_event_create(&t->ev[i]) != SERAPH_OK) goto fail;
@@ -507,6 +510,81 @@ static int nan_flags_any(hip_trainer_t* t) {
     return 0;
 }
 
+/* One-shot dump of the step's buffers when the flag lattice reports a NaN/Inf, in the files and layouts of
+ * src/train.c:5562-5653 (raw little-endian FP32 / uint32, "<prefix>_<step>_<name>"), which the reference's
+ * tools/nan_dump_inspect.c reads.  Differences that the layout cannot hide: the cross entropy writes its gradient
+ * over the logits, so logits.f32 is recomputed from hidden_norm and the embedding after grad_logits has been
+ * written; silu(gate) is not cached by this step and is recomputed too; with packed batches targets and
+ * grad_logits hold the first T - 1 rows (rows of sequence-final tokens are zero). */
+static int dump_dev(hip_trainer_t* t, const char* prefix, const char* name, const void* dev, size_t count) {
+    char path[512];
+    snprintf(path, sizeof(path), "%s_%s", prefix, name);
+    FILE* f = fopen(path, "wb");
+    if (!f) return -1;
+    const size_t chunk = (size_t)16 << 20;                     /* elements per round trip */
+    uint32_t* host = (uint32_t*)malloc((count < chunk ? count : chunk) * 4);
+    int rc = host ? 0 : -1;
+    for (size_t o = 0; o < count && rc == 0; o += chunk) {
+        const size_t n = count - o < chunk ? count - o : chunk;
+        if (seraph_hip_d2h(host, (const uint32_t*)dev + o, n * 4, t->stream) != SERAPH_OK || fwrite(host, 4, n, f) != n) rc = -1;
+    }
+    free(host);
+    fclose(f);
+    return rc;
+}
+
+static void nan_dump(hip_trainer_t* t, int total_tokens) {
+    if (!t->nan_dump_prefix[0]) return;
+    const hip_model_config_t* c = &t->cfg;
+    const size_t T = (size_t)total_tokens, h = (size_t)c->hidden, f = (size_t)c->ffn, V = (size_t)c->vocab;
+    const size_t qd = (size_t)c->heads * c->head_dim, kv = (size_t)c->kv_heads * c->head_dim, np = T - 1;
+    char prefix[320], path[400];
+    snprintf(prefix, sizeof(prefix), "%s_%d", t->nan_dump_prefix, t->step_counter + 1);
+    snprintf(path, sizeof(path), "%s_meta.txt", prefix);
+    FILE* meta = fopen(path, "wb");
+    if (meta) {
+        fprintf(meta, "step=%d\nseq=%d\nnum_predictions=%d\nhidden_size=%d\nq_dim=%d\nkv_dim=%d\nvocab_size=%d\n"
+                "num_layers=%d\nnum_heads=%d\nkv_heads=%d\nhead_dim=%d\nlr=%g\n", t->step_counter + 1, total_tokens, (int)np,
+                c->hidden, (int)qd, (int)kv, c->vocab, c->layers, c->heads, c->kv_heads, c->head_dim, (double)t->opt.learning_rate);
+        fclose(meta);
+    }
+    dump_dev(t, prefix, "tokens.u32", t->d_tokens, T);
+    dump_dev(t, prefix, "targets.u32", t->d_targets, np);
+    dump_dev(t, prefix, "hidden.f32", t->final_in, T * h);
+    dump_dev(t, prefix, "hidden_norm.f32", t->xn_final, T * h);
+    dump_dev(t, prefix, "grad_logits.f32", t->logits, np * V);
+    if (seraph_gemm(t->xn_final, t->P + t->off_embed, t->logits, (int64_t)T, (int64_t)V, (int64_t)h, 0, 1, 0, t->stream) == SERAPH_OK)
+        dump_dev(t, prefix, "logits.f32", t->logits, T * V);
+    dump_dev(t, prefix, "grad_hidden.f32", t->g_hidden, T * h);
+    dump_dev(t, prefix, "grad_tmp_hidden.f32", t->g_tmp, T * h);
+    dump_dev(t, prefix, "grad_x_norm.f32", t->g_xn, T * h);
+    dump_dev(t, prefix, "grad_hidden_start.f32", t->g_hidden, T * h);
+    dump_dev(t, prefix, "grad_ffn.f32", t->g_ffn, T * f);
+    dump_dev(t, prefix, "grad_gate.f32", t->g_gate, T * f);
+    dump_dev(t, prefix, "grad_up.f32", t->g_up, T * f);
+    if (c->layers > 0) {
+        const layer_act_t* a = &t->act[0];
+        dump_dev(t, prefix, "L0_layer_in.f32", a->layer_in, T * h);
+        dump_dev(t, prefix, "L0_x_norm_attn.f32", a->xn_attn, T * h);
+        dump_dev(t, prefix, "L0_post_attn_in.f32", a->post_in, T * h);
+        dump_dev(t, prefix, "L0_x_norm_ffn.f32", a->xn_ffn, T * h);
+        dump_dev(t, prefix, "L0_ffn_gate.f32", a->gate, T * f);
+        dump_dev(t, prefix, "L0_ffn_up.f32", a->up, T * f);
+        if (seraph_silu(a->gate, t->g_ffn, T * f, t->stream) == SERAPH_OK)     /* grad_ffn is on disk already */
+            dump_dev(t, prefix, "L0_silu.f32", t->g_ffn, T * f);
+        dump_dev(t, prefix, "L0_ffn_hidden.f32", a->ffn_h, T * f);
+        dump_dev(t, prefix, "L0_q.f32", a->q, T * qd);
+        dump_dev(t, prefix, "L0_k.f32", a->k, T * kv);
+        dump_dev(t, prefix, "L0_v.f32", a->v, T * kv);
+        dump_dev(t, prefix, "L0_attn_out.f32", a->attn_out, T * qd);
+        dump_dev(t, prefix, "grad_attn.f32", t->g_attn, T * qd);
+        dump_dev(t, prefix, "grad_q.f32", t->g_q, T * qd);
+        dump_dev(t, prefix, "grad_k.f32", t->g_k, T * kv);
+        dump_dev(t, prefix, "grad_v.f32", t->g_v, T * kv);
+    }
+    fprintf(stderr, "[NAN-DUMP] wrote buffers with prefix %s_*\n", prefix);
+}
+
 enum { STEP_TRAIN = 0, STEP_EVAL = 1 };
 
 static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, const int* seq_starts, int batch,
@@ -708,6 +786,8 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
                 int any = nan_flags_any(t);
                 if (any) {
                     t->nan_detected = 1;
+                    if (any > 0) nan_dump(t, total_tokens);
+                    t->step_counter++;
                     op_fold(t);
                     return any < 0 ? -1.0f : NAN;
                 }
@@ -730,10 +810,13 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         int any = nan_flags_any(t);
         if (any) {
             t->nan_detected = 1;
+            if (any > 0) nan_dump(t, total_tokens);
+            t->step_counter++;
             op_fold(t);
             return any < 0 ? -1.0f : NAN;
         }
     }
+    t->step_counter++;
 
     float loss_sum = 0.0f;
     CK(seraph_hip_d2h(&loss_sum, red_in, sizeof(float), s));               /* waits for the whole step */
@@ -797,6 +880,11 @@ int hip_trainer_enable_nan_check(hip_trainer_t* t, int on) {
 }
 
 int hip_trainer_nan_detected(const hip_trainer_t* t) { return t ? t->nan_detected : 0; }
+
+void hip_trainer_set_nan_dump_prefix(hip_trainer_t* t, const char* prefix) {
+    if (!t) return;
+    snprintf(t->nan_dump_prefix, sizeof(t->nan_dump_prefix), "%s", prefix ? prefix : "");
+}
 
 int hip_trainer_nan_flags(const hip_trainer_t* t, uint32_t* out, int max) {
     if (!t || !t->h_nan_flags) return 0;

@@ -89,6 +89,7 @@ def _lib():
         lib.hip_trainer_accumulation_counter.argtypes = [C.c_void_p]
         lib.hip_trainer_enable_nan_check.argtypes = [C.c_void_p, C.c_int]
         lib.hip_trainer_nan_detected.argtypes = [C.c_void_p]
+        lib.hip_trainer_set_nan_dump_prefix.argtypes = [C.c_void_p, C.c_char_p]
         lib.hip_trainer_nan_flags.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
         lib.hip_param_layout.argtypes = [C.POINTER(ModelConfig), C.POINTER(ParamLayout)]
         lib.hip_lora_layout.argtypes = [C.POINTER(ModelConfig), C.POINTER(LoraLayout)]
@@ -194,6 +195,10 @@ class Trainer:
     def enable_nan_check(self, on=True):
         if _lib().hip_trainer_enable_nan_check(self._h, 1 if on else 0) != 0:
             raise SeraphError("could not allocate the NaN flags")
+
+    def set_nan_dump_prefix(self, prefix):
+        """Where a step that detects a NaN/Inf writes its buffers ("<prefix>_<step>_<name>"); None: nowhere."""
+        _lib().hip_trainer_set_nan_dump_prefix(self._h, prefix.encode() if prefix else None)
 
     @property
     def nan_detected(self):

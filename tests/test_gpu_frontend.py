@@ -354,6 +354,62 @@ def test_reference_batched_trainer_profile_and_lora(tmp_path, orc):
     assert os.path.exists(tmp_path / "q" / "checkpoint_final.bin")
 
 
+def test_nan_detection_writes_the_dump_files_the_reference_inspector_reads(tr, orc, tmp_path):
+    """A step that detects a NaN writes the step's buffers as the reference does (src/train.c:5562-5653).  The files are
+    read back with a restatement of what tools/nan_dump_inspect.c does with them (sizes from the token file and the model
+    dimensions, NaN / Inf counts per file) and, where the reference tree was present at build time, by that tool itself."""
+    import json
+    import subprocess
+    shape = dict(hidden=64, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=96, vocab=101)
+    ocfg, cfg = orc.make_config(**shape), tr.model_config(**shape)
+    p = init_params(orc, ocfg, 61)
+    T = 40
+    tok = np.random.default_rng(62).integers(0, 101, T).astype(np.int32)
+    L = tr.param_layout(cfg)
+    p[L.layer0 + 0 * L.layer_stride + L.q + 7] = np.nan              # layer 0's query projection: q is the first poisoned buffer
+    t = tr.Trainer(cfg, tr.optim_config(1e-3), max_tokens=T, max_batch=1)
+    t.enable_nan_check()
+    t.set_nan_dump_prefix(str(tmp_path / "seraph_nan_step"))
+    t.upload(tr.PARAMS, p)
+    t.step(tok, None)                                                # step 1: detected at once
+    assert t.nan_detected
+    t.close()
+    prefix = str(tmp_path / "seraph_nan_step_1")
+    meta = dict(line.split("=") for line in open(prefix + "_meta.txt").read().split())
+    assert meta["step"] == "1" and meta["seq"] == str(T) and meta["num_predictions"] == str(T - 1)
+    assert meta["hidden_size"] == "64" and meta["q_dim"] == "128" and meta["kv_dim"] == "64" and meta["vocab_size"] == "101"
+    toks = np.fromfile(prefix + "_tokens.u32", np.uint32)
+    assert (toks == tok.astype(np.uint32)).all()
+    assert (np.fromfile(prefix + "_targets.u32", np.uint32) == tok[1:].astype(np.uint32)).all()
+    seq, npred, h, f, V, qd, kv = T, T - 1, 64, 96, 101, 128, 64
+    items = [("hidden", seq * h, 1), ("hidden_norm", seq * h, 1), ("logits", seq * V, 1), ("grad_logits", npred * V, 1),
+             ("grad_hidden", seq * h, 1), ("grad_tmp_hidden", seq * h, 0), ("grad_x_norm", seq * h, 0), ("grad_ffn", seq * f, 0),
+             ("grad_gate", seq * f, 0), ("grad_up", seq * f, 0), ("L0_layer_in", seq * h, 0), ("L0_x_norm_attn", seq * h, 0),
+             ("L0_post_attn_in", seq * h, 0), ("L0_x_norm_ffn", seq * h, 0), ("L0_ffn_gate", seq * f, 0), ("L0_ffn_up", seq * f, 0),
+             ("L0_silu", seq * f, 0), ("L0_ffn_hidden", seq * f, 0), ("L0_q", seq * qd, 0), ("L0_k", seq * kv, 0), ("L0_v", seq * kv, 0),
+             ("L0_attn_out", seq * qd, 0), ("grad_attn", seq * qd, 0), ("grad_q", seq * qd, 0), ("grad_k", seq * kv, 0), ("grad_v", seq * kv, 0)]
+    nan_in = {}
+    for name, count, _ in items:                                     # tools/nan_dump_inspect.c:189-246
+        data = np.fromfile(f"{prefix}_{name}.f32", np.float32)
+        assert data.size == count, (name, data.size, count)
+        nan_in[name] = int(np.isnan(data).sum())
+    assert nan_in["L0_layer_in"] == 0 and nan_in["L0_x_norm_attn"] == 0 and nan_in["L0_k"] == 0 and nan_in["L0_v"] == 0
+    assert nan_in["L0_q"] == 2 * T                                   # one poisoned output feature per token, spread over its RoPE pair
+    assert nan_in["logits"] > 0 and nan_in["hidden"] > 0
+    inspector = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "_ref", "nan_dump_inspect")
+    if os.path.exists(inspector):
+        (tmp_path / "model").mkdir()
+        json.dump(dict(vocab_size=101, hidden_size=64, num_hidden_layers=2, intermediate_size=96, num_attention_heads=4,
+                       num_key_value_heads=2, head_dim=32, rms_norm_eps=1e-6, rope_theta=10000.0, model_type="llama"),
+                  open(tmp_path / "model" / "config.json", "w"))
+        out = subprocess.run([inspector, "--model-dir", str(tmp_path / "model"), "--prefix", prefix], capture_output=True, text=True)
+        assert out.returncode == 0, out.stderr
+        assert "MISSING" not in out.stderr and "WARN" not in out.stderr and "BAD SIZE" not in out.stderr, out.stderr
+        line = next(l for l in out.stdout.splitlines() if l.startswith("L0_q "))
+        assert f"n={seq * qd}" in line and f"nan={nan_in['L0_q']}" in line
+        assert f"seq={T} hidden=64 inter=96 vocab=101 q_dim=128 kv_dim=64" in out.stdout
+
+
 def test_bench_line_contract():
     """bench.py prints one JSON line with the agreed keys (33M workload, two steps)."""
     import json
