@@ -111,6 +111,17 @@ int seraph_gemm(const float* A, const float* B, float* C, int64_t M, int64_t N, 
 /* Name of the kernel instantiation seraph_gemm launches for this shape with 16-byte aligned
  * operands, as a profiler prints it (no reference counterpart; used to label timings). */
 const char* seraph_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int transpose_A, int transpose_B);
+/* Several products with the same K, orientations and accumulate flag in ONE launch: the q / k / v (or gate / up)
+ * projections of a layer, which the reference issues back to back (src/train.c:4676-4681, :4718-4725), and their weight
+ * gradients (:5143-5160, :5276-5300).  The tiles of all products form one grid, so products that are too small to
+ * fill the chip share it.  At most 4 products; each is computed as seraph_gemm would (same tile kernel, chosen
+ * for the group as a whole; a group that cannot share a launch is run as single seraph_gemm calls).  `problems`
+ * is a HOST array.  The outputs must not overlap. */
+typedef struct { const float* A; const float* B; float* C; int64_t M, N; } seraph_gemm_problem_t;
+int seraph_gemm_grouped(const seraph_gemm_problem_t* problems, int count, int64_t K,
+                        int transpose_A, int transpose_B, int accumulate, seraph_stream_t s);
+const char* seraph_gemm_grouped_kernel_name(const seraph_gemm_problem_t* problems, int count, int64_t K,
+                                            int transpose_A, int transpose_B);
 /* C (+)= alpha * op(A) op(B): the step "product, then vulkan_scale of the product" of the LoRA path
  * (src/train.c:5778-5796, :5803-5845) as one call.  With the scratch of seraph_gemm_scaled_ws_bytes a small
  * output with a long K is cut into runs of K that separate workgroups take and a second kernel adds in run

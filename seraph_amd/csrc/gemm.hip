@@ -271,19 +271,15 @@ struct FastLoader {
     }
 };
 
+// pid: the workgroup's tile number within this product (0 .. nbm * nbn - 1), already regrouped per XCD
 template <int TM, int TN, bool A_KC, bool B_KC>
-__global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_kernel(const float* __restrict__ A,
-                                                                               const float* __restrict__ B,
-                                                                               float* __restrict__ C,
-                                                                               int64_t M, int64_t N, int64_t K,
-                                                                               int accumulate, int nbm, int nbn) {
+__device__ __forceinline__ void pipelined_body(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
+                                               int64_t M, int64_t N, int64_t K, int accumulate, int nbm, int nbn, int pid) {
     constexpr int BM = 64 * TM, BN = 64 * TN;
     constexpr int A_FLOATS = lds_floats<BM, A_KC>(), B_FLOATS = lds_floats<BN, B_KC>();
     __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
     __shared__ __attribute__((aligned(16))) float lds_b[2][B_FLOATS];
 
-    const int total = nbm * nbn;
-    const int pid = xcd_regroup(blockIdx.x, total);
     const int width = kGroupM * nbn;
     const int group = pid / width;
     const int first_m = group * kGroupM;
@@ -460,6 +456,36 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_kerne
         }
 }
 
+template <int TM, int TN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_kernel(const float* __restrict__ A,
+                                                                               const float* __restrict__ B,
+                                                                               float* __restrict__ C,
+                                                                               int64_t M, int64_t N, int64_t K,
+                                                                               int accumulate, int nbm, int nbn) {
+    pipelined_body<TM, TN, A_KC, B_KC>(A, B, C, M, N, K, accumulate, nbm, nbn, xcd_regroup(blockIdx.x, nbm * nbn));
+}
+
+// Several products with the same K, operand orientations and accumulate flag in one launch (the q / k / v and the
+// gate / up projections of a layer and their weight gradients): the tiles of all of them form one grid, so a product
+// too small to fill the chip shares it with its siblings, and operands that siblings have in common (the layer input
+// forward, the activations in the weight gradients) are fetched into each L2 once.  Every tile is computed exactly as
+// the single-product kernel computes it.
+constexpr int kMaxGroup = 4;
+struct GemmGroup {
+    const float* A[kMaxGroup]; const float* B[kMaxGroup]; float* C[kMaxGroup];
+    int64_t M[kMaxGroup], N[kMaxGroup];
+    int nbm[kMaxGroup], nbn[kMaxGroup], first[kMaxGroup + 1];      // first[i]: the product's first tile in the launch
+    int count;
+};
+
+template <int TM, int TN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_grouped_kernel(const GemmGroup g, int64_t K, int accumulate) {
+    const int pid = xcd_regroup(blockIdx.x, g.first[g.count]);
+    int i = 0;
+    while (i + 1 < g.count && pid >= g.first[i + 1]) i++;          // uniform
+    pipelined_body<TM, TN, A_KC, B_KC>(g.A[i], g.B[i], g.C[i], g.M[i], g.N[i], K, accumulate, g.nbm[i], g.nbn[i], pid - g.first[i]);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Small outputs with a long K (weight gradients of narrow layers, the rank-sized LoRA products):
 // too few 64x64 tiles to occupy the chip.  Here a workgroup owns a 32x32 tile of C and its four
@@ -469,19 +495,15 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_kerne
 // With `slices` > 1 the grid's y index also cuts K into that many equal runs of stages; a workgroup then
 // stores its tile of run y, unscaled, into part[y] (M x N each) and gemm_slices_sum_kernel adds the runs.
 template <bool A_KC, bool B_KC>
-__global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_kernel(const float* __restrict__ A,
-                                                                               const float* __restrict__ B,
-                                                                               float* __restrict__ C,
-                                                                               int64_t M, int64_t N, int64_t K,
-                                                                               int accumulate, int nbm, int nbn,
-                                                                               int slices, float* __restrict__ part) {
+__device__ __forceinline__ void splitk_body(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
+                                            int64_t M, int64_t N, int64_t K, int accumulate, int nbn, int tile,
+                                            int slices, float* __restrict__ part) {
     constexpr int BT = 32;
     constexpr int A_FLOATS = lds_floats<BT, A_KC>(), B_FLOATS = lds_floats<BT, B_KC>();
     __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
     __shared__ __attribute__((aligned(16))) float lds_b[2][B_FLOATS];
     __shared__ __attribute__((aligned(16))) float red[4][BT * BT];
-    (void)nbm;
-    const int pm = blockIdx.x / nbn, pn = blockIdx.x % nbn;
+    const int pm = tile / nbn, pn = tile % nbn;
     const int64_t m0 = (int64_t)pm * BT, n0 = (int64_t)pn * BT;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
@@ -577,6 +599,26 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_kernel(c
             }
         }
     }
+}
+
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_kernel(const float* __restrict__ A,
+                                                                               const float* __restrict__ B,
+                                                                               float* __restrict__ C,
+                                                                               int64_t M, int64_t N, int64_t K,
+                                                                               int accumulate, int nbm, int nbn,
+                                                                               int slices, float* __restrict__ part) {
+    (void)nbm;
+    splitk_body<A_KC, B_KC>(A, B, C, M, N, K, accumulate, nbn, (int)blockIdx.x, slices, part);
+}
+
+// the grouped form of the above (one run of K, no slices); nbm / nbn / first count 32 x 32 tiles here
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_grouped_kernel(const GemmGroup g, int64_t K, int accumulate) {
+    const int tile = (int)blockIdx.x;
+    int i = 0;
+    while (i + 1 < g.count && tile >= g.first[i + 1]) i++;
+    splitk_body<A_KC, B_KC>(g.A[i], g.B[i], g.C[i], g.M[i], g.N[i], K, accumulate, g.nbn[i], tile - g.first[i], 1, nullptr);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -755,6 +797,81 @@ extern "C" int seraph_gemm(const float* A, const float* B, float* C, int64_t M, 
         return SERAPH_OK;
     }
     return launch_gemm<1, 1>(A, B, C, M, N, K, transpose_A, transpose_B, accumulate, vec, st);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Several products in one launch.  0: not groupable (a product that needs the general kernel), else the tile edge
+// the group runs with: 128 or 64 (pipelined kernel) or 32 (the kernel whose waves split K).
+static int group_tile(const seraph_gemm_problem_t* p, int count, int64_t K, int tA, int tB) {
+    if (count < 2 || count > kMaxGroup) return 0;
+    int64_t t128 = 0, t64 = 0, t32 = 0;
+    for (int i = 0; i < count; i++) {
+        const int64_t M = p[i].M, N = p[i].N, lda = tA ? M : K, ldb = tB ? K : N;
+        if (M <= 0 || N <= 0 || !p[i].A || !p[i].B || !p[i].C) return 0;
+        if (lda % 4 || ldb % 4 || !aligned16(p[i].A) || !aligned16(p[i].B) || !pipelined_ok(M, N, K, tA, tB)) return 0;
+        if (use_smallk(p[i].A, p[i].B, p[i].C, M, N, K, tA, tB)) return 0;
+        t128 += ceil_div(M, 128) * ceil_div(N, 128);
+        t64 += ceil_div(M, 64) * ceil_div(N, 64);
+        t32 += ceil_div(M, 32) * ceil_div(N, 32);
+    }
+    if (t32 > 0x7fffffff) return 0;
+    if (t128 >= num_compute_units()) return 128;
+    if (t64 >= num_compute_units() || K < 256) return 64;
+    return 32;
+}
+
+extern "C" const char* seraph_gemm_grouped_kernel_name(const seraph_gemm_problem_t* problems, int count, int64_t K,
+                                                       int transpose_A, int transpose_B) {
+    static const char* names[3][4] = {
+        {"seraph::gemm_f32_mfma_pipelined_grouped_kernel<2, 2, true, false>", "seraph::gemm_f32_mfma_pipelined_grouped_kernel<2, 2, true, true>",
+         "seraph::gemm_f32_mfma_pipelined_grouped_kernel<2, 2, false, false>", "seraph::gemm_f32_mfma_pipelined_grouped_kernel<2, 2, false, true>"},
+        {"seraph::gemm_f32_mfma_pipelined_grouped_kernel<1, 1, true, false>", "seraph::gemm_f32_mfma_pipelined_grouped_kernel<1, 1, true, true>",
+         "seraph::gemm_f32_mfma_pipelined_grouped_kernel<1, 1, false, false>", "seraph::gemm_f32_mfma_pipelined_grouped_kernel<1, 1, false, true>"},
+        {"seraph::gemm_f32_mfma_splitk_grouped_kernel<true, false>", "seraph::gemm_f32_mfma_splitk_grouped_kernel<true, true>",
+         "seraph::gemm_f32_mfma_splitk_grouped_kernel<false, false>", "seraph::gemm_f32_mfma_splitk_grouped_kernel<false, true>"}};
+    const int tile = problems ? group_tile(problems, count, K, transpose_A, transpose_B) : 0;
+    if (!tile) return "gemm (group run as single products)";
+    return names[tile == 128 ? 0 : tile == 64 ? 1 : 2][(transpose_A ? 2 : 0) + (transpose_B ? 1 : 0)];
+}
+
+extern "C" int seraph_gemm_grouped(const seraph_gemm_problem_t* problems, int count, int64_t K,
+                                   int transpose_A, int transpose_B, int accumulate, seraph_stream_t s) {
+    if (count <= 0) return SERAPH_OK;
+    SERAPH_REQUIRE(problems, "gemm_grouped: NULL problem list");
+    const int tile = group_tile(problems, count, K, transpose_A, transpose_B);
+    if (!tile) {                                            // one launch each, exactly as seraph_gemm
+        for (int i = 0; i < count; i++) {
+            int rc = seraph_gemm(problems[i].A, problems[i].B, problems[i].C, problems[i].M, problems[i].N, K, transpose_A, transpose_B, accumulate, s);
+            if (rc != SERAPH_OK) return rc;
+        }
+        return SERAPH_OK;
+    }
+    GemmGroup g;
+    g.count = count;
+    int total = 0;
+    for (int i = 0; i < count; i++) {
+        g.A[i] = problems[i].A; g.B[i] = problems[i].B; g.C[i] = problems[i].C; g.M[i] = problems[i].M; g.N[i] = problems[i].N;
+        g.nbm[i] = (int)ceil_div(problems[i].M, tile); g.nbn[i] = (int)ceil_div(problems[i].N, tile);
+        g.first[i] = total;
+        total += g.nbm[i] * g.nbn[i];
+    }
+    for (int i = count; i <= kMaxGroup; i++) g.first[i] = total;
+    hipStream_t st = as_stream(s);
+    const dim3 grid((unsigned)total), block(kGemmThreads);
+    const int form = (transpose_A ? 2 : 0) + (transpose_B ? 1 : 0);
+#define GOG(KERNEL, ...) \
+    switch (form) { \
+        case 0: hipLaunchKernelGGL((KERNEL<__VA_ARGS__ true, false>), grid, block, 0, st, g, K, accumulate); break; \
+        case 1: hipLaunchKernelGGL((KERNEL<__VA_ARGS__ true, true>), grid, block, 0, st, g, K, accumulate); break; \
+        case 2: hipLaunchKernelGGL((KERNEL<__VA_ARGS__ false, false>), grid, block, 0, st, g, K, accumulate); break; \
+        default: hipLaunchKernelGGL((KERNEL<__VA_ARGS__ false, true>), grid, block, 0, st, g, K, accumulate); break; \
+    }
+    if (tile == 128) { GOG(gemm_f32_mfma_pipelined_grouped_kernel, 2, 2,) }
+    else if (tile == 64) { GOG(gemm_f32_mfma_pipelined_grouped_kernel, 1, 1,) }
+    else { GOG(gemm_f32_mfma_splitk_grouped_kernel,) }
+#undef GOG
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
 }
 
 // ---------------------------------------------------------------------------------------------

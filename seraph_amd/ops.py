@@ -92,6 +92,18 @@ def gemm(A, B, M, N, K, tA=0, tB=0, out=None, accumulate=False):
     return out
 
 
+class GemmProblem(C.Structure):
+    _fields_ = [("A", C.c_void_p), ("B", C.c_void_p), ("C", C.c_void_p), ("M", C.c_int64), ("N", C.c_int64)]
+
+
+def gemm_grouped(problems, K, tA=0, tB=0, accumulate=False):
+    """problems: list of (A, B, out, M, N) sharing K, the orientations and the accumulate flag; one launch."""
+    arr = (GemmProblem * len(problems))(*[GemmProblem(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, n) for a, b, c, m, n in problems])
+    check(kernels().seraph_gemm_grouped(arr, C.c_int(len(problems)), i64(K), C.c_int(tA), C.c_int(tB),
+                                        C.c_int(1 if accumulate else 0), _stream()), "gemm_grouped")
+    return [c for _, _, c, _, _ in problems]
+
+
 def gemm_scaled(A, B, M, N, K, tA=0, tB=0, out=None, accumulate=False, alpha=1.0, scratch=True):
     """out (+)= alpha * op(A) op(B); with scratch, small outputs with a long K are computed in runs of K."""
     if out is None:

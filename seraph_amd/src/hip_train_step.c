@@ -140,6 +140,15 @@ static void op_fold(hip_trainer_t* t) {
     OP(seraph_gemm_kernel_name((M_), (N_), (K_), (tA_), (tB_)), 2.0 * (double)(M_) * (double)(N_) * (double)(K_), 0.0, \
        seraph_gemm_scaled((A_), (B_), (C_), (M_), (N_), (K_), (tA_), (tB_), (acc_), 1.0f, t->ws, t->ws_bytes, t->stream))
 
+/* several products sharing K, orientations and the accumulate flag in one launch (q / k / v, gate / up) */
+#define GEMM_GROUP(probs_, count_, K_, tA_, tB_, acc_)                                                 \
+    do {                                                                                               \
+        double fl_ = 0.0;                                                                              \
+        for (int gi_ = 0; gi_ < (count_); gi_++) fl_ += 2.0 * (double)(probs_)[gi_].M * (double)(probs_)[gi_].N * (double)(K_); \
+        OP(seraph_gemm_grouped_kernel_name((probs_), (count_), (K_), (tA_), (tB_)), fl_, 0.0,          \
+           seraph_gemm_grouped((probs_), (count_), (K_), (tA_), (tB_), (acc_), t->stream));            \
+    } while (0)
+
 /* C (+)= alpha * product; K cut into runs through the trainer's scratch when the shape gains from it */
 #define GEMM_SCALED(A_, B_, C_, M_, N_, K_, tA_, tB_, acc_, alpha_)                                    \
     OP("gemm_scaled", 2.0 * (double)(M_) * (double)(N_) * (double)(K_), 0.0,                           \
@@ -636,11 +645,13 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         float* next = (l + 1 < NL) ? t->act[l + 1].layer_in : t->final_in;
         /* the input norm of every layer but the first comes out of the add that ended the previous layer */
         if (l == 0) OP("rmsnorm", 0.0, 8.0 * (double)(T * h), seraph_rmsnorm(a->layer_in, W + t->L.in_norm, a->xn_attn, T, h, eps, s));
-        GEMM(a->xn_attn, W + t->L.q, a->q, T, qd, h, 0, 1, 0);
+        {   /* the three projections of the same input (src/train.c:4676-4681) as one launch */
+            const seraph_gemm_problem_t qkv[3] = {{a->xn_attn, W + t->L.q, a->q, T, qd}, {a->xn_attn, W + t->L.k, a->k, T, kv},
+                                                  {a->xn_attn, W + t->L.v, a->v, T, kv}};
+            GEMM_GROUP(qkv, 3, h, 0, 1, 0);
+        }
         if (lora && t->LL.A[0] >= 0 && lora_forward_add(t, a->xn_attn, a->q, LW + t->LL.A[0], LW + t->LL.B[0], T, h, qd)) return -1.0f;
-        GEMM(a->xn_attn, W + t->L.k, a->k, T, kv, h, 0, 1, 0);
         if (lora && t->LL.A[1] >= 0 && lora_forward_add(t, a->xn_attn, a->k, LW + t->LL.A[1], LW + t->LL.B[1], T, h, kv)) return -1.0f;
-        GEMM(a->xn_attn, W + t->L.v, a->v, T, kv, h, 0, 1, 0);
         if (lora && t->LL.A[2] >= 0 && lora_forward_add(t, a->xn_attn, a->v, LW + t->LL.A[2], LW + t->LL.B[2], T, h, kv)) return -1.0f;
         OP("rope", 0.0, 8.0 * (double)(T * (qd + kv)), seraph_rope_qk(a->q, a->q, H, a->k, a->k, KVH, starts, batch, T, D, theta, 0, s));
         if (c->use_qk_norm) {                                              /* after RoPE, before the attention: src/train.c:4687-4689 */
@@ -651,9 +662,11 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         GEMM(a->attn_out, W + t->L.o, t->tmp_h, T, h, qd, 0, 1, 0);
         if (lora && t->LL.A[3] >= 0 && lora_forward_add(t, a->attn_out, t->tmp_h, LW + t->LL.A[3], LW + t->LL.B[3], T, qd, h)) return -1.0f;
         OP("add_rmsnorm", 0.0, 16.0 * (double)(T * h), seraph_add_rmsnorm(a->layer_in, t->tmp_h, a->post_in, W + t->L.post_norm, a->xn_ffn, T, h, eps, s));
-        GEMM(a->xn_ffn, W + t->L.gate, a->gate, T, f, h, 0, 1, 0);
+        {   /* gate and up projections (src/train.c:4718-4725) as one launch */
+            const seraph_gemm_problem_t gu[2] = {{a->xn_ffn, W + t->L.gate, a->gate, T, f}, {a->xn_ffn, W + t->L.up, a->up, T, f}};
+            GEMM_GROUP(gu, 2, h, 0, 1, 0);
+        }
         if (lora && t->LL.A[4] >= 0 && lora_forward_add(t, a->xn_ffn, a->gate, LW + t->LL.A[4], LW + t->LL.B[4], T, h, f)) return -1.0f;
-        GEMM(a->xn_ffn, W + t->L.up, a->up, T, f, h, 0, 1, 0);
         if (lora && t->LL.A[5] >= 0 && lora_forward_add(t, a->xn_ffn, a->up, LW + t->LL.A[5], LW + t->LL.B[5], T, h, f)) return -1.0f;
         OP("swiglu", 0.0, 12.0 * (double)(T * f), seraph_swiglu(a->gate, a->up, a->ffn_h, (size_t)(T * f), s));
         GEMM(a->ffn_h, W + t->L.down, t->tmp_h, T, h, f, 0, 1, 0);
@@ -717,8 +730,8 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         if (lora && t->LL.A[5] >= 0 &&
             lora_backward(t, t->g_up, a->xn_ffn, LW + t->LL.A[5], LW + t->LL.B[5], LGW + t->LL.A[5], LGW + t->LL.B[5], T, h, f)) return -1.0f;
         if (!lora) {
-            GEMM(t->g_gate, a->xn_ffn, GW + t->L.gate, f, h, T, 1, 0, 1);
-            GEMM(t->g_up, a->xn_ffn, GW + t->L.up, f, h, T, 1, 0, 1);
+            const seraph_gemm_problem_t gu[2] = {{t->g_gate, a->xn_ffn, GW + t->L.gate, f, h}, {t->g_up, a->xn_ffn, GW + t->L.up, f, h}};
+            GEMM_GROUP(gu, 2, T, 1, 0, 1);
         }
         GEMM(t->g_gate, W + t->L.gate, t->g_xn, T, h, f, 0, 0, 0);
         GEMM(t->g_up, W + t->L.up, t->g_xn, T, h, f, 0, 0, 1);
@@ -746,9 +759,9 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         OP("rope", 0.0, 8.0 * (double)(T * (qd + kv)), seraph_rope_qk(t->g_q, t->g_q, H, t->g_k, t->g_k, KVH, starts, batch, T, D, theta, 1, s));
         NANCHK(t->g_q, T * qd, nan_bwd + 5u * (uint32_t)l + 4u);
         if (!lora) {
-            GEMM(t->g_q, a->xn_attn, GW + t->L.q, qd, h, T, 1, 0, 1);
-            GEMM(t->g_k, a->xn_attn, GW + t->L.k, kv, h, T, 1, 0, 1);
-            GEMM(t->g_v, a->xn_attn, GW + t->L.v, kv, h, T, 1, 0, 1);
+            const seraph_gemm_problem_t qkv[3] = {{t->g_q, a->xn_attn, GW + t->L.q, qd, h}, {t->g_k, a->xn_attn, GW + t->L.k, kv, h},
+                                                  {t->g_v, a->xn_attn, GW + t->L.v, kv, h}};
+            GEMM_GROUP(qkv, 3, T, 1, 0, 1);
         } else {
             float* gs[3] = {t->g_q, t->g_k, t->g_v};
             int64_t outs[3] = {qd, kv, kv};
