@@ -148,7 +148,7 @@ def gemm_table(w):
     print(f"GEMM time per step: this library {tot[0]:.1f} ms, hipBLASLt {tot[1]:.1f} ms")
 
 
-def run_workload(w, key, steps, warmup, op_timing=True, pmc_calibration=False):
+def run_workload(w, key, steps, warmup, op_timing=True, pmc_calibration=False, wgrad_overlap=True):
     """`warmup` untimed steps, then `steps` timed ones of workload `w`; returns the fields of the bench line."""
     import torch
     from seraph_amd import trainer as tr
@@ -172,6 +172,8 @@ def run_workload(w, key, steps, warmup, op_timing=True, pmc_calibration=False):
                torch.zeros(n, dtype=torch.float32, device=dev))
     torch.cuda.synchronize()
     t = tr.Trainer(cfg, opt, max_tokens=T, max_batch=w["batch"], device=0, ext=ext)
+    if not wgrad_overlap:
+        t.enable_wgrad_overlap(False)                     # else the trainer's own choice by step size
     if w["lora"]:
         nl = tr.lora_param_count(cfg)
         lo = (0.01 * np.random.default_rng(5).standard_normal(nl)).astype(np.float32)     # A ~ N(0, 0.01)
@@ -472,6 +474,8 @@ def main():
                     help="do not bracket every kernel-library call with an event pair (no roofline / kernels objects)")
     ap.add_argument("--headline-only", action="store_true",
                     help="only the headline workload: no other workloads, isolated ops or drop-in path in the line")
+    ap.add_argument("--one-stream", action="store_true",
+                    help="keep the weight gradients on the step's one stream (default: on a second stream beside the chain)")
     ap.add_argument("--gemm-table", action="store_true",
                     help="instead of the benchmark, time every GEMM shape of the workload's step beside hipBLASLt")
     args = ap.parse_args()
@@ -483,7 +487,7 @@ def main():
                  "(value is the one GPU's throughput)")
 
     w = WORKLOADS[args.workload]
-    head = run_workload(w, args.workload, args.steps, args.warmup, op_timing=not args.no_op_timing,
+    head = run_workload(w, args.workload, args.steps, args.warmup, op_timing=not args.no_op_timing, wgrad_overlap=not args.one_stream,
                         pmc_calibration=args.pmc_calibration)
     out = {
         "metric": "train tok/s (fwd+bwd+AdamW)", "value": head["value"], "unit": "tok/s",
@@ -498,7 +502,7 @@ def main():
         # configurations alone, and the unmodified reference step driver over the vulkan_* symbols
         others = {}
         for key, steps, warmup in (("c1", 30, 5), ("c4", 8, 2)):
-            r = run_workload(WORKLOADS[key], key, steps, warmup, op_timing=not args.no_op_timing)
+            r = run_workload(WORKLOADS[key], key, steps, warmup, op_timing=not args.no_op_timing, wgrad_overlap=not args.one_stream)
             others[key] = {k: r[k] for k in ("value", "unit", "ms_per_step", "steps", "warmup", "config", "loss_first_last", "roofline")}
             top = sorted(r["kernels"].items(), key=lambda kv: -kv[1]["share"])[:6]
             others[key]["kernels"] = dict(top)

@@ -155,6 +155,11 @@ typedef struct {
     double      bytes;     /* summed algorithmic bytes (0 for matrix-core classes)     */
 } hip_op_stat_t;
 void hip_trainer_enable_op_timing(hip_trainer_t* t, int on);
+/* Full-weight steps run the weight-gradient products on a second stream beside the chain of input gradients (on by
+ * default where max_tokens * hidden <= 2^22, off above, where each product fills the chip by itself; results are the
+ * same either way, each product being one kernel whichever stream carries it). Per-op timing
+ * and the NaN lattice keep the step on one stream. No counterpart in the reference, whose steps are one stream. */
+void hip_trainer_enable_wgrad_overlap(hip_trainer_t* t, int on);
 void hip_trainer_reset_op_stats(hip_trainer_t* t);
 int  hip_trainer_op_stats(const hip_trainer_t* t, hip_op_stat_t* out, int max);
 

@@ -74,6 +74,9 @@ int  seraph_hip_event_create(void** out);
 int  seraph_hip_event_destroy(void* ev);
 int  seraph_hip_event_record(void* ev, seraph_stream_t s);
 int  seraph_hip_event_elapsed_ms(void* start, void* stop, float* ms);  /* waits for stop */
+/* work submitted to `s` after this call starts only when everything recorded into `ev` has completed (two streams of
+ * one step: weight gradients beside the chain of input gradients) */
+int  seraph_hip_stream_wait_event(seraph_stream_t s, void* ev);
 
 /* ---------------------------------------------------------------- utility ops */
 /* vulkan_fill_buffer / vulkan_fill_buffer_range, include/vulkan_backend.h:411-415,525-528 */
@@ -167,6 +170,19 @@ int seraph_attention_backward_banded(const float* Q, const float* K, const float
                                      float* dQ, float* dK, float* dV,
                                      const uint32_t* seq_starts, int batch, int64_t T,
                                      int heads, int kv_heads, int head_dim, float scale, int64_t max_seq_len,
+                                     void* ws, size_t ws_bytes, seraph_stream_t s);
+
+/* The form a step driver wants: dK and dV are ASSIGNED (no zero fill before the call; their old contents are not read),
+ * and the longest sequence comes from host_seq_starts, the host's copy of the batch + 1 offsets that seq_starts holds on
+ * the device (NULL with seq_starts NULL: one sequence of T).  The dS band is then sized by a bound that cannot fail:
+ * scratch of seraph_attention_backward_ws_bytes_banded(T, ..., longest sequence) bytes selects the 5-product path, with no
+ * stand-by launch.  Offsets that do not run from 0 to T without decreasing are an error.  Otherwise as
+ * seraph_attention_backward_banded; results are bit-identical to it on zeroed dK / dV. */
+int seraph_attention_backward_assign(const float* Q, const float* K, const float* V, const float* dO,
+                                     const float* attn_out, const float* lse,
+                                     float* dQ, float* dK, float* dV,
+                                     const uint32_t* seq_starts, const uint32_t* host_seq_starts, int batch, int64_t T,
+                                     int heads, int kv_heads, int head_dim, float scale,
                                      void* ws, size_t ws_bytes, seraph_stream_t s);
 
 /* ---------------------------------------------------------------- norm / position */

@@ -452,7 +452,8 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
                                                                     int64_t T, int H, int KVH, float scale, float scale_log2e,
                                                                     unsigned int* __restrict__ queue,
                                                                     float* __restrict__ DS, int ds_slots,
-                                                                    int split, float* __restrict__ partK, float* __restrict__ partV) {
+                                                                    int split, float* __restrict__ partK, float* __restrict__ partV,
+                                                                    int assign) {
     constexpr int LD = D + 4, DB = D / 32;
     // Query rows per iteration: two 32-row sub-tiles up to head_dim 64, so that one staging phase and
     // one barrier serve 256 matrix instructions per wave, as one 32-row tile does at head_dim 128.
@@ -1023,6 +1024,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
         }
     }
     const bool rmw = split <= 1;                               // else: plain store into this item's slice
+    const bool add_old = rmw && !assign;                       // assign: dK/dV are this call's result alone
     float* outK = rmw ? dK : partK + (int64_t)sub * T * kw;
     float* outV = rmw ? dV : partV + (int64_t)sub * T * kw;
 
@@ -1035,7 +1037,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
             const int64_t j = jw0 + acc_row(v, h);
 #pragma unroll
             for (int db = 0; db < DB; db++) { oldk[v].v[db] = 0.f; oldv[v].v[db] = 0.f; }
-            if (rmw && j < T) {
+            if (add_old && j < T) {
                 oldk[v] = lds_dvec<DB>(outK + j * kw + kvh * D, r);
                 oldv[v] = lds_dvec<DB>(outV + j * kw + kvh * D, r);
             }
@@ -1065,12 +1067,13 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
     tq_.leave();
 }
 
-// dK += sum of the split items' slices, in slice order (likewise dV)
+// dK += sum of the split items' slices, in slice order (likewise dV); with `assign` the sum starts from zero
 __global__ __launch_bounds__(256) void attn_split_reduce_kernel(float* __restrict__ dK, float* __restrict__ dV,
                                                                 const float* __restrict__ partK, const float* __restrict__ partV,
-                                                                int64_t n4, int split) {
+                                                                int64_t n4, int split, int assign) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
-        float4 a = reinterpret_cast<float4*>(dK)[i], b = reinterpret_cast<float4*>(dV)[i];
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+        if (!assign) { a = reinterpret_cast<float4*>(dK)[i]; b = reinterpret_cast<float4*>(dV)[i]; }
         for (int p = 0; p < split; p++) {
             const float4 x = reinterpret_cast<const float4*>(partK)[p * n4 + i], y = reinterpret_cast<const float4*>(partV)[p * n4 + i];
             a.x += x.x; a.y += x.y; a.z += x.z; a.w += x.w;
@@ -1429,7 +1432,7 @@ template <int D>
 static int run_backward(const float* Q, const float* K, const float* V, const float* dO, const float* O, const float* lse,
                         float* delta, int* row_start, int* overflow, float* dQ, float* dK, float* dV, const uint32_t* seq_starts, int batch,
                         int64_t T, int H, int KVH, float scale, int64_t longest_seq, float* ds, int ds_slots, float* partK, float* partV,
-                        hipStream_t st) {
+                        bool assign, bool bound_verified, hipStream_t st) {
     unsigned int *qkv = nullptr, *qq = nullptr;
     int rc = acquire_tile_queue(&qkv);
     if (rc == SERAPH_OK) rc = acquire_tile_queue(&qq);
@@ -1438,7 +1441,7 @@ static int run_backward(const float* Q, const float* K, const float* V, const fl
     // launch number that the scratch cannot hold by accident marks "this launch overflowed its band".
     static std::atomic<int> launch_counter{0};
     const int epoch = (launch_counter.fetch_add(1) & 0x3fffffff) + 1;
-    const bool bound_can_fail = ds && (int64_t)ds_slots < ceil_div(T, 32) + 1;
+    const bool bound_can_fail = ds && !bound_verified && (int64_t)ds_slots < ceil_div(T, 32) + 1;
     hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)ceil_div(T, 4)), dim3(256), 0, st, dO, O, delta, T, H, seq_starts, batch, row_start,
                        ds ? ds_slots : 0, epoch, overflow, qkv, qq);
     SERAPH_LAUNCH_CHECK();
@@ -1457,15 +1460,15 @@ static int run_backward(const float* Q, const float* K, const float* V, const fl
     dim3 gkv(persistent_grid(kv_items * split, kv_per_cu)), gq(persistent_grid(ceil_div(T, 128) * H, per_cu));
     if (ds)
         hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, true>), gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, row_start, dK, dV, seq_starts, batch,
-                           T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots, split, partK, partV);
+                           T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots, split, partK, partV, assign ? 1 : 0);
     else
         hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, false>), gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, row_start, dK, dV, seq_starts, batch,
-                           T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots, split, partK, partV);
+                           T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots, split, partK, partV, assign ? 1 : 0);
     if (split > 1) {
         SERAPH_LAUNCH_CHECK();
         const int64_t n4 = T * KVH * D / 4;
         hipLaunchKernelGGL(attn_split_reduce_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(n4, 256), 4096)), dim3(256), 0, st,
-                           dK, dV, partK, partV, n4, split);
+                           dK, dV, partK, partV, n4, split, assign ? 1 : 0);
     }
     SERAPH_LAUNCH_CHECK();
     if (ds) {
@@ -1536,12 +1539,54 @@ int seraph_attention_backward(const float* Q, const float* K, const float* V, co
                                             head_dim, scale, T, ws, ws_bytes, s);
 }
 
+static int attention_backward_any(const float* Q, const float* K, const float* V, const float* dO,
+                                  const float* attn_out, const float* lse,
+                                  float* dQ, float* dK, float* dV,
+                                  const uint32_t* seq_starts, int batch, int64_t T,
+                                  int heads, int kv_heads, int head_dim, float scale, int64_t max_seq_len,
+                                  bool assign, bool bound_verified,
+                                  void* ws, size_t ws_bytes, seraph_stream_t s);
+
 int seraph_attention_backward_banded(const float* Q, const float* K, const float* V, const float* dO,
                                      const float* attn_out, const float* lse,
                                      float* dQ, float* dK, float* dV,
                                      const uint32_t* seq_starts, int batch, int64_t T,
                                      int heads, int kv_heads, int head_dim, float scale, int64_t max_seq_len,
                                      void* ws, size_t ws_bytes, seraph_stream_t s) {
+    return attention_backward_any(Q, K, V, dO, attn_out, lse, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, head_dim, scale,
+                                  max_seq_len, false, false, ws, ws_bytes, s);
+}
+
+int seraph_attention_backward_assign(const float* Q, const float* K, const float* V, const float* dO,
+                                     const float* attn_out, const float* lse,
+                                     float* dQ, float* dK, float* dV,
+                                     const uint32_t* seq_starts, const uint32_t* host_seq_starts, int batch, int64_t T,
+                                     int heads, int kv_heads, int head_dim, float scale,
+                                     void* ws, size_t ws_bytes, seraph_stream_t s) {
+    // The host's copy of the offsets gives the exact longest sequence, so the dS band is sized by a bound that
+    // cannot fail and the launch that stands by for a failed bound is left out.
+    int64_t longest = T;
+    if (seq_starts) {
+        SERAPH_REQUIRE(host_seq_starts && batch >= 1, "attention_backward_assign: packed call needs the host copy of seq_starts");
+        SERAPH_REQUIRE(host_seq_starts[0] == 0 && (int64_t)host_seq_starts[batch] == T, "attention_backward_assign: seq_starts must run from 0 to T");
+        longest = 1;
+        for (int b = 0; b < batch; b++) {
+            SERAPH_REQUIRE(host_seq_starts[b + 1] >= host_seq_starts[b], "attention_backward_assign: seq_starts must not decrease");
+            const int64_t len = (int64_t)host_seq_starts[b + 1] - host_seq_starts[b];
+            longest = len > longest ? len : longest;
+        }
+    }
+    return attention_backward_any(Q, K, V, dO, attn_out, lse, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, head_dim, scale,
+                                  longest, true, true, ws, ws_bytes, s);
+}
+
+static int attention_backward_any(const float* Q, const float* K, const float* V, const float* dO,
+                                  const float* attn_out, const float* lse,
+                                  float* dQ, float* dK, float* dV,
+                                  const uint32_t* seq_starts, int batch, int64_t T,
+                                  int heads, int kv_heads, int head_dim, float scale, int64_t max_seq_len,
+                                  bool assign, bool bound_verified,
+                                  void* ws, size_t ws_bytes, seraph_stream_t s) {
     if (T == 0) return SERAPH_OK;
     SERAPH_REQUIRE(Q && K && V && dO && dQ && dK && dV, "attention_backward: NULL pointer");
     int rc = check_attn_shape("attention_backward", T, heads, kv_heads, head_dim);
@@ -1574,9 +1619,9 @@ int seraph_attention_backward_banded(const float* Q, const float* K, const float
         O = w.out; L = w.lse;
     }
     switch (head_dim) {
-        case 32: return run_backward<32>(Q, K, V, dO, O, L, w.delta, w.row_start, w.overflow, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, max_seq_len, ds, ds_slots, w.partK, w.partV, st);
-        case 64: return run_backward<64>(Q, K, V, dO, O, L, w.delta, w.row_start, w.overflow, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, max_seq_len, ds, ds_slots, w.partK, w.partV, st);
-        default: return run_backward<128>(Q, K, V, dO, O, L, w.delta, w.row_start, w.overflow, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, max_seq_len, ds, ds_slots, w.partK, w.partV, st);
+        case 32: return run_backward<32>(Q, K, V, dO, O, L, w.delta, w.row_start, w.overflow, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, max_seq_len, ds, ds_slots, w.partK, w.partV, assign, bound_verified, st);
+        case 64: return run_backward<64>(Q, K, V, dO, O, L, w.delta, w.row_start, w.overflow, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, max_seq_len, ds, ds_slots, w.partK, w.partV, assign, bound_verified, st);
+        default: return run_backward<128>(Q, K, V, dO, O, L, w.delta, w.row_start, w.overflow, dQ, dK, dV, seq_starts, batch, T, heads, kv_heads, scale, max_seq_len, ds, ds_slots, w.partK, w.partV, assign, bound_verified, st);
     }
 }
 

@@ -163,6 +163,12 @@ int seraph_hip_event_record(void* ev, seraph_stream_t s) {
     return SERAPH_OK;
 }
 
+int seraph_hip_stream_wait_event(seraph_stream_t s, void* ev) {
+    SERAPH_REQUIRE(ev, "stream_wait_event: NULL event");
+    SERAPH_HIP_CHECK(hipStreamWaitEvent(as_stream(s), reinterpret_cast<hipEvent_t>(ev), 0));
+    return SERAPH_OK;
+}
+
 int seraph_hip_event_elapsed_ms(void* start, void* stop, float* ms) {
     SERAPH_REQUIRE(start && stop && ms, "event_elapsed: NULL argument");
     SERAPH_HIP_CHECK(hipEventSynchronize(reinterpret_cast<hipEvent_t>(stop)));

@@ -151,6 +151,29 @@ def attention_backward(Q, K, V, dO, heads, kv_heads, head_dim, seq_starts=None, 
     return dQ, dK, dV
 
 
+def attention_backward_assign(Q, K, V, dO, heads, kv_heads, head_dim, seq_starts=None, host_starts=None, scale=None,
+                              out=None, lse=None, dQ=None, dK=None, dV=None):
+    """dK / dV assigned (given buffers may hold anything); the dS band sized from the host copy of the offsets."""
+    T = Q.shape[0]
+    dQ = torch.empty_like(Q) if dQ is None else dQ
+    dK = torch.empty_like(K) if dK is None else dK
+    dV = torch.empty_like(V) if dV is None else dV
+    scale = head_dim ** -0.5 if scale is None else scale
+    hs = None
+    longest = T
+    if seq_starts is not None:
+        hs = (C.c_uint32 * len(host_starts))(*[int(x) for x in host_starts])
+        longest = max(1, max(int(host_starts[i + 1]) - int(host_starts[i]) for i in range(len(host_starts) - 1)))
+    nbytes = kernels().seraph_attention_backward_ws_bytes_banded(i64(T), C.c_int(heads), C.c_int(kv_heads),
+                                                                 C.c_int(head_dim), i64(longest))
+    ws = _workspace(nbytes)
+    check(kernels().seraph_attention_backward_assign(_p(Q), _p(K), _p(V), _p(dO), _p(out), _p(lse), _p(dQ), _p(dK), _p(dV),
+                                                     _p(seq_starts), hs, C.c_int(_batch(seq_starts)), i64(T), C.c_int(heads),
+                                                     C.c_int(kv_heads), C.c_int(head_dim), f32(scale), _p(ws), sz(nbytes),
+                                                     _stream()), "attention_backward_assign")
+    return dQ, dK, dV
+
+
 def rmsnorm(x, scale, eps):
     y = torch.empty_like(x)
     check(kernels().seraph_rmsnorm(_p(x), _p(scale), _p(y), i64(x.shape[0]), i64(x.shape[1]), f32(eps), _stream()),

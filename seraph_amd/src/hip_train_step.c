@@ -40,6 +40,14 @@ struct hip_trainer {
     layer_layout_t L;
     lora_layout_t LL;
     seraph_stream_t stream;
+    /* full-weight mode: the weight gradients run on a second stream beside the chain of input gradients, which
+     * alone decides how soon the next kernel of the chain can start; events order the two streams around every
+     * buffer they share */
+    seraph_stream_t stream2;
+    void* side_ev[6];            /* fork | down | gate-up | o | q-k-v | end */
+    void* ws2;                   /* scratch of the products on stream2 */
+    size_t ws2_bytes;
+    int overlap;
     /* arenas */
     float *P, *G, *M, *V;
     int own_P, own_G, own_M, own_V;
@@ -140,6 +148,11 @@ static void op_fold(hip_trainer_t* t) {
     OP(seraph_gemm_kernel_name((M_), (N_), (K_), (tA_), (tB_)), 2.0 * (double)(M_) * (double)(N_) * (double)(K_), 0.0, \
        seraph_gemm_scaled((A_), (B_), (C_), (M_), (N_), (K_), (tA_), (tB_), (acc_), 1.0f, t->ws, t->ws_bytes, t->stream))
 
+/* a weight gradient: on the second stream with its own scratch when the step overlaps them (sw / w2 / w2b of run_step) */
+#define WGEMM(A_, B_, C_, M_, N_, K_)                                                                  \
+    OP(seraph_gemm_kernel_name((M_), (N_), (K_), 1, 0), 2.0 * (double)(M_) * (double)(N_) * (double)(K_), 0.0, \
+       seraph_gemm_scaled((A_), (B_), (C_), (M_), (N_), (K_), 1, 0, 1, 1.0f, w2, w2b, sw))
+
 /* several products sharing K, orientations and the accumulate flag in one launch (q / k / v, gate / up) */
 #define GEMM_GROUP(probs_, count_, K_, tA_, tB_, acc_)                                                 \
     do {                                                                                               \
@@ -148,6 +161,19 @@ static void op_fold(hip_trainer_t* t) {
         OP(seraph_gemm_grouped_kernel_name((probs_), (count_), (K_), (tA_), (tB_)), fl_, 0.0,          \
            seraph_gemm_grouped((probs_), (count_), (K_), (tA_), (tB_), (acc_), t->stream));            \
     } while (0)
+
+#define WGEMM_GROUP(probs_, count_, K_)                                                                \
+    do {                                                                                               \
+        double fl_ = 0.0;                                                                              \
+        for (int gi_ = 0; gi_ < (count_); gi_++) fl_ += 2.0 * (double)(probs_)[gi_].M * (double)(probs_)[gi_].N * (double)(K_); \
+        OP(seraph_gemm_grouped_kernel_name((probs_), (count_), (K_), 1, 0), fl_, 0.0,                  \
+           seraph_gemm_grouped((probs_), (count_), (K_), 1, 0, 1, sw));                                \
+    } while (0)
+
+/* the second stream picks up from this point of the first | marks a point of the second | the first waits for a mark */
+#define SIDE_FORK()  do { if (ov) { CK(seraph_hip_event_record(t->side_ev[0], s)); CK(seraph_hip_stream_wait_event(sw, t->side_ev[0])); } } while (0)
+#define SIDE_MARK(i) do { if (ov) CK(seraph_hip_event_record(t->side_ev[(i)], sw)); } while (0)
+#define SIDE_JOIN(i) do { if (ov) CK(seraph_hip_stream_wait_event(s, t->side_ev[(i)])); } while (0)
 
 /* C (+)= alpha * product; K cut into runs through the trainer's scratch when the shape gains from it */
 #define GEMM_SCALED(A_, B_, C_, M_, N_, K_, tA_, tB_, acc_, alpha_)                                    \
@@ -267,6 +293,14 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
     make_layouts(t);
     if (seraph_hip_stream_create(&t->stream) != SERAPH_OK) goto fail;
     for (int i = 0; i < 4; i++) if (seraph_hip_event_create(&t->ev[i]) != SERAPH_OK) goto fail;
+    if (!t->lora) {
+        if (seraph_hip_stream_create(&t->stream2) != SERAPH_OK) goto fail;
+        for (int i = 0; i < 6; i++) if (seraph_hip_event_create(&t->side_ev[i]) != SERAPH_OK) goto fail;
+        /* Beside a chain of small products the second stream fills CUs that the chain's ramps and tails leave idle
+         * (+3 % at 2048 tokens x 512); beside products that fill the chip by themselves it only interleaves two tile
+         * orders in every L2 (-7 % at 16384 tokens x 2048).  hip_trainer_enable_wgrad_overlap overrides the choice. */
+        t->overlap = (int64_t)max_tokens * cfg->hidden <= ((int64_t)1 << 22);
+    }
 
     const size_t pbytes = (size_t)t->nparams * sizeof(float);
     t->P = ext_params;
@@ -337,11 +371,16 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
                 t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(dims[i], r, Tm, 1, 0));
                 t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(r, dims[i], Tm, 1, 0));
             } else {
-                for (int j = 0; j < 4; j++) t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(dims[i], dims[j], Tm, 1, 0));
+                for (int j = 0; j < 4; j++) {
+                    t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(dims[i], dims[j], Tm, 1, 0));
+                    t->ws2_bytes = max_sz(t->ws2_bytes, seraph_gemm_scaled_ws_bytes(dims[i], dims[j], Tm, 1, 0));
+                }
             }
         }
+        if (r <= 0) t->ws2_bytes = max_sz(t->ws2_bytes, seraph_gemm_scaled_ws_bytes(cfg->vocab, cfg->hidden, Tm, 1, 0));
     }
     if (dev_alloc(t, &t->ws, t->ws_bytes)) goto fail;
+    if (t->stream2 && t->ws2_bytes && dev_alloc(t, &t->ws2, t->ws2_bytes)) goto fail;
     if (seraph_hip_host_alloc((void**)&t->h_stage, ((size_t)2 * max_tokens + max_batch + 1) * 4) != SERAPH_OK) goto fail;
     if (seraph_hip_stream_sync(t->stream) != SERAPH_OK) goto fail;
     return t;
@@ -353,6 +392,7 @@ fail:
 
 void hip_trainer_free(hip_trainer_t* t) {
     if (!t) return;
+    if (t->stream2) seraph_hip_stream_sync(t->stream2);
     if (t->stream) seraph_hip_stream_sync(t->stream);
     if (t->own_P) seraph_hip_free(t->P);
     if (t->own_G) seraph_hip_free(t->G);
@@ -361,6 +401,7 @@ void hip_trainer_free(hip_trainer_t* t) {
     seraph_hip_free(t->LP); seraph_hip_free(t->LG); seraph_hip_free(t->LM); seraph_hip_free(t->LV);
     seraph_hip_free(t->act_arena);
     seraph_hip_free(t->ws);
+    seraph_hip_free(t->ws2);
     seraph_hip_free(t->attn_ws);
     seraph_hip_free(t->d_nan_flags);
     free(t->h_nan_flags);
@@ -370,6 +411,8 @@ void hip_trainer_free(hip_trainer_t* t) {
         for (int i = 0; i < 2 * t->op_ev_made; i++) seraph_hip_event_destroy(t->op_ev[i]);
         free(t->op_ev);
     }
+    for (int i = 0; i < 6; i++) if (t->side_ev[i]) seraph_hip_event_destroy(t->side_ev[i]);
+    if (t->stream2) seraph_hip_stream_destroy(t->stream2);
     seraph_hip_stream_destroy(t->stream);
     free(t->act);
     free(t);
@@ -439,6 +482,8 @@ void hip_trainer_last_timing(const hip_trainer_t* t, float ms[3]) {
 }
 
 void hip_trainer_enable_op_timing(hip_trainer_t* t, int on) { if (t) t->op_timing = on ? 1 : 0; }
+
+void hip_trainer_enable_wgrad_overlap(hip_trainer_t* t, int on) { if (t) t->overlap = (on && t->stream2) ? 1 : 0; }
 void hip_trainer_reset_op_stats(hip_trainer_t* t) { if (t) { t->op_classes = 0; t->op_ev_used = 0; } }
 int hip_trainer_op_stats(const hip_trainer_t* t, hip_op_stat_t* out, int max) {
     if (!t || !out) return 0;
@@ -703,9 +748,19 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
     /* ---------------- backward */
     float* glog = t->logits;
     NANCHK(glog, T * V, 3u);
+    /* Weight gradients leave the chain: each one starts on the second stream once its two operands are complete
+     * (fork), and the first stream waits for it (join) only where it is about to overwrite one of them: g_hidden at
+     * the next norm backward, g_gate / g_up and g_q / g_k / g_v in the next layer down. With per-op timing or the NaN
+     * lattice on, everything stays on one stream. */
+    const int ov = t->overlap && !lora && !t->op_timing && !t->nan_check;
+    seraph_stream_t sw = ov ? t->stream2 : s;
+    void* w2 = ov ? t->ws2 : t->ws;
+    const size_t w2b = ov ? t->ws2_bytes : t->ws_bytes;
+    enum { MK_DOWN = 1, MK_GU = 2, MK_O = 3, MK_QKV = 4, MK_END = 5 };
+    SIDE_FORK();
+    if (!lora) WGEMM(glog, t->xn_final, t->G + t->off_embed, V, h, T);      /* LM head wgrad */
     GEMM(glog, P + t->off_embed, t->g_hidden, T, h, V, 0, 0, 0);            /* LM head dgrad */
     NANCHK(t->g_hidden, T * h, 4u);
-    if (!lora) GEMM(glog, t->xn_final, t->G + t->off_embed, V, h, T, 1, 0, 1); /* LM head wgrad */
     OP("rmsnorm_backward", 0.0, 12.0 * (double)(T * h), seraph_rmsnorm_backward(t->final_in, P + t->off_final_norm, t->g_hidden, t->g_tmp,
                                lora ? t->scratch_gs : t->G + t->off_final_norm, T, h, eps, t->ws, t->ws_bytes, s));
     NANCHK(t->g_tmp, T * h, 5u);
@@ -720,10 +775,13 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         layer_act_t* a = &t->act[l];
 
         /* FFN */
-        if (!lora) GEMM(t->g_hidden, a->ffn_h, GW + t->L.down, h, f, T, 1, 0, 1);
+        SIDE_FORK();
+        if (!lora) WGEMM(t->g_hidden, a->ffn_h, GW + t->L.down, h, f, T);
+        SIDE_MARK(MK_DOWN);
         GEMM(t->g_hidden, W + t->L.down, t->g_ffn, T, f, h, 0, 0, 0);
         if (lora && t->LL.A[6] >= 0 &&                                       /* src/train.c:6422-6429 */
             lora_backward(t, t->g_hidden, a->ffn_h, LW + t->LL.A[6], LW + t->LL.B[6], LGW + t->LL.A[6], LGW + t->LL.B[6], T, f, h)) return -1.0f;
+        SIDE_JOIN(MK_GU);                                                    /* the layer above still reads g_gate / g_up */
         OP("swiglu_backward", 0.0, 20.0 * (double)(T * f), seraph_swiglu_backward(a->gate, a->up, t->g_ffn, t->g_gate, t->g_up, (size_t)(T * f), s));
         if (lora && t->LL.A[4] >= 0 &&                                       /* src/train.c:6446-6461 */
             lora_backward(t, t->g_gate, a->xn_ffn, LW + t->LL.A[4], LW + t->LL.B[4], LGW + t->LL.A[4], LGW + t->LL.B[4], T, h, f)) return -1.0f;
@@ -731,24 +789,30 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
             lora_backward(t, t->g_up, a->xn_ffn, LW + t->LL.A[5], LW + t->LL.B[5], LGW + t->LL.A[5], LGW + t->LL.B[5], T, h, f)) return -1.0f;
         if (!lora) {
             const seraph_gemm_problem_t gu[2] = {{t->g_gate, a->xn_ffn, GW + t->L.gate, f, h}, {t->g_up, a->xn_ffn, GW + t->L.up, f, h}};
-            GEMM_GROUP(gu, 2, T, 1, 0, 1);
+            SIDE_FORK();
+            WGEMM_GROUP(gu, 2, T);
+            SIDE_MARK(MK_GU);
         }
         GEMM(t->g_gate, W + t->L.gate, t->g_xn, T, h, f, 0, 0, 0);
         GEMM(t->g_up, W + t->L.up, t->g_xn, T, h, f, 0, 0, 1);
+        SIDE_JOIN(MK_DOWN);                                                  /* g_hidden is rewritten next */
         /* the input gradient is added to the residual stream's gradient as it is stored (src/train.c:5180-5193) */
         OP("rmsnorm_backward", 0.0, 16.0 * (double)(T * h), seraph_rmsnorm_backward_residual(a->post_in, W + t->L.post_norm, t->g_xn, t->g_hidden, t->g_hidden,
                                    lora ? t->scratch_gs : GW + t->L.post_norm, T, h, eps, t->ws, t->ws_bytes, s));
 
         /* attention */
-        if (!lora) GEMM(t->g_hidden, a->attn_out, GW + t->L.o, h, qd, T, 1, 0, 1);
+        SIDE_FORK();
+        if (!lora) WGEMM(t->g_hidden, a->attn_out, GW + t->L.o, h, qd, T);
+        SIDE_MARK(MK_O);
         GEMM(t->g_hidden, W + t->L.o, t->g_attn, T, qd, h, 0, 0, 0);
         NANCHK(t->g_attn, T * qd, nan_bwd + 5u * (uint32_t)l + 0u);
         if (lora && t->LL.A[3] >= 0 &&
             lora_backward(t, t->g_hidden, a->attn_out, LW + t->LL.A[3], LW + t->LL.B[3], LGW + t->LL.A[3], LGW + t->LL.B[3], T, qd, h)) return -1.0f;
-        OP("fill", 0.0, 4.0 * (double)(T * kv), seraph_fill_u32(t->g_k, 0, (size_t)(T * kv), s));                               /* src/train.c:5221-5222 */
-        OP("fill", 0.0, 4.0 * (double)(T * kv), seraph_fill_u32(t->g_v, 0, (size_t)(T * kv), s));
-        OP("attention_backward", 10.0 * D * t->attn_pairs * H, 0.0, seraph_attention_backward_banded(a->q, a->k, a->v, t->g_attn, a->attn_out, a->lse, t->g_q, t->g_k, t->g_v,
-                                     starts, batch, T, H, KVH, D, scale, t->max_seq_len, t->attn_ws, t->attn_ws_bytes, s));
+        SIDE_JOIN(MK_QKV);                                                   /* the layer above still reads g_q / g_k / g_v */
+        /* dK / dV are assigned, so the zero fills of src/train.c:5221-5222 have nothing left to do; the host's copy
+         * of the offsets sizes the dS band */
+        OP("attention_backward", 10.0 * D * t->attn_pairs * H, 0.0, seraph_attention_backward_assign(a->q, a->k, a->v, t->g_attn, a->attn_out, a->lse, t->g_q, t->g_k, t->g_v,
+                                     starts, t->h_stage + 2 * (size_t)T, batch, T, H, KVH, D, scale, t->attn_ws, t->attn_ws_bytes, s));
         NANCHK(t->g_q, T * qd, nan_bwd + 5u * (uint32_t)l + 1u);
         NANCHK(t->g_k, T * kv, nan_bwd + 5u * (uint32_t)l + 2u);
         NANCHK(t->g_v, T * kv, nan_bwd + 5u * (uint32_t)l + 3u);
@@ -761,7 +825,9 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         if (!lora) {
             const seraph_gemm_problem_t qkv[3] = {{t->g_q, a->xn_attn, GW + t->L.q, qd, h}, {t->g_k, a->xn_attn, GW + t->L.k, kv, h},
                                                   {t->g_v, a->xn_attn, GW + t->L.v, kv, h}};
-            GEMM_GROUP(qkv, 3, T, 1, 0, 1);
+            SIDE_FORK();
+            WGEMM_GROUP(qkv, 3, T);
+            SIDE_MARK(MK_QKV);
         } else {
             float* gs[3] = {t->g_q, t->g_k, t->g_v};
             int64_t outs[3] = {qd, kv, kv};
@@ -772,11 +838,14 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         GEMM(t->g_q, W + t->L.q, t->g_xn, T, h, qd, 0, 0, 0);
         GEMM(t->g_k, W + t->L.k, t->g_xn, T, h, kv, 0, 0, 1);
         GEMM(t->g_v, W + t->L.v, t->g_xn, T, h, kv, 0, 0, 1);
+        SIDE_JOIN(MK_O);                                                     /* g_hidden is rewritten next */
         OP("rmsnorm_backward", 0.0, 16.0 * (double)(T * h), seraph_rmsnorm_backward_residual(a->layer_in, W + t->L.in_norm, t->g_xn, t->g_hidden, t->g_hidden,
                                    lora ? t->scratch_gs : GW + t->L.in_norm, T, h, eps, t->ws, t->ws_bytes, s));       /* src/train.c:5342-5355 */
         NANCHK(t->g_hidden, T * h, nan_gh + (uint32_t)l);
     }
     NANCHK(t->g_hidden, T * h, 8u);
+    SIDE_MARK(MK_END);
+    SIDE_JOIN(MK_END);                                                       /* every weight gradient is complete from here on */
     if (!lora) OP("embedding_backward", 0.0, 12.0 * (double)(T * h), seraph_embedding_backward(t->d_tokens, t->g_hidden, t->G + t->off_embed, T, h, V, t->ws, t->ws_bytes, s));
     if (!lora) NANCHK(t->G + t->off_embed, V * h, 9u);
     CK(seraph_hip_event_record(t->ev[2], s));

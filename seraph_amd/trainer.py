@@ -74,6 +74,8 @@ def _lib():
         lib.hip_trainer_device_bytes.restype = C.c_size_t
         lib.hip_trainer_device_bytes.argtypes = [C.c_void_p]
         lib.hip_trainer_enable_op_timing.argtypes = [C.c_void_p, C.c_int]
+        lib.hip_trainer_enable_wgrad_overlap.argtypes = [C.c_void_p, C.c_int]
+        lib.hip_trainer_enable_wgrad_overlap.restype = None
         lib.hip_trainer_reset_op_stats.argtypes = [C.c_void_p]
         lib.hip_trainer_op_stats.argtypes = [C.c_void_p, C.POINTER(OpStat), C.c_int]
         lib.hip_trainer_upload_at.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_void_p, C.c_int64]
@@ -225,6 +227,10 @@ class Trainer:
 
     def enable_op_timing(self, on=True):
         _lib().hip_trainer_enable_op_timing(self._h, 1 if on else 0)
+
+    def enable_wgrad_overlap(self, on=True):
+        """Weight gradients on a second stream beside the input-gradient chain (full-weight mode; on by default)."""
+        _lib().hip_trainer_enable_wgrad_overlap(self._h, 1 if on else 0)
 
     def reset_op_stats(self):
         _lib().hip_trainer_reset_op_stats(self._h)

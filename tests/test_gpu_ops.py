@@ -454,6 +454,31 @@ def test_attention_backward(ops, orc, starts, H, KVH, D, saved, banded):
     parity(dQ, rdQ, "dQ"); parity(dK, rdK, "dK"); parity(dV, rdV, "dV")
 
 
+@pytest.mark.parametrize("starts,H,KVH,D", ATTN_CASES_BWD)
+def test_attention_backward_assign_equals_the_adding_form_on_zeroed_buffers(ops, starts, H, KVH, D):
+    """dK / dV assigned over buffers that hold NaN, the dS band sized from the host's copy of the offsets: bit-identical to
+    the adding form run on zeroed dK / dV with the exact bound (which the case above holds against the oracle)."""
+    Q, K, V, dO = _attn_inputs(12, starts, H, KVH, D)
+    sd = dev(np.array(starts, np.int32))
+    out, lse = ops.attention_forward(dev(Q), dev(K), dev(V), H, KVH, D, sd)
+    ref = ops.attention_backward(dev(Q), dev(K), dev(V), dev(dO), H, KVH, D, sd, out=out, lse=lse,
+                                 max_seq_len=int(np.diff(starts).max()))
+    junk = np.full(K.shape, np.nan, np.float32)
+    got = ops.attention_backward_assign(dev(Q), dev(K), dev(V), dev(dO), H, KVH, D, sd, starts, out=out, lse=lse,
+                                        dK=dev(junk), dV=dev(junk))
+    for g, r, name in zip(got, ref, ("dQ", "dK", "dV")):
+        assert np.array_equal(host(g), host(r)), name
+
+
+def test_attention_backward_assign_checks_the_host_offsets(ops):
+    from seraph_amd._lib import SeraphError
+    Q, K, V, dO = _attn_inputs(13, [0, 40, 100], 2, 2, 32)
+    sd = dev(np.array([0, 40, 100], np.int32))
+    for bad in ([0, 40, 90], [1, 40, 100], [0, 60, 50, 100][:3]):
+        with pytest.raises(SeraphError):
+            ops.attention_backward_assign(dev(Q), dev(K), dev(V), dev(dO), 2, 2, 32, sd, bad)
+
+
 def test_rope_and_cross_entropy_many_short_sequences(ops, orc):
     """Thousands of packed sequences: positions restart and the last token of each has no target."""
     n_seq = 3000

@@ -132,6 +132,30 @@ def test_full_step_gradient_accumulation(tr, orc):
     t.close()
 
 
+def test_weight_gradients_on_the_second_stream_change_no_bit(tr, orc):
+    """Three optimizer steps with the weight gradients beside the input-gradient chain (default) and with everything on
+    one stream: every product is one kernel either way, so weights, gradients and moments must be identical; a missing
+    wait between the streams would show as a difference (and the step above already pins the default against the oracle)."""
+    case = dict(hidden=256, layers=4, heads=4, kv_heads=2, head_dim=64, ffn=704, vocab=4096)
+    ocfg = orc.make_config(**case)
+    cfg = tr.model_config(**case)
+    p = init_params(orc, ocfg, 31)
+    starts = np.array([0, 256, 300, 1024], np.int32)
+    toks = [rng(40 + i).integers(0, case["vocab"], 1024).astype(np.int32) for i in range(3)]
+    out = []
+    for overlap in (True, False):
+        t = tr.Trainer(cfg, tr.optim_config(1e-3, warmup_steps=1), max_tokens=1024, max_batch=3)
+        t.enable_wgrad_overlap(overlap)
+        t.upload(tr.PARAMS, p)
+        losses = [t.step(tok, starts) for tok in toks]
+        out.append((losses, t.download(tr.PARAMS), t.download(tr.GRADS), t.download(tr.ADAM_V)))
+        t.close()
+    assert out[0][0] == out[1][0]
+    for a, b in zip(out[0][1:], out[1][1:]):
+        assert np.array_equal(a, b)
+    assert np.abs(out[0][1] - p).max() > 0
+
+
 @pytest.mark.parametrize("mask", [0b0001111, 0b1111111, 0b1010101])
 @pytest.mark.parametrize("b_zero", [True, False])
 def test_lora_step(tr, orc, b_zero, mask):
