@@ -125,6 +125,16 @@ int seraph_gemm_grouped(const seraph_gemm_problem_t* problems, int count, int64_
                         int transpose_A, int transpose_B, int accumulate, seraph_stream_t s);
 const char* seraph_gemm_grouped_kernel_name(const seraph_gemm_problem_t* problems, int count, int64_t K,
                                             int transpose_A, int transpose_B);
+
+/* C (+)= op(A_0) op(B_0) + op(A_1) op(B_1) (+ op(A_2) op(B_2)): products that share M, N and the orientations but not K,
+ * as the input gradient of a layer's gate and up projections (src/train.c:5162-5179) or of q, k and v (:5294-5339), which
+ * the reference forms as separate vulkan_matmul products joined by vulkan_add.  One launch (the sum forms in the accumulators and C is
+ * written once) when every term suits the pipelined kernel, else one seraph_gemm per term.  count 1..3. */
+typedef struct { const float* A; const float* B; int64_t K; } seraph_gemm_term_t;
+int seraph_gemm_chain(const seraph_gemm_term_t* terms, int count, float* C, int64_t M, int64_t N,
+                      int transpose_A, int transpose_B, int accumulate, seraph_stream_t s);
+const char* seraph_gemm_chain_kernel_name(const seraph_gemm_term_t* terms, int count, const float* C, int64_t M, int64_t N,
+                                          int transpose_A, int transpose_B);
 /* C (+)= alpha * op(A) op(B): the step "product, then vulkan_scale of the product" of the LoRA path
  * (src/train.c:5778-5796, :5803-5845) as one call.  With the scratch of seraph_gemm_scaled_ws_bytes a small
  * output with a long K is cut into runs of K that separate workgroups take and a second kernel adds in run

@@ -28,6 +28,7 @@ def kernels():
                      "seraph_gemm_scaled_ws_bytes", "seraph_rmsnorm_backward_static_max_bytes"):
             getattr(lib, name).restype = C.c_size_t
         lib.seraph_gemm_grouped_kernel_name.restype = C.c_char_p
+        lib.seraph_gemm_chain_kernel_name.restype = C.c_char_p
         lib.seraph_gemm_kernel_name.restype = C.c_char_p
         _kernels = lib
     return _kernels

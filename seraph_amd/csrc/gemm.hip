@@ -272,9 +272,19 @@ struct FastLoader {
 };
 
 // pid: the workgroup's tile number within this product (0 .. nbm * nbn - 1), already regrouped per XCD
-template <int TM, int TN, bool A_KC, bool B_KC>
+// With CHAIN the tile is the sum of several products that share M and N (terms of one input gradient: gate and up, or
+// q, k and v): the accumulators stay in registers from one term to the next and C is written once.
+constexpr int kMaxChain = 3;
+struct GemmChain {
+    const float* A[kMaxChain]; const float* B[kMaxChain];
+    int64_t K[kMaxChain];
+    int count;
+};
+
+template <int TM, int TN, bool A_KC, bool B_KC, bool CHAIN = false>
 __device__ __forceinline__ void pipelined_body(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
-                                               int64_t M, int64_t N, int64_t K, int accumulate, int nbm, int nbn, int pid) {
+                                               int64_t M, int64_t N, int64_t K, int accumulate, int nbm, int nbn, int pid,
+                                               const GemmChain* chain = nullptr) {
     constexpr int BM = 64 * TM, BN = 64 * TN;
     constexpr int A_FLOATS = lds_floats<BM, A_KC>(), B_FLOATS = lds_floats<BN, B_KC>();
     __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
@@ -291,7 +301,6 @@ __device__ __forceinline__ void pipelined_body(const float* __restrict__ A, cons
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int wm0 = (wave >> 1) * (32 * TM), wn0 = (wave & 1) * (32 * TN);
-    const int64_t lda = A_KC ? K : M, ldb = B_KC ? K : N;
 
     v16f acc[TM][TN];
 #pragma unroll
@@ -301,6 +310,13 @@ __device__ __forceinline__ void pipelined_body(const float* __restrict__ A, cons
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
+    const int terms = CHAIN ? chain->count : 1;
+    for (int term = 0; term < terms; term++) {
+    if (CHAIN) {
+        A = chain->A[term]; B = chain->B[term]; K = chain->K[term];
+        if (term > 0) __syncthreads();                       // the previous term's last fragment reads precede this term's first LDS writes
+    }
+    const int64_t lda = A_KC ? K : M, ldb = B_KC ? K : N;
     FastLoader<BM, A_KC> la;
     FastLoader<BN, B_KC> lb;
     la.init(lda, m0, M);
@@ -435,6 +451,7 @@ __device__ __forceinline__ void pipelined_body(const float* __restrict__ A, cons
         stage(std::integral_constant<int, 1>{}, kt + 1);
     }
     if (kt < nk) stage(std::integral_constant<int, 0>{}, kt);
+    }   // term
 
     // ---- epilogue: uniform tile pointer + 32-bit lane offsets; predicates only on edge tiles
     float* ct = scalar_ptr(C + m0 * N + n0);
@@ -463,6 +480,12 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_kerne
                                                                                int64_t M, int64_t N, int64_t K,
                                                                                int accumulate, int nbm, int nbn) {
     pipelined_body<TM, TN, A_KC, B_KC>(A, B, C, M, N, K, accumulate, nbm, nbn, xcd_regroup(blockIdx.x, nbm * nbn));
+}
+
+template <int TM, int TN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_chain_kernel(const GemmChain chain, float* __restrict__ C,
+                                                                                     int64_t M, int64_t N, int accumulate, int nbm, int nbn) {
+    pipelined_body<TM, TN, A_KC, B_KC, true>(nullptr, nullptr, C, M, N, 0, accumulate, nbm, nbn, xcd_regroup(blockIdx.x, nbm * nbn), &chain);
 }
 
 // Several products with the same K, operand orientations and accumulate flag in one launch (the q / k / v and the
@@ -870,6 +893,69 @@ extern "C" int seraph_gemm_grouped(const seraph_gemm_problem_t* problems, int co
     else if (tile == 64) { GOG(gemm_f32_mfma_pipelined_grouped_kernel, 1, 1,) }
     else { GOG(gemm_f32_mfma_splitk_grouped_kernel,) }
 #undef GOG
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// C (+)= sum of products that share M and N: one launch when every term suits the pipelined kernel and the output has
+// enough 64x64 tiles for it, else one product after the other.
+static bool chain_ok(const seraph_gemm_term_t* t, int count, const float* C, int64_t M, int64_t N, int tA, int tB) {
+    if (count < 2 || count > kMaxChain || M <= 0 || N <= 0 || !C) return false;
+    int64_t ksum = 0;
+    for (int i = 0; i < count; i++) {
+        const int64_t K = t[i].K, lda = tA ? M : K, ldb = tB ? K : N;
+        if (!t[i].A || !t[i].B || lda % 4 || ldb % 4 || !aligned16(t[i].A) || !aligned16(t[i].B)) return false;
+        if (!pipelined_ok(M, N, K, tA, tB)) return false;
+        ksum += K;
+    }
+    return !use_splitk(M, N, ksum, tA, tB);
+}
+
+extern "C" const char* seraph_gemm_chain_kernel_name(const seraph_gemm_term_t* terms, int count, const float* C, int64_t M, int64_t N,
+                                                     int transpose_A, int transpose_B) {
+    static const char* names[2][4] = {
+        {"seraph::gemm_f32_mfma_pipelined_chain_kernel<1, 1, true, false>", "seraph::gemm_f32_mfma_pipelined_chain_kernel<1, 1, true, true>",
+         "seraph::gemm_f32_mfma_pipelined_chain_kernel<1, 1, false, false>", "seraph::gemm_f32_mfma_pipelined_chain_kernel<1, 1, false, true>"},
+        {"seraph::gemm_f32_mfma_pipelined_chain_kernel<2, 2, true, false>", "seraph::gemm_f32_mfma_pipelined_chain_kernel<2, 2, true, true>",
+         "seraph::gemm_f32_mfma_pipelined_chain_kernel<2, 2, false, false>", "seraph::gemm_f32_mfma_pipelined_chain_kernel<2, 2, false, true>"}};
+    if (!terms || !chain_ok(terms, count, C, M, N, transpose_A, transpose_B)) return "gemm (chain run as single products)";
+    return names[use_big_tiles(M, N) ? 1 : 0][(transpose_A ? 2 : 0) + (transpose_B ? 1 : 0)];
+}
+
+extern "C" int seraph_gemm_chain(const seraph_gemm_term_t* terms, int count, float* C, int64_t M, int64_t N,
+                                 int transpose_A, int transpose_B, int accumulate, seraph_stream_t s) {
+    if (count <= 0 || M == 0 || N == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(terms && C, "gemm_chain: NULL pointer");
+    if (!chain_ok(terms, count, C, M, N, transpose_A, transpose_B)) {
+        for (int i = 0; i < count; i++) {
+            int rc = seraph_gemm(terms[i].A, terms[i].B, C, M, N, terms[i].K, transpose_A, transpose_B, (accumulate || i > 0) ? 1 : 0, s);
+            if (rc != SERAPH_OK) return rc;
+        }
+        return SERAPH_OK;
+    }
+    GemmChain ch;
+    ch.count = count;
+    for (int i = 0; i < kMaxChain; i++) {
+        const int j = i < count ? i : count - 1;
+        ch.A[i] = terms[j].A; ch.B[i] = terms[j].B; ch.K[i] = terms[j].K;
+    }
+    const bool big = use_big_tiles(M, N);
+    const int tile = big ? 128 : 64;
+    const int64_t nbm = ceil_div(M, tile), nbn = ceil_div(N, tile);
+    SERAPH_REQUIRE(nbm * nbn <= 0x7fffffff, "gemm_chain: too many tiles");
+    hipStream_t st = as_stream(s);
+    const dim3 grid((unsigned)(nbm * nbn)), block(kGemmThreads);
+    const int form = (transpose_A ? 2 : 0) + (transpose_B ? 1 : 0);
+#define GOC(TMN) \
+    switch (form) { \
+        case 0: hipLaunchKernelGGL((gemm_f32_mfma_pipelined_chain_kernel<TMN, TMN, true, false>), grid, block, 0, st, ch, C, M, N, accumulate, (int)nbm, (int)nbn); break; \
+        case 1: hipLaunchKernelGGL((gemm_f32_mfma_pipelined_chain_kernel<TMN, TMN, true, true>), grid, block, 0, st, ch, C, M, N, accumulate, (int)nbm, (int)nbn); break; \
+        case 2: hipLaunchKernelGGL((gemm_f32_mfma_pipelined_chain_kernel<TMN, TMN, false, false>), grid, block, 0, st, ch, C, M, N, accumulate, (int)nbm, (int)nbn); break; \
+        default: hipLaunchKernelGGL((gemm_f32_mfma_pipelined_chain_kernel<TMN, TMN, false, true>), grid, block, 0, st, ch, C, M, N, accumulate, (int)nbm, (int)nbn); break; \
+    }
+    if (big) { GOC(2) } else { GOC(1) }
+#undef GOC
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }

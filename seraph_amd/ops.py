@@ -104,6 +104,25 @@ def gemm_grouped(problems, K, tA=0, tB=0, accumulate=False):
     return [c for _, _, c, _, _ in problems]
 
 
+class GemmTerm(C.Structure):
+    _fields_ = [("A", C.c_void_p), ("B", C.c_void_p), ("K", C.c_int64)]
+
+
+def gemm_chain(terms, M, N, tA=0, tB=0, out=None, accumulate=False):
+    """out (+)= sum of op(A_i) op(B_i) over terms (A_i, B_i, K_i) that share M, N and the orientations."""
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=terms[0][0].device)
+    arr = (GemmTerm * len(terms))(*[GemmTerm(a.data_ptr(), b.data_ptr(), k) for a, b, k in terms])
+    check(kernels().seraph_gemm_chain(arr, C.c_int(len(terms)), _p(out), i64(M), i64(N), C.c_int(tA), C.c_int(tB),
+                                      C.c_int(1 if accumulate else 0), _stream()), "gemm_chain")
+    return out
+
+
+def gemm_chain_kernel_name(terms, out, M, N, tA=0, tB=0):
+    arr = (GemmTerm * len(terms))(*[GemmTerm(a.data_ptr(), b.data_ptr(), k) for a, b, k in terms])
+    return kernels().seraph_gemm_chain_kernel_name(arr, C.c_int(len(terms)), _p(out), i64(M), i64(N), C.c_int(tA), C.c_int(tB)).decode()
+
+
 def gemm_scaled(A, B, M, N, K, tA=0, tB=0, out=None, accumulate=False, alpha=1.0, scratch=True):
     """out (+)= alpha * op(A) op(B); with scratch, small outputs with a long K are computed in runs of K."""
     if out is None:

@@ -162,6 +162,15 @@ static void op_fold(hip_trainer_t* t) {
            seraph_gemm_grouped((probs_), (count_), (K_), (tA_), (tB_), (acc_), t->stream));            \
     } while (0)
 
+/* an input gradient that is the sum of several products (gate + up, q + k + v) in one launch */
+#define GEMM_CHAIN(terms_, count_, C_, M_, N_)                                                         \
+    do {                                                                                               \
+        double fl_ = 0.0;                                                                              \
+        for (int gi_ = 0; gi_ < (count_); gi_++) fl_ += 2.0 * (double)(M_) * (double)(N_) * (double)(terms_)[gi_].K; \
+        OP(seraph_gemm_chain_kernel_name((terms_), (count_), (C_), (M_), (N_), 0, 0), fl_, 0.0,        \
+           seraph_gemm_chain((terms_), (count_), (C_), (M_), (N_), 0, 0, 0, t->stream));               \
+    } while (0)
+
 #define WGEMM_GROUP(probs_, count_, K_)                                                                \
     do {                                                                                               \
         double fl_ = 0.0;                                                                              \
@@ -793,8 +802,10 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
             WGEMM_GROUP(gu, 2, T);
             SIDE_MARK(MK_GU);
         }
-        GEMM(t->g_gate, W + t->L.gate, t->g_xn, T, h, f, 0, 0, 0);
-        GEMM(t->g_up, W + t->L.up, t->g_xn, T, h, f, 0, 0, 1);
+        {   /* grad_x_norm_ffn = grad_gate Wgate + grad_up Wup (src/train.c:5162-5179) */
+            const seraph_gemm_term_t gu[2] = {{t->g_gate, W + t->L.gate, f}, {t->g_up, W + t->L.up, f}};
+            GEMM_CHAIN(gu, 2, t->g_xn, T, h);
+        }
         SIDE_JOIN(MK_DOWN);                                                  /* g_hidden is rewritten next */
         /* the input gradient is added to the residual stream's gradient as it is stored (src/train.c:5180-5193) */
         OP("rmsnorm_backward", 0.0, 16.0 * (double)(T * h), seraph_rmsnorm_backward_residual(a->post_in, W + t->L.post_norm, t->g_xn, t->g_hidden, t->g_hidden,
@@ -835,9 +846,10 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
                 if (t->LL.A[p] >= 0 &&
                     lora_backward(t, gs[p], a->xn_attn, LW + t->LL.A[p], LW + t->LL.B[p], LGW + t->LL.A[p], LGW + t->LL.B[p], T, h, outs[p])) return -1.0f;
         }
-        GEMM(t->g_q, W + t->L.q, t->g_xn, T, h, qd, 0, 0, 0);
-        GEMM(t->g_k, W + t->L.k, t->g_xn, T, h, kv, 0, 0, 1);
-        GEMM(t->g_v, W + t->L.v, t->g_xn, T, h, kv, 0, 0, 1);
+        {   /* grad_x_norm = grad_q Wq + grad_k Wk + grad_v Wv (src/train.c:5294-5339) */
+            const seraph_gemm_term_t qkv[3] = {{t->g_q, W + t->L.q, qd}, {t->g_k, W + t->L.k, kv}, {t->g_v, W + t->L.v, kv}};
+            GEMM_CHAIN(qkv, 3, t->g_xn, T, h);
+        }
         SIDE_JOIN(MK_O);                                                     /* g_hidden is rewritten next */
         OP("rmsnorm_backward", 0.0, 16.0 * (double)(T * h), seraph_rmsnorm_backward_residual(a->layer_in, W + t->L.in_norm, t->g_xn, t->g_hidden, t->g_hidden,
                                    lora ? t->scratch_gs : GW + t->L.in_norm, T, h, eps, t->ws, t->ws_bytes, s));       /* src/train.c:5342-5355 */

@@ -246,6 +246,34 @@ def test_gemm_grouped(ops, orc, tA, tB, shapes, K):
         parity(o, orc.matmul(host(a), host(b), m, n, K, tA, tB), "grouped gemm, overwrite", atol=1e-4)
 
 
+@pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("M,N,Ks", [(2048, 512, (1408, 1408)), (2048, 512, (512, 512, 512)), (1024, 2048, (2048, 1024, 1024)),
+                                    (4100, 2048, (512, 256)),            # 128x128 tiles with a ragged edge
+                                    (300, 260, (64, 32, 96)),            # edge tiles in both directions
+                                    (96, 64, (2048, 1024)),              # too few tiles: runs as single products
+                                    (130, 70, (36, 64)),                 # a K that is not whole stages: single products
+                                    (512, 512, (128,))])
+def test_gemm_chain(ops, orc, tA, tB, M, N, Ks):
+    """C (+)= sum of products with different K in one launch: against the oracle's products added in double precision,
+    for the overwriting and the accumulating form."""
+    r = rng(M + N + sum(Ks) + 2 * tA + tB)
+    terms, ref = [], np.zeros((M, N), np.float64)
+    for K in Ks:
+        A = (0.25 * r.standard_normal((K, M) if tA else (M, K))).astype(np.float32)     # sums of up to 4096 terms stay O(1)
+        B = (0.25 * r.standard_normal((N, K) if tB else (K, N))).astype(np.float32)
+        terms.append((dev(A), dev(B), K))
+        ref += orc.matmul(A, B, M, N, K, tA, tB).astype(np.float64)
+    out = ops.gemm_chain(terms, M, N, tA, tB, out=torch.full((M, N), float("nan"), device="cuda"))
+    parity(out, ref.astype(np.float32), f"gemm chain {M}x{N}x{Ks}", atol=1e-4)
+    C0 = r.standard_normal((M, N)).astype(np.float32)
+    out = ops.gemm_chain(terms, M, N, tA, tB, out=dev(C0), accumulate=True)
+    parity(out, (ref + C0).astype(np.float32), f"gemm chain {M}x{N}x{Ks}, accumulate", atol=1e-4)
+    name = ops.gemm_chain_kernel_name(terms, out, M, N, tA, tB)
+    few_tiles = ((M + 63) // 64) * ((N + 63) // 64) < 256             # with a long K such an output is cut along K instead
+    one_launch = len(Ks) > 1 and all(K % 32 == 0 for K in Ks) and not (few_tiles and sum(Ks) >= 256)
+    assert ("chain_kernel" in name) == one_launch, name
+
+
 # ------------------------------------------------------------------ rmsnorm
 @pytest.mark.parametrize("rows,cols", [(33, 512), (17, 2048), (5, 4096), (9, 100), (4, 8192), (1, 4)])
 def test_rmsnorm_forward_backward(ops, orc, rows, cols):
