@@ -71,7 +71,14 @@ int  seraph_hip_stream_sync(seraph_stream_t s);
 int  seraph_hip_device_sync(void);
 /* event pair timing on a stream (vulkan_profiler_* stand-in, include/vulkan_backend.h:638-642) */
 int  seraph_hip_event_create(void** out);
+int  seraph_hip_event_create_sync(void** out);                         /* orders streams of one device only: no timestamps, not for the host to wait on */
 int  seraph_hip_event_destroy(void* ev);
+/* Arms `ev` for the calling thread: the next op of this library that supports it (SwiGLU backward, RoPE, RMSNorm backward,
+ * reduce_sum) completes the event with its last kernel, which is what hipEventRecord after the op would give, minus the
+ * marker packet that a record puts between that kernel and the next.  seraph_hip_event_armed() tells afterwards whether
+ * the event is still waiting for such an op (then record it the ordinary way; calling seraph_hip_event_on_next_op(NULL) disarms). */
+int  seraph_hip_event_on_next_op(void* ev);
+int  seraph_hip_event_armed(void);
 int  seraph_hip_event_record(void* ev, seraph_stream_t s);
 int  seraph_hip_event_elapsed_ms(void* start, void* stop, float* ms);  /* waits for stop */
 /* work submitted to `s` after this call starts only when everything recorded into `ev` has completed (two streams of

@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdio.h>
 
@@ -33,6 +34,18 @@ void set_error(const char* fmt, ...);
     } while (0)
 
 #define SERAPH_LAUNCH_CHECK() SERAPH_HIP_CHECK(hipGetLastError())
+
+// Launch of the kernel that ends an op.  When the caller has armed an event for this thread
+// (seraph_hip_event_on_next_op) the event completes with this very dispatch, so a second stream can wait for
+// the op without a marker packet between this kernel and the next one on its own stream.
+hipEvent_t take_armed_event();
+void arm_event(hipEvent_t ev);      // an op with several launches takes the event at entry and arms it again before its last one
+#define SERAPH_LAUNCH_LAST(kernel, grid, block, shmem, st, ...)                                          \
+    do {                                                                                                 \
+        hipEvent_t ev_ = ::seraph::take_armed_event();                                                   \
+        if (ev_) hipExtLaunchKernelGGL(kernel, grid, block, shmem, st, nullptr, ev_, 0, __VA_ARGS__);    \
+        else hipLaunchKernelGGL(kernel, grid, block, shmem, st, __VA_ARGS__);                            \
+    } while (0)
 
 static inline hipStream_t as_stream(seraph_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -34,7 +34,7 @@ static int launch_stream(F f, size_t n, bool vec_ok, hipStream_t st) {
     const size_t lanes = n4 + (n - 4 * n4);
     const size_t grid = (lanes + BLOCK - 1) / BLOCK;
     SERAPH_REQUIRE(grid <= 0x7fffffffu, "streaming op over %zu elements exceeds the launch limit", n);
-    hipLaunchKernelGGL((stream_kernel<F, BLOCK>), dim3((unsigned)grid), dim3(BLOCK), 0, st, f, n4, n);
+    SERAPH_LAUNCH_LAST((stream_kernel<F, BLOCK>), dim3((unsigned)grid), dim3(BLOCK), 0, st, f, n4, n);
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }
@@ -355,7 +355,7 @@ int seraph_reduce_sum(const float* in, float* out, size_t count, seraph_stream_t
     SERAPH_REQUIRE(in && out, "reduce_sum: NULL pointer");
     size_t groups = (count + 511) / 512;
     SERAPH_REQUIRE(groups <= 0x7fffffffu, "reduce_sum: count too large");
-    hipLaunchKernelGGL(reduce_sum_512_kernel, dim3((unsigned)groups), dim3(kBlock), 0, as_stream(s), in, out, count);
+    SERAPH_LAUNCH_LAST(reduce_sum_512_kernel, dim3((unsigned)groups), dim3(kBlock), 0, as_stream(s), in, out, count);
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }

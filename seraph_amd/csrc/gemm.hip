@@ -742,9 +742,19 @@ static int launch_gemm(const float* A, const float* B, float* C, int64_t M, int6
 
 using namespace seraph;
 
-// 128x128 tiles when they fill the machine at least once, else 64x64.
+// 128x128 or 64x64 tiles, by the rounds the chip needs for them.  A CU works through ceil(tiles / CUs) big tiles, or
+// through its small tiles two at a time (half a round is the step there); a small tile costs a quarter of a big one
+// and runs at about 0.88 of its rate (measured: 2048 x 2816, K 512 with 352 big tiles 67 us, with 1408 small ones
+// 57 us; 2048 x 8192, K 512 with 1024 / 4096 tiles 151 / 167 us; 2048 x 2048 x 2048 with 256 / 1024 tiles 135 / 140 us).
+static bool big_tiles_pay(int64_t t128, int64_t t64) {
+    const int64_t cus = num_compute_units();
+    if (10 * t128 < 9 * cus) return false;                       // big tiles would leave more than a tenth of the chip idle
+    const double cost128 = 4.0 * (double)ceil_div(t128, cus);
+    const double cost64 = 0.5 * (double)ceil_div(2 * t64, cus) / 0.88;
+    return cost128 <= cost64;
+}
 static bool use_big_tiles(int64_t M, int64_t N) {
-    return ceil_div(M, 128) * ceil_div(N, 128) >= num_compute_units();
+    return big_tiles_pay(ceil_div(M, 128) * ceil_div(N, 128), ceil_div(M, 64) * ceil_div(N, 64));
 }
 
 // A k-contiguous pair of operands with at most 32 values of k and a C of whole 16-byte groups.
@@ -838,7 +848,7 @@ static int group_tile(const seraph_gemm_problem_t* p, int count, int64_t K, int 
         t32 += ceil_div(M, 32) * ceil_div(N, 32);
     }
     if (t32 > 0x7fffffff) return 0;
-    if (t128 >= num_compute_units()) return 128;
+    if (big_tiles_pay(t128, t64)) return 128;
     if (t64 >= num_compute_units() || K < 256) return 64;
     return 32;
 }

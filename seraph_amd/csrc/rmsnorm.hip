@@ -638,6 +638,7 @@ static int rmsnorm_backward_launch(const float* x, const float* scale, const flo
                                    float* grad_scale, int64_t rows, int64_t cols, float eps, float* partial,
                                    seraph_stream_t s) {
     hipStream_t st = as_stream(s);
+    const hipEvent_t done = take_armed_event();                 // belongs to the column sum, the last launch
     const bool aligned = aligned16(x) && aligned16(scale) && aligned16(dy) && aligned16(dx) && aligned16(partial) && (!res || aligned16(res));
     const int bvpl = aligned ? pick_block_vpl(cols) : 0;
     const int wvpl = (aligned && !bvpl && cols <= 512) ? pick_vpl(cols) : 0;
@@ -668,10 +669,11 @@ static int rmsnorm_backward_launch(const float* x, const float* scale, const flo
         hipLaunchKernelGGL(rmsnorm_bwd_generic_kernel, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, res, dx, partial, rows, cols, eps);
     }
     SERAPH_LAUNCH_CHECK();
+    arm_event(done);
     if (cols % 4 == 0 && aligned16(partial))
-        hipLaunchKernelGGL(colsum_add_kernel<true>, dim3((unsigned)ceil_div(cols, 64)), dim3(1024), 0, st, partial, nparts, cols, grad_scale);
+        SERAPH_LAUNCH_LAST(colsum_add_kernel<true>, dim3((unsigned)ceil_div(cols, 64)), dim3(1024), 0, st, partial, nparts, cols, grad_scale);
     else
-        hipLaunchKernelGGL(colsum_add_kernel<false>, dim3((unsigned)ceil_div(cols, 64)), dim3(1024), 0, st, partial, nparts, cols, grad_scale);
+        SERAPH_LAUNCH_LAST(colsum_add_kernel<false>, dim3((unsigned)ceil_div(cols, 64)), dim3(1024), 0, st, partial, nparts, cols, grad_scale);
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }

@@ -144,9 +144,9 @@ static int rope_launch(const float* in, float* out, int heads, const float* in2,
     if (wide) {
         dim3 grid4((unsigned)ceil_div(T * (head_dim / 4), (int64_t)kRope4Block));
         if (backward)
-            hipLaunchKernelGGL(rope4_kernel<true>, grid4, dim3(kRope4Block), 0, st, in, out, in2, out2, table, seq_starts, batch, T, heads, heads2, head_dim);
+            SERAPH_LAUNCH_LAST(rope4_kernel<true>, grid4, dim3(kRope4Block), 0, st, in, out, in2, out2, table, seq_starts, batch, T, heads, heads2, head_dim);
         else
-            hipLaunchKernelGGL(rope4_kernel<false>, grid4, dim3(kRope4Block), 0, st, in, out, in2, out2, table, seq_starts, batch, T, heads, heads2, head_dim);
+            SERAPH_LAUNCH_LAST(rope4_kernel<false>, grid4, dim3(kRope4Block), 0, st, in, out, in2, out2, table, seq_starts, batch, T, heads, heads2, head_dim);
         SERAPH_LAUNCH_CHECK();
         return SERAPH_OK;
     }

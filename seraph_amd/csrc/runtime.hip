@@ -7,6 +7,15 @@
 namespace seraph {
 
 static thread_local char g_err[512] = "";
+static thread_local hipEvent_t g_armed_event = nullptr;
+
+void arm_event(hipEvent_t ev) { g_armed_event = ev; }
+
+hipEvent_t take_armed_event() {
+    hipEvent_t ev = g_armed_event;
+    g_armed_event = nullptr;
+    return ev;
+}
 static int g_cu_count = 0;
 
 void set_error(const char* fmt, ...) {
@@ -151,6 +160,23 @@ int seraph_hip_event_create(void** out) {
     *out = reinterpret_cast<void*>(ev);
     return SERAPH_OK;
 }
+
+int seraph_hip_event_create_sync(void** out) {
+    SERAPH_REQUIRE(out, "event_create_sync: NULL out");
+    hipEvent_t ev;
+    // no timestamps, and no system-scope fence when the event completes: it orders streams of this device, whose
+    // kernels release their writes at device scope anyway; the host never inspects it
+    SERAPH_HIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming | hipEventDisableSystemFence));
+    *out = reinterpret_cast<void*>(ev);
+    return SERAPH_OK;
+}
+
+int seraph_hip_event_on_next_op(void* ev) {
+    g_armed_event = reinterpret_cast<hipEvent_t>(ev);
+    return SERAPH_OK;
+}
+
+int seraph_hip_event_armed(void) { return g_armed_event != nullptr; }
 
 int seraph_hip_event_destroy(void* ev) {
     if (ev) SERAPH_HIP_CHECK(hipEventDestroy(reinterpret_cast<hipEvent_t>(ev)));

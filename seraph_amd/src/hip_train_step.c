@@ -180,7 +180,10 @@ static void op_fold(hip_trainer_t* t) {
     } while (0)
 
 /* the second stream picks up from this point of the first | marks a point of the second | the first waits for a mark */
-#define SIDE_FORK()  do { if (ov) { CK(seraph_hip_event_record(t->side_ev[0], s)); CK(seraph_hip_stream_wait_event(sw, t->side_ev[0])); } } while (0)
+#define SIDE_FORK()  do { if (ov) { if (!fork_armed || seraph_hip_event_armed()) { seraph_hip_event_on_next_op(NULL); CK(seraph_hip_event_record(t->side_ev[0], s)); } \
+                                    fork_armed = 0; CK(seraph_hip_stream_wait_event(sw, t->side_ev[0])); } } while (0)
+/* before the op that ends at a fork point: its last kernel completes the fork's event itself */
+#define SIDE_ARM()   do { if (ov) { CK(seraph_hip_event_on_next_op(t->side_ev[0])); fork_armed = 1; } } while (0)
 #define SIDE_MARK(i) do { if (ov) CK(seraph_hip_event_record(t->side_ev[(i)], sw)); } while (0)
 #define SIDE_JOIN(i) do { if (ov) CK(seraph_hip_stream_wait_event(s, t->side_ev[(i)])); } while (0)
 
@@ -304,7 +307,8 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
     for (int i = 0; i < 4; i++) if (seraph_hip_event_create(&t->ev[i]) != SERAPH_OK) goto fail;
     if (!t->lora) {
         if (seraph_hip_stream_create(&t->stream2) != SERAPH_OK) goto fail;
-        for (int i = 0; i < 6; i++) if (seraph_hip_event_create(&t->side_ev[i]) != SERAPH_OK) goto fail;
+        for (int i = 0; i < 6; i++)
+            if (seraph_hip_event_create_sync(&t->side_ev[i]) != SERAPH_OK) goto fail;
         /* Beside a chain of small products the second stream fills CUs that the chain's ramps and tails leave idle
          * (+3 % at 2048 tokens x 512); beside products that fill the chip by themselves it only interleaves two tile
          * orders in every L2 (-7 % at 16384 tokens x 2048).  hip_trainer_enable_wgrad_overlap overrides the choice. */
@@ -766,10 +770,12 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
     void* w2 = ov ? t->ws2 : t->ws;
     const size_t w2b = ov ? t->ws2_bytes : t->ws_bytes;
     enum { MK_DOWN = 1, MK_GU = 2, MK_O = 3, MK_QKV = 4, MK_END = 5 };
+    int fork_armed = 0;
     SIDE_FORK();
     if (!lora) WGEMM(glog, t->xn_final, t->G + t->off_embed, V, h, T);      /* LM head wgrad */
     GEMM(glog, P + t->off_embed, t->g_hidden, T, h, V, 0, 0, 0);            /* LM head dgrad */
     NANCHK(t->g_hidden, T * h, 4u);
+    SIDE_ARM();
     OP("rmsnorm_backward", 0.0, 12.0 * (double)(T * h), seraph_rmsnorm_backward(t->final_in, P + t->off_final_norm, t->g_hidden, t->g_tmp,
                                lora ? t->scratch_gs : t->G + t->off_final_norm, T, h, eps, t->ws, t->ws_bytes, s));
     NANCHK(t->g_tmp, T * h, 5u);
@@ -791,6 +797,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         if (lora && t->LL.A[6] >= 0 &&                                       /* src/train.c:6422-6429 */
             lora_backward(t, t->g_hidden, a->ffn_h, LW + t->LL.A[6], LW + t->LL.B[6], LGW + t->LL.A[6], LGW + t->LL.B[6], T, f, h)) return -1.0f;
         SIDE_JOIN(MK_GU);                                                    /* the layer above still reads g_gate / g_up */
+        if (!lora) SIDE_ARM();
         OP("swiglu_backward", 0.0, 20.0 * (double)(T * f), seraph_swiglu_backward(a->gate, a->up, t->g_ffn, t->g_gate, t->g_up, (size_t)(T * f), s));
         if (lora && t->LL.A[4] >= 0 &&                                       /* src/train.c:6446-6461 */
             lora_backward(t, t->g_gate, a->xn_ffn, LW + t->LL.A[4], LW + t->LL.B[4], LGW + t->LL.A[4], LGW + t->LL.B[4], T, h, f)) return -1.0f;
@@ -808,6 +815,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         }
         SIDE_JOIN(MK_DOWN);                                                  /* g_hidden is rewritten next */
         /* the input gradient is added to the residual stream's gradient as it is stored (src/train.c:5180-5193) */
+        SIDE_ARM();
         OP("rmsnorm_backward", 0.0, 16.0 * (double)(T * h), seraph_rmsnorm_backward_residual(a->post_in, W + t->L.post_norm, t->g_xn, t->g_hidden, t->g_hidden,
                                    lora ? t->scratch_gs : GW + t->L.post_norm, T, h, eps, t->ws, t->ws_bytes, s));
 
@@ -831,6 +839,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
             OP("qk_norm_backward", 0.0, 12.0 * (double)(T * qd), seraph_qk_norm_backward_saved(a->q, a->rms_q, t->g_q, t->g_q, T, H, D, eps, s));
             OP("qk_norm_backward", 0.0, 12.0 * (double)(T * kv), seraph_qk_norm_backward_saved(a->k, a->rms_k, t->g_k, t->g_k, T, KVH, D, eps, s));
         }
+        if (!lora) SIDE_ARM();
         OP("rope", 0.0, 8.0 * (double)(T * (qd + kv)), seraph_rope_qk(t->g_q, t->g_q, H, t->g_k, t->g_k, KVH, starts, batch, T, D, theta, 1, s));
         NANCHK(t->g_q, T * qd, nan_bwd + 5u * (uint32_t)l + 4u);
         if (!lora) {
@@ -851,6 +860,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
             GEMM_CHAIN(qkv, 3, t->g_xn, T, h);
         }
         SIDE_JOIN(MK_O);                                                     /* g_hidden is rewritten next */
+        if (l > 0) SIDE_ARM();
         OP("rmsnorm_backward", 0.0, 16.0 * (double)(T * h), seraph_rmsnorm_backward_residual(a->layer_in, W + t->L.in_norm, t->g_xn, t->g_hidden, t->g_hidden,
                                    lora ? t->scratch_gs : GW + t->L.in_norm, T, h, eps, t->ws, t->ws_bytes, s));       /* src/train.c:5342-5355 */
         NANCHK(t->g_hidden, T * h, nan_gh + (uint32_t)l);
