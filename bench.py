@@ -207,9 +207,10 @@ def run_workload(w, key, steps, warmup, op_timing=True, pmc_calibration=False, w
 
     # Per-kernel timing brackets every kernel-library call of the step with a HIP event pair on the step's
     # stream.  On a step of hundreds of milliseconds that costs well under 1 % and runs inside the timed
-    # region.  On a step of a few milliseconds (c1) the ~1000 event records would take a third of the step,
-    # so the timed region runs without them and the same batches are replayed once more with them.
-    in_region = op_timing and (warmup == 0 or warm_ms >= 100.0)
+    # region.  On a step of a few milliseconds (c1) the ~1000 event records would take a third of the step, and
+    # the ~12000 of the LoRA step (c4, 130 ms) a tenth of it, so there the timed region runs without them and the
+    # same batches are replayed once more with them.
+    in_region = op_timing and (warmup == 0 or warm_ms >= 400.0)
     t.enable_op_timing(in_region)
     t.reset_op_stats()
     torch.cuda.synchronize()
