@@ -131,6 +131,11 @@ def gemm_table(w):
     T, h, f, V = w["batch"] * w["seq"], w["hidden"], w["ffn"], w["vocab"]
     qd, kv, L = w["heads"] * w["head_dim"], w["kv_heads"] * w["head_dim"], w["layers"]
     tot = [0.0, 0.0]
+    warm_a, warm_b = torch.randn(4096, 4096, device="cuda"), torch.randn(4096, 4096, device="cuda")
+    for _ in range(60):                                        # the clocks settle before the first row is timed
+        torch.matmul(warm_a, warm_b)
+    torch.cuda.synchronize()
+    del warm_a, warm_b
     for name, o, i, per_step in (("q", qd, h, L), ("k/v", kv, h, 2 * L), ("o", h, qd, L), ("gate/up", f, h, 2 * L),
                                  ("down", h, f, L), ("lm head", V, h, 1)):
         for form, M, N, K, tA, tB in ((f"fwd {name} NT", T, o, i, 0, 1), (f"dgrad {name} NN", T, i, o, 0, 0),
@@ -145,7 +150,34 @@ def gemm_table(w):
             print(f"{form:18s} {M:6d} x {N:6d} x {K:6d}: {ms:8.3f} ms {2 * M * N * K / ms / 1e9:6.1f} TFLOP/s | "
                   f"hipBLASLt {ref:8.3f} ms {2 * M * N * K / ref / 1e9:6.1f} TFLOP/s | x{per_step} per step", flush=True)
             del A, B, C
-    print(f"GEMM time per step: this library {tot[0]:.1f} ms, hipBLASLt {tot[1]:.1f} ms")
+    print(f"GEMM time per step, one launch per product: this library {tot[0]:.1f} ms, hipBLASLt {tot[1]:.1f} ms")
+
+    # The launches the step really makes for projections that share an operand: q/k/v and gate/up forward and their
+    # weight gradients as one grouped launch each, their input gradients as one launch that sums the products.
+    print("\nproducts the step joins in one launch (hipBLASLt column: the same products one call each, the sum with beta = 1):")
+    R = lambda *sh: torch.randn(*sh, device="cuda")
+    fused = [0.0, 0.0]
+    for name, outs in (("q+k+v", (qd, kv, kv)), ("gate+up", (f, f))):
+        x, ws = R(T, h), [R(o, h) for o in outs]
+        ys, gs, dws = [torch.empty(T, o, device="cuda") for o in outs], [R(T, o) for o in outs], [torch.zeros(o, h, device="cuda") for o in outs]
+        dx = torch.empty(T, h, device="cuda")
+        flops = 2.0 * T * h * sum(outs)
+        cases = (
+            (f"fwd {name} grouped NT", lambda: ops.gemm_grouped([(x, w_, y, T, o) for w_, y, o in zip(ws, ys, outs)], h, 0, 1),
+             lambda: [torch.matmul(x, w_.T, out=y) for w_, y in zip(ws, ys)]),
+            (f"dgrad {name} summed NN", lambda: ops.gemm_chain([(g_, w_, o) for g_, w_, o in zip(gs, ws, outs)], T, h, 0, 0, out=dx),
+             lambda: [torch.matmul(gs[0], ws[0], out=dx)] + [dx.addmm_(g_, w_) for g_, w_ in zip(gs[1:], ws[1:])]),
+            (f"wgrad {name} grouped TN", lambda: ops.gemm_grouped([(g_, x, dw, o, h) for g_, dw, o in zip(gs, dws, outs)], T, 1, 0, accumulate=True),
+             lambda: [dw.addmm_(g_.T, x) for g_, dw in zip(gs, dws)]),
+        )
+        for form, ours, theirs in cases:
+            ms, ref = timeit(ours), timeit(theirs)
+            fused[0] += L * ms
+            fused[1] += L * ref
+            print(f"{form:26s} {T} tokens, widths {h} <-> {'+'.join(str(o) for o in outs)}: {ms:8.3f} ms {flops / ms / 1e9:6.1f} TFLOP/s | "
+                  f"hipBLASLt {ref:8.3f} ms {flops / ref / 1e9:6.1f} TFLOP/s | x{L} per step", flush=True)
+        del x, ws, ys, gs, dws, dx
+    print(f"these launches per step: this library {fused[0]:.1f} ms, hipBLASLt {fused[1]:.1f} ms")
 
 
 def run_workload(w, key, steps, warmup, op_timing=True, pmc_calibration=False, wgrad_overlap=True):
