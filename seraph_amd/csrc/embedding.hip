@@ -8,6 +8,10 @@
 // positions, puts them in ascending order and adds their rows of dH in that order, with a single
 // read-modify-write of the table row.  Three launches; HBM traffic: dH once, each touched row once in and
 // once out.  The sum does not depend on the order in which positions joined, so reruns are bit-identical.
+// A token that fills a large part of the batch (padding, a begin-of-sequence token in thousands of short packed
+// sequences) would leave one wavefront adding thousands of rows alone: such a group is cut along the row's width
+// instead, the first positions of the group to arrive taking one 64-slot slab of columns each, every slab added in
+// the same ascending order - still no scratch, no second level of sums, and the same bits whoever takes which slab.
 #include "common.hpp"
 
 namespace seraph {
@@ -34,7 +38,8 @@ __global__ __launch_bounds__(256) void embed_lookup_kernel(const uint32_t* __res
 // ---------------------------------------------------------------- backward
 constexpr uint32_t kNil = 0xffffffffu;
 struct EmbWs {
-    uint2* tab;         // [vocab]  x = most recent position that joined the token's chain (kNil: none), y = positions so far
+    uint4* tab;         // [vocab]  x = most recent position that joined the token's chain (kNil: none), y = positions so far,
+                        //          z = column slabs of a long group handed out so far
     uint32_t* link;     // [T]      the position that had joined the same token's chain before this one; kNil for the first
 };
 
@@ -42,18 +47,18 @@ static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 
 static size_t emb_ws_layout(int64_t T, int64_t vocab, char* base, EmbWs* w) {
     size_t o = 0;
-    char* tab = base + o; o += align_up((size_t)vocab * 8);
+    char* tab = base + o; o += align_up((size_t)vocab * 16);
     char* link = base + o; o += align_up((size_t)T * 4);
-    if (w) { w->tab = (uint2*)tab; w->link = (uint32_t*)link; }
+    if (w) { w->tab = (uint4*)tab; w->link = (uint32_t*)link; }
     return o;
 }
 
-__global__ __launch_bounds__(256) void emb_init_kernel(uint2* __restrict__ tab, int64_t vocab) {
+__global__ __launch_bounds__(256) void emb_init_kernel(uint4* __restrict__ tab, int64_t vocab) {
     const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (v < vocab) tab[v] = make_uint2(kNil, 0u);
+    if (v < vocab) tab[v] = make_uint4(kNil, 0u, 0u, 0u);
 }
 
-__global__ __launch_bounds__(256) void emb_link_kernel(const uint32_t* __restrict__ tokens, uint2* tab, uint32_t* __restrict__ link,
+__global__ __launch_bounds__(256) void emb_link_kernel(const uint32_t* __restrict__ tokens, uint4* tab, uint32_t* __restrict__ link,
                                                        int64_t T, int64_t vocab) {
     const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (p >= T) return;
@@ -69,8 +74,68 @@ __global__ __launch_bounds__(256) void emb_link_kernel(const uint32_t* __restric
 constexpr int kEmbList = 1024;          // positions gathered per batch
 constexpr int kEmbWalk = 16;            // up to this many positions the chain is walked; longer groups are found by scanning the tokens
 constexpr int kEmbVpl = 8;              // float4 per lane and pass: 2048 floats of a row
+constexpr uint32_t kEmbLong = 128;      // from this many positions on a group is cut into column slabs (rows of more than one slab)
+constexpr int kEmbAhead = 32;           // rows in flight per slab wavefront (32 KB: a round trip of memory at some 10 GB/s per wavefront)
 
-__global__ __launch_bounds__(64) void emb_sum_kernel(const uint32_t* __restrict__ tokens, const uint2* __restrict__ tab,
+// One slab (64 float4 slots of the row's width) of a long group: draw a slab number, leave if all are taken, else sweep the
+// token array for the group's positions (ascending by construction) a batch at a time and add the slab's part of their
+// rows in that order, kEmbAhead rows' loads in flight; one read-modify-write of the slab's part of the table row.
+__device__ __forceinline__ void emb_sum_slab(const uint32_t* __restrict__ tokens, uint4* entry, const float* __restrict__ dH,
+                                             float* row, int64_t T, int64_t hidden, uint32_t tok, uint32_t count, uint32_t* list) {
+    const int lane = threadIdx.x;
+    const int64_t n4 = hidden >> 2, nslabs = (n4 + 63) / 64;
+    uint32_t slab = 0;
+    if (lane == 0) slab = atomicAdd(&entry->z, 1u);
+    slab = __shfl(slab, 0, 64);
+    if ((int64_t)slab >= nslabs) return;
+    const int64_t i4 = (int64_t)slab * 64 + lane;
+    const bool ok = i4 < n4;
+    float4 acc = make_float4(0, 0, 0, 0);
+    int64_t cursor = 0;
+    uint32_t found = 0;
+    while (found < count && cursor < T) {
+        constexpr int U = 8;
+        int len = 0;
+        while (len + 64 * U <= kEmbList && cursor < T && found + (uint32_t)len < count) {
+            uint32_t tk[U];
+#pragma unroll
+            for (int j = 0; j < U; j++) {
+                const int64_t q = cursor + 64 * j + lane;
+                tk[j] = q < T ? tokens[q] : kNil;
+            }
+#pragma unroll
+            for (int j = 0; j < U; j++) {
+                const bool hit = tk[j] == tok;
+                const unsigned long long mask = __ballot(hit);
+                if (hit) list[len + __popcll(mask & ((1ull << lane) - 1ull))] = (uint32_t)(cursor + 64 * j + lane);
+                len += __popcll(mask);
+            }
+            cursor += 64 * U;
+        }
+        __syncthreads();
+        found += (uint32_t)len;
+        int m = 0;
+        for (; m + kEmbAhead <= len; m += kEmbAhead) {
+            float4 g[kEmbAhead];
+#pragma unroll
+            for (int u = 0; u < kEmbAhead; u++)
+                g[u] = ok ? reinterpret_cast<const float4*>(dH + (int64_t)list[m + u] * hidden)[i4] : make_float4(0, 0, 0, 0);
+#pragma unroll
+            for (int u = 0; u < kEmbAhead; u++) { acc.x += g[u].x; acc.y += g[u].y; acc.z += g[u].z; acc.w += g[u].w; }
+        }
+        for (; m < len; m++) {
+            if (ok) { const float4 g = reinterpret_cast<const float4*>(dH + (int64_t)list[m] * hidden)[i4]; acc.x += g.x; acc.y += g.y; acc.z += g.z; acc.w += g.w; }
+        }
+        __syncthreads();
+    }
+    if (ok) {
+        float4 r = reinterpret_cast<float4*>(row)[i4];
+        r.x += acc.x; r.y += acc.y; r.z += acc.z; r.w += acc.w;
+        reinterpret_cast<float4*>(row)[i4] = r;
+    }
+}
+
+__global__ __launch_bounds__(64) void emb_sum_kernel(const uint32_t* __restrict__ tokens, uint4* tab,
                                                      const uint32_t* __restrict__ link,
                                                      const float* __restrict__ dH, float* __restrict__ grad_embed,
                                                      int64_t T, int64_t hidden, int64_t vocab, int vec) {
@@ -89,8 +154,17 @@ __global__ __launch_bounds__(64) void emb_sum_kernel(const uint32_t* __restrict_
     }
     const uint32_t tok = tokens[p];
     const uint32_t lk = link[p];
-    if ((int64_t)tok >= vocab || lk != kNil) return;
+    if ((int64_t)tok >= vocab) return;
     float* row = grad_embed + (int64_t)tok * hidden;
+    const int64_t nslabs = (n4 + 63) / 64;
+    if (lk != kNil) {
+        // Not the owner.  Positions of a long group each offer to take a slab of columns; the rest leave.
+        if (!vec || nslabs < 2) return;
+        const uint4 e = tab[tok];
+        if (e.y < kEmbLong || (int64_t)e.z >= nslabs) return;  // a stale z only costs the draw below
+        emb_sum_slab(tokens, &tab[tok], dH, row, T, hidden, tok, e.y, list);
+        return;
+    }
     float4 old[kEmbVpl];
     if (vec) {
 #pragma unroll
@@ -99,8 +173,12 @@ __global__ __launch_bounds__(64) void emb_sum_kernel(const uint32_t* __restrict_
             old[k] = i < n4 ? reinterpret_cast<const float4*>(row)[i] : make_float4(0, 0, 0, 0);
         }
     }
-    const uint2 e = tab[tok];
+    const uint4 e = tab[tok];
     const uint32_t count = e.y;
+    if (vec && nslabs >= 2 && count >= kEmbLong) {             // a long group: the owner is one slab taker among the others
+        emb_sum_slab(tokens, &tab[tok], dH, row, T, hidden, tok, count, list);
+        return;
+    }
 
     if (count == 1 && vec) {                                   // the common case: nothing to gather
 #pragma unroll

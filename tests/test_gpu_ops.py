@@ -652,13 +652,16 @@ def test_cross_entropy_long_rows_are_deterministic_and_alias_safe(ops, rows, col
     assert float(g_ref[~live].abs().max()) == 0 if (~live).any() else True
 
 
+@pytest.mark.parametrize("h", [256, 520, 2048])
 @pytest.mark.parametrize("case", ["one token", "few tokens", "pairs", "mixed"])
-def test_embedding_backward_repeated_tokens(ops, orc, case):
+def test_embedding_backward_repeated_tokens(ops, orc, case, h):
     """Groups of every size: a batch that is one token repeated (a padding-dominated batch), a handful of tokens, every
-    token twice, and a mixture whose groups straddle the lengths at which the gathering changes method (16) and the
-    batch size of the gather list (1024).  Integer-valued gradients: the sums are exact, so the check is bit-exact."""
+    token twice, and a mixture whose groups straddle the lengths at which the gathering changes method (16), at which a
+    group is cut along the row's width (128, for rows of more than 256 columns: 520 has a ragged third slab, 2048 has
+    eight) and the batch size of the gather list (1024).  Integer-valued gradients: the sums are exact, so the check is
+    bit-exact."""
     r = rng(15)
-    T, h, V = 5000, 256, 3000
+    T, V = 5000, 3000
     if case == "one token":
         tok = np.full(T, 7, np.uint32)
     elif case == "few tokens":
@@ -666,7 +669,7 @@ def test_embedding_backward_repeated_tokens(ops, orc, case):
     elif case == "pairs":
         tok = np.concatenate([r.permutation(T // 2), r.permutation(T // 2)]).astype(np.uint32)
     else:
-        sizes = [1, 2, 15, 16, 17, 63, 64, 65, 1023, 1024, 1025]
+        sizes = [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 1023, 1024, 1025]
         tok = np.concatenate([np.full(n, 10 + i, np.uint32) for i, n in enumerate(sizes)] +
                              [np.arange(100, 100 + T - sum(sizes), dtype=np.uint32)])
         tok = tok[r.permutation(T)]
