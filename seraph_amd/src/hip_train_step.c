@@ -56,7 +56,7 @@ struct hip_trainer {
     char* act_arena;
     size_t act_bytes;
     layer_act_t* act;
-    float *final_in, *xn_final, *logits, *loss_rows, *red_a, *red_b, *tmp_h, *lora_tmp;
+    float *final_in, *xn_final, *logits, *loss_rows, *red_a, *red_b, *tmp_h, *lora_tmp, *lora_tmp2;
     float *g_hidden, *g_tmp, *g_xn, *g_ffn, *g_gate, *g_up, *g_attn, *g_q, *g_k, *g_v, *scratch_gs;
     uint32_t *d_tokens, *d_targets, *d_starts;
     uint32_t* h_stage;           /* pinned: tokens | targets | starts */
@@ -305,15 +305,17 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
     make_layouts(t);
     if (seraph_hip_stream_create(&t->stream) != SERAPH_OK) goto fail;
     for (int i = 0; i < 4; i++) if (seraph_hip_event_create(&t->ev[i]) != SERAPH_OK) goto fail;
-    if (!t->lora) {
-        if (seraph_hip_stream_create(&t->stream2) != SERAPH_OK) goto fail;
-        for (int i = 0; i < 6; i++)
-            if (seraph_hip_event_create_sync(&t->side_ev[i]) != SERAPH_OK) goto fail;
-        /* Beside a chain of small products the second stream fills CUs that the chain's ramps and tails leave idle
-         * (+3 % at 2048 tokens x 512); beside products that fill the chip by themselves it only interleaves two tile
-         * orders in every L2 (-7 % at 16384 tokens x 2048).  hip_trainer_enable_wgrad_overlap overrides the choice. */
-        t->overlap = (int64_t)max_tokens * cfg->hidden <= ((int64_t)1 << 22);
-    }
+    if (seraph_hip_stream_create(&t->stream2) != SERAPH_OK) goto fail;
+    for (int i = 0; i < 6; i++)
+        if (seraph_hip_event_create_sync(&t->side_ev[i]) != SERAPH_OK) goto fail;
+    /* Beside a chain of small products the second stream fills CUs that the chain's ramps and tails leave idle
+     * (+3 % at 2048 tokens x 512); beside products that fill the chip by themselves it only interleaves two tile
+     * orders in every L2 (-7 % at 16384 tokens x 2048).  The adapter gradients of a LoRA step (rank-sized products,
+     * eight short launches per adapter that nothing on the chain waits for) can leave the chain the same way, but
+     * beside the frozen model's large products that costs more than the launches it hides (1 x 2048 tokens of the
+     * 1.7B shape: 128.9 against 126.5 ms), so a LoRA step stays on one stream unless told otherwise.
+     * hip_trainer_enable_wgrad_overlap overrides the choice. */
+    t->overlap = t->lora ? 0 : (int64_t)max_tokens * cfg->hidden <= ((int64_t)1 << 22);
 
     const size_t pbytes = (size_t)t->nparams * sizeof(float);
     t->P = ext_params;
@@ -341,7 +343,7 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
         const size_t r = cfg->lora_rank > 0 ? (size_t)cfg->lora_rank : 1;
         const size_t per_layer = 4 * up256(T * h * 4) + 2 * up256(T * qd * 4) + 2 * up256(T * kv * 4) +
                                  up256(T * cfg->heads * 4) + 3 * up256(T * f * 4) + (cfg->use_qk_norm ? 2 * up256(T * 4) : 0);
-        const size_t rest = 2 * up256(T * h * 4) + up256(T * Vv * 4) + 3 * up256(T * 4) + up256(T * h * 4) + up256(T * r * 4) +
+        const size_t rest = 2 * up256(T * h * 4) + up256(T * Vv * 4) + 3 * up256(T * 4) + up256(T * h * 4) + 2 * up256(T * r * 4) +
                             3 * up256(T * h * 4) + 3 * up256(T * f * 4) + 2 * up256(T * qd * 4) + 2 * up256(T * kv * 4) +
                             up256(h * 4) + 2 * up256(T * 4) + up256(((size_t)max_batch + 1) * 4);
         t->act_bytes = per_layer * (size_t)cfg->layers + rest;
@@ -360,7 +362,7 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
         }
         TAKE(t->final_in, T * h * 4); TAKE(t->xn_final, T * h * 4); TAKE(t->logits, T * Vv * 4);
         TAKE(t->loss_rows, T * 4); TAKE(t->red_a, T * 4); TAKE(t->red_b, T * 4);
-        TAKE(t->tmp_h, T * h * 4); TAKE(t->lora_tmp, T * r * 4);
+        TAKE(t->tmp_h, T * h * 4); TAKE(t->lora_tmp, T * r * 4); TAKE(t->lora_tmp2, T * r * 4);
         TAKE(t->g_hidden, T * h * 4); TAKE(t->g_tmp, T * h * 4); TAKE(t->g_xn, T * h * 4);
         TAKE(t->g_ffn, T * f * 4); TAKE(t->g_gate, T * f * 4); TAKE(t->g_up, T * f * 4);
         TAKE(t->g_attn, T * qd * 4); TAKE(t->g_q, T * qd * 4); TAKE(t->g_k, T * kv * 4); TAKE(t->g_v, T * kv * 4);
@@ -383,6 +385,7 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
                 t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(Tm, r, dims[i], 0, 0));
                 t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(dims[i], r, Tm, 1, 0));
                 t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(r, dims[i], Tm, 1, 0));
+                t->ws2_bytes = t->ws_bytes;
             } else {
                 for (int j = 0; j < 4; j++) {
                     t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(dims[i], dims[j], Tm, 1, 0));
@@ -517,14 +520,24 @@ static int lora_forward_add(hip_trainer_t* t, const float* x, float* out, const 
 }
 
 /* src/train.c:5803-5845 with grad_input == NULL, as every call site passes it */
+/* The four products are rank-sized and nothing on the chain of input gradients reads their results, so the step may
+ * run them on its second stream (side != 0: that stream's scratch and its own tmp). */
 static int lora_backward(hip_trainer_t* t, const float* dY, const float* x, const float* A, const float* B,
-                         float* gA, float* gB, int64_t T, int64_t in, int64_t outd) {
+                         float* gA, float* gB, int64_t T, int64_t in, int64_t outd, int side) {
     const int r = t->cfg.lora_rank;
     const float s = t->cfg.lora_alpha / (float)r;
-    GEMM_SCALED(x, A, t->lora_tmp, T, r, in, 0, 1, 0, s);
-    GEMM_SCALED(dY, t->lora_tmp, gB, outd, r, T, 1, 0, 1, 1.0f);
-    GEMM_SCALED(dY, B, t->lora_tmp, T, r, outd, 0, 0, 0, s);
-    GEMM_SCALED(t->lora_tmp, x, gA, r, in, T, 1, 0, 1, 1.0f);
+    float* tmp = side ? t->lora_tmp2 : t->lora_tmp;
+    void* ws = side ? t->ws2 : t->ws;
+    const size_t wsb = side ? t->ws2_bytes : t->ws_bytes;
+    seraph_stream_t st = side ? t->stream2 : t->stream;
+#define LGEMM(A_, B_, C_, M_, N_, K_, tA_, tB_, acc_, alpha_)                                          \
+    OP("gemm_scaled", 2.0 * (double)(M_) * (double)(N_) * (double)(K_), 0.0,                           \
+       seraph_gemm_scaled((A_), (B_), (C_), (M_), (N_), (K_), (tA_), (tB_), (acc_), (alpha_), ws, wsb, st))
+    LGEMM(x, A, tmp, T, r, in, 0, 1, 0, s);
+    LGEMM(dY, tmp, gB, outd, r, T, 1, 0, 1, 1.0f);
+    LGEMM(dY, B, tmp, T, r, outd, 0, 0, 0, s);
+    LGEMM(tmp, x, gA, r, in, T, 1, 0, 1, 1.0f);
+#undef LGEMM
     return 0;
 }
 
@@ -765,7 +778,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
      * (fork), and the first stream waits for it (join) only where it is about to overwrite one of them: g_hidden at
      * the next norm backward, g_gate / g_up and g_q / g_k / g_v in the next layer down. With per-op timing or the NaN
      * lattice on, everything stays on one stream. */
-    const int ov = t->overlap && !lora && !t->op_timing && !t->nan_check;
+    const int ov = t->overlap && t->stream2 && !t->op_timing && !t->nan_check;
     seraph_stream_t sw = ov ? t->stream2 : s;
     void* w2 = ov ? t->ws2 : t->ws;
     const size_t w2b = ov ? t->ws2_bytes : t->ws_bytes;
@@ -790,25 +803,27 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         layer_act_t* a = &t->act[l];
 
         /* FFN */
+        /* what leaves the chain at each fork: the weight gradient of the projection, or (LoRA) its adapter's gradients */
         SIDE_FORK();
         if (!lora) WGEMM(t->g_hidden, a->ffn_h, GW + t->L.down, h, f, T);
+        else if (t->LL.A[6] >= 0 &&                                          /* src/train.c:6422-6429 */
+                 lora_backward(t, t->g_hidden, a->ffn_h, LW + t->LL.A[6], LW + t->LL.B[6], LGW + t->LL.A[6], LGW + t->LL.B[6], T, f, h, ov)) return -1.0f;
         SIDE_MARK(MK_DOWN);
         GEMM(t->g_hidden, W + t->L.down, t->g_ffn, T, f, h, 0, 0, 0);
-        if (lora && t->LL.A[6] >= 0 &&                                       /* src/train.c:6422-6429 */
-            lora_backward(t, t->g_hidden, a->ffn_h, LW + t->LL.A[6], LW + t->LL.B[6], LGW + t->LL.A[6], LGW + t->LL.B[6], T, f, h)) return -1.0f;
         SIDE_JOIN(MK_GU);                                                    /* the layer above still reads g_gate / g_up */
-        if (!lora) SIDE_ARM();
+        SIDE_ARM();
         OP("swiglu_backward", 0.0, 20.0 * (double)(T * f), seraph_swiglu_backward(a->gate, a->up, t->g_ffn, t->g_gate, t->g_up, (size_t)(T * f), s));
-        if (lora && t->LL.A[4] >= 0 &&                                       /* src/train.c:6446-6461 */
-            lora_backward(t, t->g_gate, a->xn_ffn, LW + t->LL.A[4], LW + t->LL.B[4], LGW + t->LL.A[4], LGW + t->LL.B[4], T, h, f)) return -1.0f;
-        if (lora && t->LL.A[5] >= 0 &&
-            lora_backward(t, t->g_up, a->xn_ffn, LW + t->LL.A[5], LW + t->LL.B[5], LGW + t->LL.A[5], LGW + t->LL.B[5], T, h, f)) return -1.0f;
+        SIDE_FORK();
         if (!lora) {
             const seraph_gemm_problem_t gu[2] = {{t->g_gate, a->xn_ffn, GW + t->L.gate, f, h}, {t->g_up, a->xn_ffn, GW + t->L.up, f, h}};
-            SIDE_FORK();
             WGEMM_GROUP(gu, 2, T);
-            SIDE_MARK(MK_GU);
+        } else {                                                             /* src/train.c:6446-6461 */
+            if (t->LL.A[4] >= 0 &&
+                lora_backward(t, t->g_gate, a->xn_ffn, LW + t->LL.A[4], LW + t->LL.B[4], LGW + t->LL.A[4], LGW + t->LL.B[4], T, h, f, ov)) return -1.0f;
+            if (t->LL.A[5] >= 0 &&
+                lora_backward(t, t->g_up, a->xn_ffn, LW + t->LL.A[5], LW + t->LL.B[5], LGW + t->LL.A[5], LGW + t->LL.B[5], T, h, f, ov)) return -1.0f;
         }
+        SIDE_MARK(MK_GU);
         {   /* grad_x_norm_ffn = grad_gate Wgate + grad_up Wup (src/train.c:5162-5179) */
             const seraph_gemm_term_t gu[2] = {{t->g_gate, W + t->L.gate, f}, {t->g_up, W + t->L.up, f}};
             GEMM_CHAIN(gu, 2, t->g_xn, T, h);
@@ -822,11 +837,11 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         /* attention */
         SIDE_FORK();
         if (!lora) WGEMM(t->g_hidden, a->attn_out, GW + t->L.o, h, qd, T);
+        else if (t->LL.A[3] >= 0 &&
+                 lora_backward(t, t->g_hidden, a->attn_out, LW + t->LL.A[3], LW + t->LL.B[3], LGW + t->LL.A[3], LGW + t->LL.B[3], T, qd, h, ov)) return -1.0f;
         SIDE_MARK(MK_O);
         GEMM(t->g_hidden, W + t->L.o, t->g_attn, T, qd, h, 0, 0, 0);
         NANCHK(t->g_attn, T * qd, nan_bwd + 5u * (uint32_t)l + 0u);
-        if (lora && t->LL.A[3] >= 0 &&
-            lora_backward(t, t->g_hidden, a->attn_out, LW + t->LL.A[3], LW + t->LL.B[3], LGW + t->LL.A[3], LGW + t->LL.B[3], T, qd, h)) return -1.0f;
         SIDE_JOIN(MK_QKV);                                                   /* the layer above still reads g_q / g_k / g_v */
         /* dK / dV are assigned, so the zero fills of src/train.c:5221-5222 have nothing left to do; the host's copy
          * of the offsets sizes the dS band */
@@ -839,22 +854,22 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
             OP("qk_norm_backward", 0.0, 12.0 * (double)(T * qd), seraph_qk_norm_backward_saved(a->q, a->rms_q, t->g_q, t->g_q, T, H, D, eps, s));
             OP("qk_norm_backward", 0.0, 12.0 * (double)(T * kv), seraph_qk_norm_backward_saved(a->k, a->rms_k, t->g_k, t->g_k, T, KVH, D, eps, s));
         }
-        if (!lora) SIDE_ARM();
+        SIDE_ARM();
         OP("rope", 0.0, 8.0 * (double)(T * (qd + kv)), seraph_rope_qk(t->g_q, t->g_q, H, t->g_k, t->g_k, KVH, starts, batch, T, D, theta, 1, s));
         NANCHK(t->g_q, T * qd, nan_bwd + 5u * (uint32_t)l + 4u);
+        SIDE_FORK();
         if (!lora) {
             const seraph_gemm_problem_t qkv[3] = {{t->g_q, a->xn_attn, GW + t->L.q, qd, h}, {t->g_k, a->xn_attn, GW + t->L.k, kv, h},
                                                   {t->g_v, a->xn_attn, GW + t->L.v, kv, h}};
-            SIDE_FORK();
             WGEMM_GROUP(qkv, 3, T);
-            SIDE_MARK(MK_QKV);
         } else {
             float* gs[3] = {t->g_q, t->g_k, t->g_v};
             int64_t outs[3] = {qd, kv, kv};
             for (int p = 0; p < 3; p++)
                 if (t->LL.A[p] >= 0 &&
-                    lora_backward(t, gs[p], a->xn_attn, LW + t->LL.A[p], LW + t->LL.B[p], LGW + t->LL.A[p], LGW + t->LL.B[p], T, h, outs[p])) return -1.0f;
+                    lora_backward(t, gs[p], a->xn_attn, LW + t->LL.A[p], LW + t->LL.B[p], LGW + t->LL.A[p], LGW + t->LL.B[p], T, h, outs[p], ov)) return -1.0f;
         }
+        SIDE_MARK(MK_QKV);
         {   /* grad_x_norm = grad_q Wq + grad_k Wk + grad_v Wv (src/train.c:5294-5339) */
             const seraph_gemm_term_t qkv[3] = {{t->g_q, W + t->L.q, qd}, {t->g_k, W + t->L.k, kv}, {t->g_v, W + t->L.v, kv}};
             GEMM_CHAIN(qkv, 3, t->g_xn, T, h);

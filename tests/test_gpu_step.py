@@ -156,6 +156,33 @@ def test_weight_gradients_on_the_second_stream_change_no_bit(tr, orc):
     assert np.abs(out[0][1] - p).max() > 0
 
 
+def test_adapter_gradients_on_the_second_stream_change_no_bit(tr, orc):
+    """The LoRA step sends the rank-sized products of every adapter's gradients to the second stream (default); with
+    everything on one stream the same kernels run in another order of launches: adapters, their gradients and moments
+    must be identical over three optimizer steps, with all seven adapter kinds present."""
+    case = dict(hidden=256, layers=3, heads=4, kv_heads=2, head_dim=64, ffn=704, vocab=4096, lora_rank=16,
+                lora_alpha=32.0, lora_mask=0b1111111)
+    ocfg = orc.make_config(**case)
+    cfg = tr.model_config(**case)
+    p = init_params(orc, ocfg, 33)
+    lo = (0.05 * rng(34).standard_normal(orc.lora_param_count(ocfg))).astype(np.float32)
+    starts = np.array([0, 256, 300, 1024], np.int32)
+    toks = [rng(50 + i).integers(0, case["vocab"], 1024).astype(np.int32) for i in range(3)]
+    out = []
+    for overlap in (True, False):
+        t = tr.Trainer(cfg, tr.optim_config(1e-3, warmup_steps=1), max_tokens=1024, max_batch=3)
+        t.enable_wgrad_overlap(overlap)
+        t.upload(tr.PARAMS, p)
+        t.upload(tr.LORA_PARAMS, lo)
+        losses = [t.step(tok, starts) for tok in toks]
+        out.append((losses, t.download(tr.LORA_PARAMS), t.download(tr.LORA_GRADS), t.download(tr.LORA_V)))
+        t.close()
+    assert out[0][0] == out[1][0]
+    for a, b in zip(out[0][1:], out[1][1:]):
+        assert np.array_equal(a, b)
+    assert np.abs(out[0][1] - lo).max() > 0
+
+
 @pytest.mark.parametrize("mask", [0b0001111, 0b1111111, 0b1010101])
 @pytest.mark.parametrize("b_zero", [True, False])
 def test_lora_step(tr, orc, b_zero, mask):
