@@ -763,10 +763,20 @@ static bool use_smallk(const float* A, const float* B, const float* C, int64_t M
            (!A || (aligned16(A) && aligned16(B) && aligned16(C)));
 }
 
-// Fewer 64x64 tiles than compute units and a K long enough to be worth splitting between waves.
+// 32x32 tiles whose four waves share out every K stage, instead of 64x64 tiles.  Always when there are fewer 64x64
+// tiles than compute units.  Beyond that the small-tile kernel (four workgroups per CU, so a CU's last tiles still
+// overlap each other's ramps) keeps winning while a CU would see only a few 64x64 tiles: measured on 2048 x 512 ...
+// 2816 x 1024 outputs in all orientations, 352 tiles 55 against 75 us at K 2048 and 19 against 21 us at K 512, 512
+// tiles 74 against 81 us (K 2048) but 24 against 22 us (K 512), 704 tiles 100 against 107 us (K 2048) and 31 against
+// 30 us (K 512); from 1024 tiles on the 128x128 kernel is ahead of both.
+static bool small_tiles_pay(int64_t t64, int64_t K) {
+    const int64_t cus = num_compute_units();
+    if (t64 < cus) return true;
+    if (K >= 1024) return t64 < 4 * cus;
+    return t64 > cus && 4 * t64 < 7 * cus;
+}
 static bool use_splitk(int64_t M, int64_t N, int64_t K, int tA, int tB) {
-    return !use_big_tiles(M, N) && ceil_div(M, 64) * ceil_div(N, 64) < num_compute_units() && K >= 256 &&
-           pipelined_ok(M, N, K, tA, tB);
+    return !use_big_tiles(M, N) && K >= 256 && small_tiles_pay(ceil_div(M, 64) * ceil_div(N, 64), K) && pipelined_ok(M, N, K, tA, tB);
 }
 
 extern "C" const char* seraph_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int transpose_A, int transpose_B) {
@@ -849,8 +859,7 @@ static int group_tile(const seraph_gemm_problem_t* p, int count, int64_t K, int 
     }
     if (t32 > 0x7fffffff) return 0;
     if (big_tiles_pay(t128, t64)) return 128;
-    if (t64 >= num_compute_units() || K < 256) return 64;
-    return 32;
+    return (K >= 256 && small_tiles_pay(t64, K)) ? 32 : 64;
 }
 
 extern "C" const char* seraph_gemm_grouped_kernel_name(const seraph_gemm_problem_t* problems, int count, int64_t K,
@@ -919,7 +928,8 @@ static bool chain_ok(const seraph_gemm_term_t* t, int count, const float* C, int
         if (!pipelined_ok(M, N, K, tA, tB)) return false;
         ksum += K;
     }
-    return !use_splitk(M, N, ksum, tA, tB);
+    // (no 32x32 form of the sum: with fewer 64x64 tiles than compute units the products run one after the other)
+    return ksum < 256 || use_big_tiles(M, N) || ceil_div(M, 64) * ceil_div(N, 64) >= num_compute_units();
 }
 
 extern "C" const char* seraph_gemm_chain_kernel_name(const seraph_gemm_term_t* terms, int count, const float* C, int64_t M, int64_t N,
