@@ -108,6 +108,31 @@ def run_full_case(tr, orc, c, starts, lr, clip, seed):
 C1 = dict(hidden=512, layers=8, heads=8, kv_heads=8, head_dim=64, ffn=1408, vocab=8192, rms_eps=1e-6, rope_theta=10000.0)
 
 
+def test_33m_model_hundred_steps_identical_on_one_and_two_streams(tr):
+    """The 33M model's step runs its weight gradients on a second stream, ordered by events that the producing
+    kernels complete themselves.  A hundred optimizer steps with and without the second stream: every loss, the weights
+    and the second moments agree to the bit (one ordering edge too few would let a product read or overwrite a buffer
+    early, sooner or later), and the loss falls on the eight batches it keeps seeing."""
+    cfg = tr.model_config(**C1)
+    n = tr.param_count(cfg)
+    p = seeded_params(C1, n, 3)
+    starts = np.arange(0, 2049, 256, dtype=np.int32)
+    toks = [np.random.default_rng(100 + i).integers(0, C1["vocab"], 2048).astype(np.int32) for i in range(8)]
+    res = []
+    for overlap in (True, False):
+        t = tr.Trainer(cfg, tr.optim_config(3e-4, warmup_steps=1), max_tokens=2048, max_batch=8)
+        try:
+            t.enable_wgrad_overlap(overlap)
+            t.upload(tr.PARAMS, p)
+            losses = np.array([t.step(toks[i % 8], starts) for i in range(100)])
+            res.append((losses, t.download(tr.PARAMS), t.download(tr.ADAM_V)))
+        finally:
+            t.close()
+    for a, b in zip(res[0], res[1]):
+        assert np.array_equal(a, b)
+    assert np.isfinite(res[0][0]).all() and res[0][0][-1] < res[0][0][0] - 1.0
+
+
 @pytest.mark.parametrize("clip", [0.0, 1.0])
 def test_33m_model_step_8_x_256(tr, orc, clip):
     """The 33M configuration exactly; clip 0 is the reference's AdamW, clip 1.0 the configuration's clipped variant."""
