@@ -29,6 +29,7 @@ typedef struct { int64_t A[7], B[7], in[7], out[7], stride; } lora_layout_t;   /
 typedef struct {
     float *layer_in, *xn_attn, *q, *k, *v, *attn_out, *lse, *post_in, *xn_ffn, *gate, *up, *ffn_h;
     float *rms_q, *rms_k;        /* per token, with use_qk_norm */
+    float* xa[7];                /* LoRA: scale * x A^T of each adapter present, kept for the backward */
 } layer_act_t;
 
 struct hip_trainer {
@@ -341,8 +342,11 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
         const size_t T = (size_t)max_tokens, h = (size_t)cfg->hidden, f = (size_t)cfg->ffn, Vv = (size_t)cfg->vocab;
         const size_t qd = (size_t)cfg->heads * cfg->head_dim, kv = (size_t)cfg->kv_heads * cfg->head_dim;
         const size_t r = cfg->lora_rank > 0 ? (size_t)cfg->lora_rank : 1;
+        size_t adapters = 0;
+        for (int q = 0; q < 7; q++) adapters += t->LL.A[q] >= 0 ? 1 : 0;
         const size_t per_layer = 4 * up256(T * h * 4) + 2 * up256(T * qd * 4) + 2 * up256(T * kv * 4) +
-                                 up256(T * cfg->heads * 4) + 3 * up256(T * f * 4) + (cfg->use_qk_norm ? 2 * up256(T * 4) : 0);
+                                 up256(T * cfg->heads * 4) + 3 * up256(T * f * 4) + (cfg->use_qk_norm ? 2 * up256(T * 4) : 0) +
+                                 adapters * up256(T * r * 4);
         const size_t rest = 2 * up256(T * h * 4) + up256(T * Vv * 4) + 3 * up256(T * 4) + up256(T * h * 4) + 2 * up256(T * r * 4) +
                             3 * up256(T * h * 4) + 3 * up256(T * f * 4) + 2 * up256(T * qd * 4) + 2 * up256(T * kv * 4) +
                             up256(h * 4) + 2 * up256(T * 4) + up256(((size_t)max_batch + 1) * 4);
@@ -359,6 +363,7 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
             TAKE(a->lse, T * cfg->heads * 4);
             if (cfg->use_qk_norm) { TAKE(a->rms_q, T * 4); TAKE(a->rms_k, T * 4); }
             TAKE(a->gate, T * f * 4); TAKE(a->up, T * f * 4); TAKE(a->ffn_h, T * f * 4);
+            for (int q = 0; q < 7; q++) if (t->LL.A[q] >= 0) TAKE(a->xa[q], T * r * 4);
         }
         TAKE(t->final_in, T * h * 4); TAKE(t->xn_final, T * h * 4); TAKE(t->logits, T * Vv * 4);
         TAKE(t->loss_rows, T * 4); TAKE(t->red_a, T * 4); TAKE(t->red_b, T * 4);
@@ -510,19 +515,21 @@ int hip_trainer_op_stats(const hip_trainer_t* t, hip_op_stat_t* out, int max) {
 
 /* ------------------------------------------------------------------ the step */
 /* out (+)= ((x A^T) s) B^T, src/train.c:5778-5796 */
+/* xa receives (x A^T) s and stays: the backward's first product (src/train.c:5815-5822) is this same one */
 static int lora_forward_add(hip_trainer_t* t, const float* x, float* out, const float* A, const float* B,
-                            int64_t T, int64_t in, int64_t outd) {
+                            int64_t T, int64_t in, int64_t outd, float* xa) {
     const int r = t->cfg.lora_rank;
     const float s = t->cfg.lora_alpha / (float)r;
-    GEMM_SCALED(x, A, t->lora_tmp, T, r, in, 0, 1, 0, s);
-    GEMM(t->lora_tmp, B, out, T, outd, r, 0, 1, 1);
+    GEMM_SCALED(x, A, xa, T, r, in, 0, 1, 0, s);
+    GEMM(xa, B, out, T, outd, r, 0, 1, 1);
     return 0;
 }
 
-/* src/train.c:5803-5845 with grad_input == NULL, as every call site passes it */
+/* src/train.c:5803-5845 with grad_input == NULL, as every call site passes it; (x A^T) s comes from the forward (xa)
+ * instead of being formed again */
 /* The four products are rank-sized and nothing on the chain of input gradients reads their results, so the step may
  * run them on its second stream (side != 0: that stream's scratch and its own tmp). */
-static int lora_backward(hip_trainer_t* t, const float* dY, const float* x, const float* A, const float* B,
+static int lora_backward(hip_trainer_t* t, const float* dY, const float* x, const float* xa, const float* B,
                          float* gA, float* gB, int64_t T, int64_t in, int64_t outd, int side) {
     const int r = t->cfg.lora_rank;
     const float s = t->cfg.lora_alpha / (float)r;
@@ -533,8 +540,7 @@ static int lora_backward(hip_trainer_t* t, const float* dY, const float* x, cons
 #define LGEMM(A_, B_, C_, M_, N_, K_, tA_, tB_, acc_, alpha_)                                          \
     OP("gemm_scaled", 2.0 * (double)(M_) * (double)(N_) * (double)(K_), 0.0,                           \
        seraph_gemm_scaled((A_), (B_), (C_), (M_), (N_), (K_), (tA_), (tB_), (acc_), (alpha_), ws, wsb, st))
-    LGEMM(x, A, tmp, T, r, in, 0, 1, 0, s);
-    LGEMM(dY, tmp, gB, outd, r, T, 1, 0, 1, 1.0f);
+    LGEMM(dY, xa, gB, outd, r, T, 1, 0, 1, 1.0f);
     LGEMM(dY, B, tmp, T, r, outd, 0, 0, 0, s);
     LGEMM(tmp, x, gA, r, in, T, 1, 0, 1, 1.0f);
 #undef LGEMM
@@ -721,9 +727,9 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
                                                   {a->xn_attn, W + t->L.v, a->v, T, kv}};
             GEMM_GROUP(qkv, 3, h, 0, 1, 0);
         }
-        if (lora && t->LL.A[0] >= 0 && lora_forward_add(t, a->xn_attn, a->q, LW + t->LL.A[0], LW + t->LL.B[0], T, h, qd)) return -1.0f;
-        if (lora && t->LL.A[1] >= 0 && lora_forward_add(t, a->xn_attn, a->k, LW + t->LL.A[1], LW + t->LL.B[1], T, h, kv)) return -1.0f;
-        if (lora && t->LL.A[2] >= 0 && lora_forward_add(t, a->xn_attn, a->v, LW + t->LL.A[2], LW + t->LL.B[2], T, h, kv)) return -1.0f;
+        if (lora && t->LL.A[0] >= 0 && lora_forward_add(t, a->xn_attn, a->q, LW + t->LL.A[0], LW + t->LL.B[0], T, h, qd, a->xa[0])) return -1.0f;
+        if (lora && t->LL.A[1] >= 0 && lora_forward_add(t, a->xn_attn, a->k, LW + t->LL.A[1], LW + t->LL.B[1], T, h, kv, a->xa[1])) return -1.0f;
+        if (lora && t->LL.A[2] >= 0 && lora_forward_add(t, a->xn_attn, a->v, LW + t->LL.A[2], LW + t->LL.B[2], T, h, kv, a->xa[2])) return -1.0f;
         OP("rope", 0.0, 8.0 * (double)(T * (qd + kv)), seraph_rope_qk(a->q, a->q, H, a->k, a->k, KVH, starts, batch, T, D, theta, 0, s));
         if (c->use_qk_norm) {                                              /* after RoPE, before the attention: src/train.c:4687-4689 */
             OP("qk_norm", 0.0, 8.0 * (double)(T * qd), seraph_qk_norm_saved(a->q, a->rms_q, T, H, D, eps, s));
@@ -731,17 +737,17 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         }
         OP("attention_forward", 4.0 * D * t->attn_pairs * H, 0.0, seraph_attention_forward(a->q, a->k, a->v, a->attn_out, a->lse, starts, batch, T, H, KVH, D, scale, s));
         GEMM(a->attn_out, W + t->L.o, t->tmp_h, T, h, qd, 0, 1, 0);
-        if (lora && t->LL.A[3] >= 0 && lora_forward_add(t, a->attn_out, t->tmp_h, LW + t->LL.A[3], LW + t->LL.B[3], T, qd, h)) return -1.0f;
+        if (lora && t->LL.A[3] >= 0 && lora_forward_add(t, a->attn_out, t->tmp_h, LW + t->LL.A[3], LW + t->LL.B[3], T, qd, h, a->xa[3])) return -1.0f;
         OP("add_rmsnorm", 0.0, 16.0 * (double)(T * h), seraph_add_rmsnorm(a->layer_in, t->tmp_h, a->post_in, W + t->L.post_norm, a->xn_ffn, T, h, eps, s));
         {   /* gate and up projections (src/train.c:4718-4725) as one launch */
             const seraph_gemm_problem_t gu[2] = {{a->xn_ffn, W + t->L.gate, a->gate, T, f}, {a->xn_ffn, W + t->L.up, a->up, T, f}};
             GEMM_GROUP(gu, 2, h, 0, 1, 0);
         }
-        if (lora && t->LL.A[4] >= 0 && lora_forward_add(t, a->xn_ffn, a->gate, LW + t->LL.A[4], LW + t->LL.B[4], T, h, f)) return -1.0f;
-        if (lora && t->LL.A[5] >= 0 && lora_forward_add(t, a->xn_ffn, a->up, LW + t->LL.A[5], LW + t->LL.B[5], T, h, f)) return -1.0f;
+        if (lora && t->LL.A[4] >= 0 && lora_forward_add(t, a->xn_ffn, a->gate, LW + t->LL.A[4], LW + t->LL.B[4], T, h, f, a->xa[4])) return -1.0f;
+        if (lora && t->LL.A[5] >= 0 && lora_forward_add(t, a->xn_ffn, a->up, LW + t->LL.A[5], LW + t->LL.B[5], T, h, f, a->xa[5])) return -1.0f;
         OP("swiglu", 0.0, 12.0 * (double)(T * f), seraph_swiglu(a->gate, a->up, a->ffn_h, (size_t)(T * f), s));
         GEMM(a->ffn_h, W + t->L.down, t->tmp_h, T, h, f, 0, 1, 0);
-        if (lora && t->LL.A[6] >= 0 && lora_forward_add(t, a->ffn_h, t->tmp_h, LW + t->LL.A[6], LW + t->LL.B[6], T, f, h)) return -1.0f;
+        if (lora && t->LL.A[6] >= 0 && lora_forward_add(t, a->ffn_h, t->tmp_h, LW + t->LL.A[6], LW + t->LL.B[6], T, f, h, a->xa[6])) return -1.0f;
         /* residual add and the norm that reads its result: the next layer's input norm, or the final norm */
         const float* next_gain = (l + 1 < NL) ? P + t->off_layer0 + t->L.stride * (l + 1) + t->L.in_norm : P + t->off_final_norm;
         float* next_xn = (l + 1 < NL) ? t->act[l + 1].xn_attn : t->xn_final;
@@ -807,7 +813,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         SIDE_FORK();
         if (!lora) WGEMM(t->g_hidden, a->ffn_h, GW + t->L.down, h, f, T);
         else if (t->LL.A[6] >= 0 &&                                          /* src/train.c:6422-6429 */
-                 lora_backward(t, t->g_hidden, a->ffn_h, LW + t->LL.A[6], LW + t->LL.B[6], LGW + t->LL.A[6], LGW + t->LL.B[6], T, f, h, ov)) return -1.0f;
+                 lora_backward(t, t->g_hidden, a->ffn_h, a->xa[6], LW + t->LL.B[6], LGW + t->LL.A[6], LGW + t->LL.B[6], T, f, h, ov)) return -1.0f;
         SIDE_MARK(MK_DOWN);
         GEMM(t->g_hidden, W + t->L.down, t->g_ffn, T, f, h, 0, 0, 0);
         SIDE_JOIN(MK_GU);                                                    /* the layer above still reads g_gate / g_up */
@@ -819,9 +825,9 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
             WGEMM_GROUP(gu, 2, T);
         } else {                                                             /* src/train.c:6446-6461 */
             if (t->LL.A[4] >= 0 &&
-                lora_backward(t, t->g_gate, a->xn_ffn, LW + t->LL.A[4], LW + t->LL.B[4], LGW + t->LL.A[4], LGW + t->LL.B[4], T, h, f, ov)) return -1.0f;
+                lora_backward(t, t->g_gate, a->xn_ffn, a->xa[4], LW + t->LL.B[4], LGW + t->LL.A[4], LGW + t->LL.B[4], T, h, f, ov)) return -1.0f;
             if (t->LL.A[5] >= 0 &&
-                lora_backward(t, t->g_up, a->xn_ffn, LW + t->LL.A[5], LW + t->LL.B[5], LGW + t->LL.A[5], LGW + t->LL.B[5], T, h, f, ov)) return -1.0f;
+                lora_backward(t, t->g_up, a->xn_ffn, a->xa[5], LW + t->LL.B[5], LGW + t->LL.A[5], LGW + t->LL.B[5], T, h, f, ov)) return -1.0f;
         }
         SIDE_MARK(MK_GU);
         {   /* grad_x_norm_ffn = grad_gate Wgate + grad_up Wup (src/train.c:5162-5179) */
@@ -838,7 +844,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         SIDE_FORK();
         if (!lora) WGEMM(t->g_hidden, a->attn_out, GW + t->L.o, h, qd, T);
         else if (t->LL.A[3] >= 0 &&
-                 lora_backward(t, t->g_hidden, a->attn_out, LW + t->LL.A[3], LW + t->LL.B[3], LGW + t->LL.A[3], LGW + t->LL.B[3], T, qd, h, ov)) return -1.0f;
+                 lora_backward(t, t->g_hidden, a->attn_out, a->xa[3], LW + t->LL.B[3], LGW + t->LL.A[3], LGW + t->LL.B[3], T, qd, h, ov)) return -1.0f;
         SIDE_MARK(MK_O);
         GEMM(t->g_hidden, W + t->L.o, t->g_attn, T, qd, h, 0, 0, 0);
         NANCHK(t->g_attn, T * qd, nan_bwd + 5u * (uint32_t)l + 0u);
@@ -867,7 +873,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
             int64_t outs[3] = {qd, kv, kv};
             for (int p = 0; p < 3; p++)
                 if (t->LL.A[p] >= 0 &&
-                    lora_backward(t, gs[p], a->xn_attn, LW + t->LL.A[p], LW + t->LL.B[p], LGW + t->LL.A[p], LGW + t->LL.B[p], T, h, outs[p], ov)) return -1.0f;
+                    lora_backward(t, gs[p], a->xn_attn, a->xa[p], LW + t->LL.B[p], LGW + t->LL.A[p], LGW + t->LL.B[p], T, h, outs[p], ov)) return -1.0f;
         }
         SIDE_MARK(MK_QKV);
         {   /* grad_x_norm = grad_q Wq + grad_k Wk + grad_v Wv (src/train.c:5294-5339) */
