@@ -119,7 +119,17 @@ struct TileQueue {
     unsigned int* q;        // q[0] next item, q[1] workgroups finished
     int* slot;              // one int of LDS
     int total;
-    __device__ __forceinline__ int next() const {
+    int drawn = 0;
+    // A launch with no more workgroups than items' worth of residency gets exactly one workgroup per item
+    // (persistent_grid): the item is then the workgroup's index and the counters stay untouched, which
+    // saves the two round trips of the atomics, the whole cost of the queue for a short item.
+    __device__ __forceinline__ bool one_each() const { return total <= (int)gridDim.x; }
+    __device__ __forceinline__ int next() {
+        if (one_each()) {
+            const int item = drawn ? -1 : (int)blockIdx.x;
+            drawn = 1;
+            return item < total ? item : -1;
+        }
         if (threadIdx.x == 0) *slot = (int)atomicAdd(&q[0], 1u);
         __syncthreads();
         const int item = __builtin_amdgcn_readfirstlane(*slot);    // the same for every lane: keep it, and what follows from it, scalar
@@ -127,6 +137,7 @@ struct TileQueue {
         return item < total ? item : -1;
     }
     __device__ __forceinline__ void leave() const {
+        if (one_each()) return;
         if (threadIdx.x == 0 && atomicAdd(&q[1], 1u) == gridDim.x - 1) {
             q[0] = 0u;
             q[1] = 0u;
@@ -229,7 +240,7 @@ __global__ __launch_bounds__(kAttnThreads, (KSPLIT ? 1 : 2)) void attn_fwd_kerne
     __shared__ int sItem;
     const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
     const int nqt = (int)((T + QROWS - 1) / QROWS);
-    const TileQueue tq_{queue, &sItem, nqt * H};
+    TileQueue tq_{queue, &sItem, nqt * H};
     __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
     // key tiles a query tile runs over: from the start of its first query's sequence to its last query
     const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, [&](int q) {
@@ -475,7 +486,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
     // iterations of each (key tile, kv head) round-robin to that many work items; each writes its partial
     // dK/dV to its own slice of partK/partV and a second kernel adds the slices in a fixed order.
     const int nkt = (int)((T + 127) / 128);
-    const TileQueue tq_{queue, &sItem, nkt * KVH * split};
+    TileQueue tq_{queue, &sItem, nkt * KVH * split};
     __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
     // query tiles a 128-key tile is visible to: up to the end of its last key's sequence
     const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nkt, false, [&](int k) {
@@ -1103,7 +1114,7 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dq_k
     __shared__ int sItem;
     const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
     const int nqt = (int)((T + 127) / 128);
-    const TileQueue tq_{queue, &sItem, nqt * H};
+    TileQueue tq_{queue, &sItem, nqt * H};
     __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
     const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, [&](int q) {
         const int64_t a = (int64_t)q * 128, z = (a + 127 < T - 1) ? a + 127 : T - 1;
@@ -1222,7 +1233,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const f
     const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
     const int nqt = (int)((T + QROWS - 1) / QROWS);
     const int64_t nqt32 = (T + 31) >> 5;
-    const TileQueue tq_{queue, &sItem, nqt * H};
+    TileQueue tq_{queue, &sItem, nqt * H};
     __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
     const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, [&](int q) {
         const int64_t a = (int64_t)q * QROWS, z = (a + QROWS - 1 < T - 1) ? a + QROWS - 1 : T - 1;
