@@ -125,17 +125,25 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const float* __rest
         gs[k] = make_float4(0, 0, 0, 0);
     }
 
-    for (int64_t row = wave; row < rows; row += nwaves) {
-        const float4* xr = reinterpret_cast<const float4*>(x + row * cols);
-        const float4* gr = reinterpret_cast<const float4*>(dy + row * cols);
-        float4 xv[VPL], gv[VPL], rv[VPL];
+    // The next row is requested before the current one is reduced: a wave has few rows (two at 2048 x 512), and
+    // without this each pays the full memory latency in turn.
+    float4 xv[VPL], gv[VPL], rv[VPL];
+    auto request = [&](int64_t row, float4* xo, float4* go, float4* ro) {
+        const bool live = row < rows;
+        const int64_t at = live ? row * cols : 0;
 #pragma unroll
         for (int k = 0; k < VPL; k++) {
-            int i4 = lane + 64 * k;
-            xv[k] = i4 < n4 ? xr[i4] : make_float4(0, 0, 0, 0);
-            gv[k] = i4 < n4 ? gr[i4] : make_float4(0, 0, 0, 0);
-            rv[k] = (res && i4 < n4) ? reinterpret_cast<const float4*>(res + row * cols)[i4] : make_float4(0, 0, 0, 0);
+            const int i4 = lane + 64 * k;
+            const bool in = live && i4 < n4;
+            xo[k] = in ? reinterpret_cast<const float4*>(x + at)[i4] : make_float4(0, 0, 0, 0);
+            go[k] = in ? reinterpret_cast<const float4*>(dy + at)[i4] : make_float4(0, 0, 0, 0);
+            ro[k] = (res && in) ? reinterpret_cast<const float4*>(res + at)[i4] : make_float4(0, 0, 0, 0);
         }
+    };
+    request(wave, xv, gv, rv);
+    for (int64_t row = wave; row < rows; row += nwaves) {
+        float4 xn[VPL], gn[VPL], rn[VPL];
+        request(row + nwaves, xn, gn, rn);
         double ssq = 0.0, cp = 0.0;
 #pragma unroll
         for (int k = 0; k < VPL; k++) {
@@ -164,6 +172,8 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const float* __rest
             }
             if (i4 < n4) dr[i4] = make_float4(rv[k].x + o[0], rv[k].y + o[1], rv[k].z + o[2], rv[k].w + o[3]);
         }
+#pragma unroll
+        for (int k = 0; k < VPL; k++) { xv[k] = xn[k]; gv[k] = gn[k]; rv[k] = rn[k]; }
     }
 
     // combine the block's waves, then one partial row per block
