@@ -223,6 +223,18 @@ int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy,
 int seraph_rmsnorm_backward_residual(const float* x, const float* scale, const float* dy, const float* residual, float* dx,
                                      float* grad_scale, int64_t rows, int64_t cols, float eps, void* ws, size_t ws_bytes,
                                      seraph_stream_t s);
+/* seraph_rmsnorm_backward_residual in two halves, for a step driver whose norms are small enough that the launch of
+ * each column sum counts (the 2 L + 1 vulkan_rmsnorm_backward_batch calls of src/train.c:5071-5355): the row pass
+ * completes dx and leaves *nparts partial rows of cols floats at the start of ws; seraph_rmsnorm_colsum_multi later
+ * adds the column sums of any number of such passes of one width into their grad_scale in one launch, each summed in
+ * the order seraph_rmsnorm_backward_residual uses, so the results are the same bits.  ws must stay untouched between
+ * the two calls; `jobs` is a HOST array.  A caller that has no use for grad_scale (frozen norms) calls the row pass
+ * alone. */
+int seraph_rmsnorm_backward_rows(const float* x, const float* scale, const float* dy, const float* residual, float* dx,
+                                 int64_t rows, int64_t cols, float eps, void* ws, size_t ws_bytes, int* nparts,
+                                 seraph_stream_t s);
+typedef struct { const float* partial; int nparts; float* grad_scale; } seraph_colsum_job_t;
+int seraph_rmsnorm_colsum_multi(const seraph_colsum_job_t* jobs, int count, int64_t cols, seraph_stream_t s);
 /* seraph_rmsnorm_backward_residual for callers that cannot allocate device memory or bring a workspace
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  The partial rows of the column reduction live in an array built into the

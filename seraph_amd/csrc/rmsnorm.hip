@@ -350,8 +350,8 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_generic_kernel(const float
 // allows 16-byte loads (a lane takes four columns of rows g, g + 64, ..., all loads in flight, added in double in row
 // order; the 64 group sums are then combined in group order), else 64 columns x 16 row groups with scalar loads.
 template <bool VEC>
-__global__ __launch_bounds__(1024) void colsum_add_kernel(const float* __restrict__ partial, int nparts,
-                                                           int64_t cols, float* __restrict__ grad_scale) {
+__device__ __forceinline__ void colsum_add_body(const float* __restrict__ partial, int nparts,
+                                                int64_t cols, float* __restrict__ grad_scale) {
     constexpr int GROUPS = VEC ? 64 : 16;
     __shared__ double part[GROUPS][64];
     double t4[4] = {0.0, 0.0, 0.0, 0.0};
@@ -402,6 +402,26 @@ __global__ __launch_bounds__(1024) void colsum_add_kernel(const float* __restric
             grad_scale[c] = (float)((double)grad_scale[c] + t);
         }
     }
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(1024) void colsum_add_kernel(const float* __restrict__ partial, int nparts,
+                                                           int64_t cols, float* __restrict__ grad_scale) {
+    colsum_add_body<VEC>(partial, nparts, cols, grad_scale);
+}
+
+// The column sums of several backward passes of one width in one launch (grid y = the pass): a step driver whose
+// norms are small lets their partial rows lie until the end of its backward and folds them all here, which takes
+// one launch per norm off its chain of dependent kernels.  Each pass is summed exactly as colsum_add_kernel does it.
+constexpr int kMaxColsumJobs = 64;
+struct ColsumJobs {
+    const float* partial[kMaxColsumJobs];
+    float* grad_scale[kMaxColsumJobs];
+    int nparts[kMaxColsumJobs];
+};
+template <bool VEC>
+__global__ __launch_bounds__(1024) void colsum_add_multi_kernel(ColsumJobs jobs, int64_t cols) {
+    colsum_add_body<VEC>(jobs.partial[blockIdx.y], jobs.nparts[blockIdx.y], cols, jobs.grad_scale[blockIdx.y]);
 }
 
 // ---------------------------------------------------------------- qk_norm
@@ -644,11 +664,12 @@ int seraph_rmsnorm_backward(const float* x, const float* scale, const float* dy,
 }
 
 // Launches of the backward on checked arguments; `partial` holds seraph_rmsnorm_backward_ws_bytes(rows, cols).
+// With nparts_out the column sum is left out: the partial rows stay in `partial` and their number is reported.
 static int rmsnorm_backward_launch(const float* x, const float* scale, const float* dy, const float* res, float* dx,
                                    float* grad_scale, int64_t rows, int64_t cols, float eps, float* partial,
-                                   seraph_stream_t s) {
+                                   seraph_stream_t s, int* nparts_out = nullptr) {
     hipStream_t st = as_stream(s);
-    const hipEvent_t done = take_armed_event();                 // belongs to the column sum, the last launch
+    const hipEvent_t done = take_armed_event();                 // belongs to the last launch: the column sum, or the row pass alone
     const bool aligned = aligned16(x) && aligned16(scale) && aligned16(dy) && aligned16(dx) && aligned16(partial) && (!res || aligned16(res));
     const int bvpl = aligned ? pick_block_vpl(cols) : 0;
     const int wvpl = (aligned && !bvpl && cols <= 512) ? pick_vpl(cols) : 0;
@@ -656,7 +677,8 @@ static int rmsnorm_backward_launch(const float* x, const float* scale, const flo
     if (bvpl) {
         const int grid = bwd_block_grid(rows);
         nparts = grid;
-#define BBWD(V) hipLaunchKernelGGL((rmsnorm_bwd_block_kernel<V, 0>), dim3(grid), dim3(kBlock), 0, st, x, scale, dy, res, dx, partial, rows, (int)cols, eps)
+        if (nparts_out) arm_event(done);
+#define BBWD(V) SERAPH_LAUNCH_LAST((rmsnorm_bwd_block_kernel<V, 0>), dim3(grid), dim3(kBlock), 0, st, x, scale, dy, res, dx, partial, rows, (int)cols, eps)
         switch (bvpl) {
             case 1: BBWD(1); break;
             case 2: BBWD(2); break;
@@ -668,7 +690,8 @@ static int rmsnorm_backward_launch(const float* x, const float* scale, const flo
         const int grid = bwd_grid(rows);
         nparts = grid;
         const size_t lds = (size_t)kWavesPerBlock * cols * sizeof(float);
-#define BWD(V) hipLaunchKernelGGL(rmsnorm_bwd_kernel<V>, dim3(grid), dim3(kBlock), lds, st, x, scale, dy, res, dx, partial, rows, (int)cols, eps)
+        if (nparts_out) arm_event(done);
+#define BWD(V) SERAPH_LAUNCH_LAST(rmsnorm_bwd_kernel<V>, dim3(grid), dim3(kBlock), lds, st, x, scale, dy, res, dx, partial, rows, (int)cols, eps)
         if (wvpl == 1) BWD(1); else BWD(2);
 #undef BWD
     } else {
@@ -676,9 +699,11 @@ static int rmsnorm_backward_launch(const float* x, const float* scale, const flo
         nparts = grid * kWavesPerBlock;
         int rc = seraph_fill_u32(partial, 0u, (size_t)nparts * cols, s);
         if (rc != SERAPH_OK) return rc;
-        hipLaunchKernelGGL(rmsnorm_bwd_generic_kernel, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, res, dx, partial, rows, cols, eps);
+        if (nparts_out) arm_event(done);
+        SERAPH_LAUNCH_LAST(rmsnorm_bwd_generic_kernel, dim3(grid), dim3(kBlock), 0, st, x, scale, dy, res, dx, partial, rows, cols, eps);
     }
     SERAPH_LAUNCH_CHECK();
+    if (nparts_out) { *nparts_out = nparts; return SERAPH_OK; }
     arm_event(done);
     if (cols % 4 == 0 && aligned16(partial))
         SERAPH_LAUNCH_LAST(colsum_add_kernel<true>, dim3((unsigned)ceil_div(cols, 64)), dim3(1024), 0, st, partial, nparts, cols, grad_scale);
@@ -699,6 +724,48 @@ int seraph_rmsnorm_backward_residual(const float* x, const float* scale, const f
         return SERAPH_ERR_WORKSPACE;
     }
     return rmsnorm_backward_launch(x, scale, dy, residual, dx, grad_scale, rows, cols, eps, (float*)ws, s);
+}
+
+int seraph_rmsnorm_backward_rows(const float* x, const float* scale, const float* dy, const float* residual, float* dx,
+                                 int64_t rows, int64_t cols, float eps, void* ws, size_t ws_bytes, int* nparts,
+                                 seraph_stream_t s) {
+    SERAPH_REQUIRE(nparts, "rmsnorm_backward_rows: NULL pointer");
+    *nparts = 0;
+    if (rows == 0 || cols == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(x && scale && dy && dx, "rmsnorm_backward_rows: NULL pointer");
+    SERAPH_REQUIRE(rows > 0 && cols > 0, "rmsnorm_backward_rows: bad shape");
+    if (!ws || ws_bytes < seraph_rmsnorm_backward_ws_bytes(rows, cols)) {
+        set_error("rmsnorm_backward_rows: scratch of %zu bytes required", seraph_rmsnorm_backward_ws_bytes(rows, cols));
+        return SERAPH_ERR_WORKSPACE;
+    }
+    return rmsnorm_backward_launch(x, scale, dy, residual, dx, nullptr, rows, cols, eps, (float*)ws, s, nparts);
+}
+
+int seraph_rmsnorm_colsum_multi(const seraph_colsum_job_t* jobs, int count, int64_t cols, seraph_stream_t s) {
+    if (count == 0 || cols == 0) return SERAPH_OK;
+    SERAPH_REQUIRE(jobs && count > 0 && cols > 0, "rmsnorm_colsum_multi: bad arguments");
+    bool vec = cols % 4 == 0;
+    for (int i = 0; i < count; i++) {
+        SERAPH_REQUIRE(jobs[i].partial && jobs[i].grad_scale && jobs[i].nparts >= 0, "rmsnorm_colsum_multi: job %d is incomplete", i);
+        vec = vec && aligned16(jobs[i].partial);
+    }
+    hipStream_t st = as_stream(s);
+    for (int at = 0; at < count; at += kMaxColsumJobs) {
+        const int n = count - at < kMaxColsumJobs ? count - at : kMaxColsumJobs;
+        ColsumJobs j;
+        for (int i = 0; i < n; i++) { j.partial[i] = jobs[at + i].partial; j.grad_scale[i] = jobs[at + i].grad_scale; j.nparts[i] = jobs[at + i].nparts; }
+        for (int i = n; i < kMaxColsumJobs; i++) { j.partial[i] = nullptr; j.grad_scale[i] = nullptr; j.nparts[i] = 0; }
+        const dim3 grid((unsigned)ceil_div(cols, 64), (unsigned)n);
+        if (at + n < count) {
+            if (vec) hipLaunchKernelGGL(colsum_add_multi_kernel<true>, grid, dim3(1024), 0, st, j, cols);
+            else hipLaunchKernelGGL(colsum_add_multi_kernel<false>, grid, dim3(1024), 0, st, j, cols);
+        } else {
+            if (vec) SERAPH_LAUNCH_LAST(colsum_add_multi_kernel<true>, grid, dim3(1024), 0, st, j, cols);
+            else SERAPH_LAUNCH_LAST(colsum_add_multi_kernel<false>, grid, dim3(1024), 0, st, j, cols);
+        }
+        SERAPH_LAUNCH_CHECK();
+    }
+    return SERAPH_OK;
 }
 
 size_t seraph_rmsnorm_backward_static_max_bytes(void) { return kStaticScratchBytes; }

@@ -225,6 +225,30 @@ def rmsnorm_backward(x, scale, dy, eps, grad_scale=None, residual=None, out=None
     return dx, gs
 
 
+class ColsumJob(C.Structure):
+    _fields_ = [("partial", C.c_void_p), ("nparts", C.c_int), ("grad_scale", C.c_void_p)]
+
+
+def rmsnorm_backward_rows(x, scale, dy, eps, residual=None, out=None):
+    """The row pass alone: returns (dx, partial rows kept for rmsnorm_colsum_multi, their number)."""
+    dx = torch.empty_like(x) if out is None else out
+    rows, cols = x.shape
+    nbytes = kernels().seraph_rmsnorm_backward_ws_bytes(i64(rows), i64(cols))
+    part = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=x.device)
+    nparts = C.c_int(0)
+    check(kernels().seraph_rmsnorm_backward_rows(_p(x), _p(scale), _p(dy), _p(residual), _p(dx), i64(rows), i64(cols), f32(eps),
+                                                 _p(part), sz(nbytes), C.byref(nparts), _stream()), "rmsnorm_backward_rows")
+    return dx, part, nparts.value
+
+
+def rmsnorm_colsum_multi(jobs, cols):
+    """jobs: (partial, nparts, grad_scale) of row passes of one width; adds each pass's column sums to its grad_scale."""
+    arr = (ColsumJob * len(jobs))()
+    for i, (part, nparts, gs) in enumerate(jobs):
+        arr[i].partial, arr[i].nparts, arr[i].grad_scale = part.data_ptr(), nparts, gs.data_ptr()
+    check(kernels().seraph_rmsnorm_colsum_multi(arr, C.c_int(len(jobs)), i64(cols), _stream()), "rmsnorm_colsum_multi")
+
+
 def rmsnorm_backward_static(x, scale, dy, eps, grad_scale, dx, residual=None):
     """The backward over the library's built-in scratch array: every buffer is the caller's, nothing is allocated."""
     rows, cols = x.shape

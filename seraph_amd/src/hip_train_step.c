@@ -48,6 +48,10 @@ struct hip_trainer {
     void* side_ev[6];            /* fork | down | gate-up | o | q-k-v | end */
     void* ws2;                   /* scratch of the products on stream2 */
     size_t ws2_bytes;
+    char* norm_parts;            /* small steps: one region of partial rows per norm, folded by one launch after the backward */
+    size_t norm_part_bytes;      /* size of one region; 0 = each norm's column sum follows its row pass */
+    seraph_colsum_job_t* norm_jobs; /* host: the regions filled so far in this backward */
+    int norm_job_count;
     int overlap;
     /* arenas */
     float *P, *G, *M, *V;
@@ -58,7 +62,7 @@ struct hip_trainer {
     size_t act_bytes;
     layer_act_t* act;
     float *final_in, *xn_final, *logits, *loss_rows, *red_a, *red_b, *tmp_h, *lora_tmp, *lora_tmp2;
-    float *g_hidden, *g_tmp, *g_xn, *g_ffn, *g_gate, *g_up, *g_attn, *g_q, *g_k, *g_v, *scratch_gs;
+    float *g_hidden, *g_tmp, *g_xn, *g_ffn, *g_gate, *g_up, *g_attn, *g_q, *g_k, *g_v;
     uint32_t *d_tokens, *d_targets, *d_starts;
     uint32_t* h_stage;           /* pinned: tokens | targets | starts */
     void* ws;
@@ -178,6 +182,29 @@ static void op_fold(hip_trainer_t* t) {
         for (int gi_ = 0; gi_ < (count_); gi_++) fl_ += 2.0 * (double)(probs_)[gi_].M * (double)(probs_)[gi_].N * (double)(K_); \
         OP(seraph_gemm_grouped_kernel_name((probs_), (count_), (K_), 1, 0), fl_, 0.0,                  \
            seraph_gemm_grouped((probs_), (count_), (K_), 1, 0, 1, sw));                                \
+    } while (0)
+
+/* vulkan_rmsnorm_backward_batch of a norm (src/train.c:5071-5077, :5180-5193, :5342-5355).  A small full-weight step
+ * runs the row pass alone and books the column sum for the one launch after the backward; a LoRA step has no use
+ * for the norms' weight gradients (the reference sums them into a scratch that nothing reads, src/train.c:6381-6390)
+ * and runs the row pass alone; otherwise the column sum follows its row pass. */
+#define NORM_BWD(x_, w_, dy_, res_, dx_, gs_, bytes_)                                                  \
+    do {                                                                                               \
+        if (lora) {                                                                                    \
+            int np_ = 0;                                                                               \
+            OP("rmsnorm_backward", 0.0, (bytes_), seraph_rmsnorm_backward_rows((x_), (w_), (dy_), (res_), (dx_), T, h, eps, \
+                                                                               t->ws, t->ws_bytes, &np_, s)); \
+        } else if (t->norm_part_bytes) {                                                               \
+            seraph_colsum_job_t* j_ = &t->norm_jobs[t->norm_job_count];                                \
+            float* part_ = (float*)(t->norm_parts + (size_t)t->norm_job_count * t->norm_part_bytes);   \
+            OP("rmsnorm_backward", 0.0, (bytes_), seraph_rmsnorm_backward_rows((x_), (w_), (dy_), (res_), (dx_), T, h, eps, \
+                                                                               part_, t->norm_part_bytes, &j_->nparts, s)); \
+            j_->partial = part_; j_->grad_scale = (gs_);                                               \
+            t->norm_job_count++;                                                                       \
+        } else {                                                                                       \
+            OP("rmsnorm_backward", 0.0, (bytes_), seraph_rmsnorm_backward_residual((x_), (w_), (dy_), (res_), (dx_), (gs_), T, h, eps, \
+                                                                                   t->ws, t->ws_bytes, s)); \
+        }                                                                                              \
     } while (0)
 
 /* the second stream picks up from this point of the first | marks a point of the second | the first waits for a mark */
@@ -349,7 +376,7 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
                                  adapters * up256(T * r * 4);
         const size_t rest = 2 * up256(T * h * 4) + up256(T * Vv * 4) + 3 * up256(T * 4) + up256(T * h * 4) + 2 * up256(T * r * 4) +
                             3 * up256(T * h * 4) + 3 * up256(T * f * 4) + 2 * up256(T * qd * 4) + 2 * up256(T * kv * 4) +
-                            up256(h * 4) + 2 * up256(T * 4) + up256(((size_t)max_batch + 1) * 4);
+                            2 * up256(T * 4) + up256(((size_t)max_batch + 1) * 4);
         t->act_bytes = per_layer * (size_t)cfg->layers + rest;
         if (dev_alloc(t, (void**)&t->act_arena, t->act_bytes)) goto fail;
         t->act = (layer_act_t*)calloc((size_t)cfg->layers, sizeof(layer_act_t));
@@ -371,7 +398,6 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
         TAKE(t->g_hidden, T * h * 4); TAKE(t->g_tmp, T * h * 4); TAKE(t->g_xn, T * h * 4);
         TAKE(t->g_ffn, T * f * 4); TAKE(t->g_gate, T * f * 4); TAKE(t->g_up, T * f * 4);
         TAKE(t->g_attn, T * qd * 4); TAKE(t->g_q, T * qd * 4); TAKE(t->g_k, T * kv * 4); TAKE(t->g_v, T * kv * 4);
-        TAKE(t->scratch_gs, h * 4);
         TAKE(t->d_tokens, T * 4); TAKE(t->d_targets, T * 4); TAKE(t->d_starts, ((size_t)max_batch + 1) * 4);
 #undef TAKE
         if ((size_t)(p - t->act_arena) > t->act_bytes) { fprintf(stderr, "ERROR: activation arena layout overflow\n"); goto fail; }
@@ -402,6 +428,16 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
     }
     if (dev_alloc(t, &t->ws, t->ws_bytes)) goto fail;
     if (t->stream2 && t->ws2_bytes && dev_alloc(t, &t->ws2, t->ws2_bytes)) goto fail;
+    /* The 2 L + 1 column sums of the norms' weight gradients are 4-5 us launches on the chain of dependent kernels
+     * and nothing waits for them before the optimizer: a step small enough for that to show (the same bound as for
+     * the second stream) keeps every norm's partial rows and folds them all with one launch after the backward. */
+    if (!t->lora && (int64_t)max_tokens * cfg->hidden <= ((int64_t)1 << 22)) {
+        const size_t regions = 2 * (size_t)cfg->layers + 1;
+        t->norm_part_bytes = (seraph_rmsnorm_backward_ws_bytes(max_tokens, cfg->hidden) + 255) & ~(size_t)255;
+        if (dev_alloc(t, (void**)&t->norm_parts, regions * t->norm_part_bytes)) goto fail;
+        t->norm_jobs = (seraph_colsum_job_t*)calloc(regions, sizeof(*t->norm_jobs));
+        if (!t->norm_jobs) goto fail;
+    }
     if (seraph_hip_host_alloc((void**)&t->h_stage, ((size_t)2 * max_tokens + max_batch + 1) * 4) != SERAPH_OK) goto fail;
     if (seraph_hip_stream_sync(t->stream) != SERAPH_OK) goto fail;
     return t;
@@ -423,6 +459,8 @@ void hip_trainer_free(hip_trainer_t* t) {
     seraph_hip_free(t->act_arena);
     seraph_hip_free(t->ws);
     seraph_hip_free(t->ws2);
+    seraph_hip_free(t->norm_parts);
+    free(t->norm_jobs);
     seraph_hip_free(t->attn_ws);
     seraph_hip_free(t->d_nan_flags);
     free(t->h_nan_flags);
@@ -795,8 +833,8 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
     GEMM(glog, P + t->off_embed, t->g_hidden, T, h, V, 0, 0, 0);            /* LM head dgrad */
     NANCHK(t->g_hidden, T * h, 4u);
     SIDE_ARM();
-    OP("rmsnorm_backward", 0.0, 12.0 * (double)(T * h), seraph_rmsnorm_backward(t->final_in, P + t->off_final_norm, t->g_hidden, t->g_tmp,
-                               lora ? t->scratch_gs : t->G + t->off_final_norm, T, h, eps, t->ws, t->ws_bytes, s));
+    t->norm_job_count = 0;
+    NORM_BWD(t->final_in, P + t->off_final_norm, t->g_hidden, NULL, t->g_tmp, t->G + t->off_final_norm, 12.0 * (double)(T * h));
     NANCHK(t->g_tmp, T * h, 5u);
     { float* sw = t->g_hidden; t->g_hidden = t->g_tmp; t->g_tmp = sw; }                   /* grad_hidden = grad_tmp (copy, src/train.c:5089) */
     NANCHK(t->g_hidden, T * h, 0u);
@@ -837,8 +875,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         SIDE_JOIN(MK_DOWN);                                                  /* g_hidden is rewritten next */
         /* the input gradient is added to the residual stream's gradient as it is stored (src/train.c:5180-5193) */
         SIDE_ARM();
-        OP("rmsnorm_backward", 0.0, 16.0 * (double)(T * h), seraph_rmsnorm_backward_residual(a->post_in, W + t->L.post_norm, t->g_xn, t->g_hidden, t->g_hidden,
-                                   lora ? t->scratch_gs : GW + t->L.post_norm, T, h, eps, t->ws, t->ws_bytes, s));
+        NORM_BWD(a->post_in, W + t->L.post_norm, t->g_xn, t->g_hidden, t->g_hidden, GW + t->L.post_norm, 16.0 * (double)(T * h));
 
         /* attention */
         SIDE_FORK();
@@ -882,11 +919,14 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         }
         SIDE_JOIN(MK_O);                                                     /* g_hidden is rewritten next */
         if (l > 0) SIDE_ARM();
-        OP("rmsnorm_backward", 0.0, 16.0 * (double)(T * h), seraph_rmsnorm_backward_residual(a->layer_in, W + t->L.in_norm, t->g_xn, t->g_hidden, t->g_hidden,
-                                   lora ? t->scratch_gs : GW + t->L.in_norm, T, h, eps, t->ws, t->ws_bytes, s));       /* src/train.c:5342-5355 */
+        NORM_BWD(a->layer_in, W + t->L.in_norm, t->g_xn, t->g_hidden, t->g_hidden, GW + t->L.in_norm, 16.0 * (double)(T * h));   /* src/train.c:5342-5355 */
         NANCHK(t->g_hidden, T * h, nan_gh + (uint32_t)l);
     }
     NANCHK(t->g_hidden, T * h, 8u);
+    if (t->norm_job_count > 0) {
+        OP("rmsnorm_colsum", 0.0, 0.0, seraph_rmsnorm_colsum_multi(t->norm_jobs, t->norm_job_count, h, s));
+        t->norm_job_count = 0;
+    }
     SIDE_MARK(MK_END);
     SIDE_JOIN(MK_END);                                                       /* every weight gradient is complete from here on */
     if (!lora) OP("embedding_backward", 0.0, 12.0 * (double)(T * h), seraph_embedding_backward(t->d_tokens, t->g_hidden, t->G + t->off_embed, T, h, V, t->ws, t->ws_bytes, s));

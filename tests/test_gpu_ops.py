@@ -319,6 +319,44 @@ def test_rmsnorm_backward_with_residual(ops, rows, cols):
     assert torch.equal(inplace, want)
 
 
+@pytest.mark.parametrize("cols", [512, 2048, 100])
+def test_rmsnorm_backward_rows_then_one_column_sum_for_all(ops, cols):
+    """The row pass alone, several times, then one launch that folds every pass's partial rows: the same bits as the
+    one-call backward, with and without a residual, for every row kernel (wave per row, block per row, generic)."""
+    r = rng(cols)
+    s = dev((1 + 0.02 * r.standard_normal(cols)).astype(np.float32))
+    cases, jobs, want = [], [], []
+    for i, rows in enumerate((300, 33, 2048, 1)):
+        x = dev(r.standard_normal((rows, cols)).astype(np.float32))
+        dy = dev((1e-2 * r.standard_normal((rows, cols))).astype(np.float32))
+        res = dev(r.standard_normal((rows, cols)).astype(np.float32)) if i % 2 else None
+        g0 = r.standard_normal(cols).astype(np.float32)
+        want.append(ops.rmsnorm_backward(x, s, dy, 1e-5, grad_scale=dev(g0), residual=res))
+        dx, part, nparts = ops.rmsnorm_backward_rows(x, s, dy, 1e-5, residual=res)
+        assert nparts > 0
+        gs = dev(g0)
+        cases.append((dx, gs)); jobs.append((part, nparts, gs))
+    ops.rmsnorm_colsum_multi(jobs, cols)
+    for (dx, gs), (wdx, wgs) in zip(cases, want):
+        assert torch.equal(dx, wdx) and torch.equal(gs, wgs)
+
+
+def test_rmsnorm_colsum_multi_more_jobs_than_one_launch_holds(ops):
+    cols, rows = 256, 40
+    r = rng(11)
+    s = dev((1 + 0.02 * r.standard_normal(cols)).astype(np.float32))
+    x = dev(r.standard_normal((rows, cols)).astype(np.float32))
+    jobs, want = [], []
+    for i in range(70):
+        dy = dev((1e-2 * r.standard_normal((rows, cols))).astype(np.float32))
+        want.append(ops.rmsnorm_backward(x, s, dy, 1e-5)[1])
+        _, part, nparts = ops.rmsnorm_backward_rows(x, s, dy, 1e-5)
+        jobs.append((part, nparts, torch.zeros(cols, device="cuda")))
+    ops.rmsnorm_colsum_multi(jobs, cols)
+    for (_, _, gs), w in zip(jobs, want):
+        assert torch.equal(gs, w)
+
+
 def test_rmsnorm_backward_clamp_branch(ops, orc):
     r = rng(3)
     x = (1e-4 * r.standard_normal((6, 512))).astype(np.float32)       # sqrt(ms + 1e-5) < 0.01
