@@ -119,11 +119,12 @@ struct TileQueue {
     unsigned int* q;        // q[0] next item, q[1] workgroups finished
     int* slot;              // one int of LDS
     int total;
+    int extra = 0;          // workgroups at the end of the grid that do other work and never draw
     int drawn = 0;
     // A launch with no more workgroups than items' worth of residency gets exactly one workgroup per item
     // (persistent_grid): the item is then the workgroup's index and the counters stay untouched, which
     // saves the two round trips of the atomics, the whole cost of the queue for a short item.
-    __device__ __forceinline__ bool one_each() const { return total <= (int)gridDim.x; }
+    __device__ __forceinline__ bool one_each() const { return total <= (int)gridDim.x - extra; }
     __device__ __forceinline__ int next() {
         if (one_each()) {
             const int item = drawn ? -1 : (int)blockIdx.x;
@@ -138,7 +139,7 @@ struct TileQueue {
     }
     __device__ __forceinline__ void leave() const {
         if (one_each()) return;
-        if (threadIdx.x == 0 && atomicAdd(&q[1], 1u) == gridDim.x - 1) {
+        if (threadIdx.x == 0 && atomicAdd(&q[1], 1u) == gridDim.x - (unsigned)extra - 1) {
             q[0] = 0u;
             q[1] = 0u;
             __threadfence();
@@ -1079,10 +1080,10 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
 }
 
 // dK += sum of the split items' slices, in slice order (likewise dV); with `assign` the sum starts from zero
-__global__ __launch_bounds__(256) void attn_split_reduce_kernel(float* __restrict__ dK, float* __restrict__ dV,
-                                                                const float* __restrict__ partK, const float* __restrict__ partV,
-                                                                int64_t n4, int split, int assign) {
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+__device__ __forceinline__ void split_reduce(float* __restrict__ dK, float* __restrict__ dV,
+                                             const float* __restrict__ partK, const float* __restrict__ partV,
+                                             int64_t n4, int split, int assign, int block, int blocks) {
+    for (int64_t i = (int64_t)block * blockDim.x + threadIdx.x; i < n4; i += (int64_t)blocks * blockDim.x) {
         float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
         if (!assign) { a = reinterpret_cast<float4*>(dK)[i]; b = reinterpret_cast<float4*>(dV)[i]; }
         for (int p = 0; p < split; p++) {
@@ -1094,6 +1095,18 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(float* __restric
         reinterpret_cast<float4*>(dV)[i] = b;
     }
 }
+__global__ __launch_bounds__(256) void attn_split_reduce_kernel(float* __restrict__ dK, float* __restrict__ dV,
+                                                                const float* __restrict__ partK, const float* __restrict__ partV,
+                                                                int64_t n4, int split, int assign) {
+    split_reduce(dK, dV, partK, partV, n4, split, assign, (int)blockIdx.x, (int)gridDim.x);
+}
+// The same reduction as the last `blocks` workgroups of the dQ-from-dS launch: both only wait for the dK/dV kernel,
+// and a short step saves the launch.
+struct SplitReduce {
+    float* dK; float* dV; const float* partK; const float* partV;
+    int64_t n4;
+    int split, assign, blocks;          // blocks == 0: nothing to do
+};
 
 // ---------------------------------------------------------------- backward: dQ
 // grid (query tiles of 128, heads); wave w owns queries i0+32w .. +31; key/value tiles of 32.
@@ -1222,9 +1235,15 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const f
                                                                          float* __restrict__ dQ, const uint32_t* __restrict__ seq_starts,
                                                                          int batch, int64_t T, int H, int KVH, float scale, int ds_slots,
                                                                          unsigned int* __restrict__ queue,
-                                                                         const int* __restrict__ band_overflow, int epoch) {
+                                                                         const int* __restrict__ band_overflow, int epoch,
+                                                                         const SplitReduce red) {
     constexpr int LD = D + 4, DB = D / 32;
     constexpr int KT = KSPLIT ? 2 : 1, QROWS = KSPLIT ? 64 : 128;
+    if (red.blocks > 0 && blockIdx.x >= gridDim.x - (unsigned)red.blocks) {          // uniform over the workgroup
+        split_reduce(red.dK, red.dV, red.partK, red.partV, red.n4, red.split, red.assign,
+                     (int)(blockIdx.x - (gridDim.x - (unsigned)red.blocks)), red.blocks);
+        return;
+    }
     // Some sequence is longer than the band was sized for: dQ comes from the recomputing kernel launched next.
     if (*band_overflow == epoch) return;
     __shared__ __attribute__((aligned(16))) float sK[2][KT * 32 * LD];
@@ -1233,7 +1252,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const f
     const SeqTable seqs = load_seq_table(seq_starts, batch, (int)T, sSeq);
     const int nqt = (int)((T + QROWS - 1) / QROWS);
     const int64_t nqt32 = (T + 31) >> 5;
-    TileQueue tq_{queue, &sItem, nqt * H};
+    TileQueue tq_{queue, &sItem, nqt * H, red.blocks};
     __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
     const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, [&](int q) {
         const int64_t a = (int64_t)q * QROWS, z = (a + QROWS - 1 < T - 1) ? a + QROWS - 1 : T - 1;
@@ -1475,20 +1494,24 @@ static int run_backward(const float* Q, const float* K, const float* V, const fl
     else
         hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, false>), gkv, dim3(kAttnThreads), 0, st, Q, K, V, dO, lse, delta, row_start, dK, dV, seq_starts, batch,
                            T, H, KVH, scale, scale * kLog2e, qkv, ds, ds_slots, split, partK, partV, assign ? 1 : 0);
-    if (split > 1) {
+    const int64_t n4 = T * KVH * D / 4;
+    SplitReduce red{dK, dV, partK, partV, n4, split, assign ? 1 : 0, 0};
+    if (split > 1 && !ds) {
         SERAPH_LAUNCH_CHECK();
-        const int64_t n4 = T * KVH * D / 4;
         hipLaunchKernelGGL(attn_split_reduce_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(n4, 256), 4096)), dim3(256), 0, st,
                            dK, dV, partK, partV, n4, split, assign ? 1 : 0);
     }
     SERAPH_LAUNCH_CHECK();
     if (ds) {
+        // the slices of a split dK/dV are added by workgroups at the end of the dQ launch (nothing else is between the
+        // dK/dV kernel and either of them)
+        if (split > 1) red.blocks = (int)std::min<int64_t>(ceil_div(n4, 256), 2 * (int64_t)num_compute_units());
         if (ceil_div(T, 128) * H <= 2 * (int64_t)num_compute_units()) {        // short batch: see run_forward
-            dim3 gds((unsigned)std::min<int64_t>(ceil_div(T, 64) * H, (int64_t)num_compute_units() * 2));
-            hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<D, true>), gds, dim3(kAttnThreads), 0, st, K, ds, dQ, seq_starts, batch, T, H, KVH, scale, ds_slots, qq, overflow, epoch);
+            dim3 gds((unsigned)std::min<int64_t>(ceil_div(T, 64) * H, (int64_t)num_compute_units() * 2) + (unsigned)red.blocks);
+            hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<D, true>), gds, dim3(kAttnThreads), 0, st, K, ds, dQ, seq_starts, batch, T, H, KVH, scale, ds_slots, qq, overflow, epoch, red);
         } else {
-            dim3 gds((unsigned)std::min<int64_t>(ceil_div(T, 128) * H, (int64_t)num_compute_units() * 2));
-            hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<D, false>), gds, dim3(kAttnThreads), 0, st, K, ds, dQ, seq_starts, batch, T, H, KVH, scale, ds_slots, qq, overflow, epoch);
+            dim3 gds((unsigned)std::min<int64_t>(ceil_div(T, 128) * H, (int64_t)num_compute_units() * 2) + (unsigned)red.blocks);
+            hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<D, false>), gds, dim3(kAttnThreads), 0, st, K, ds, dQ, seq_starts, batch, T, H, KVH, scale, ds_slots, qq, overflow, epoch, red);
         }
         if (bound_can_fail) {                                   // stands down at once unless the delta kernel marked the launch
             SERAPH_LAUNCH_CHECK();
