@@ -188,7 +188,7 @@ def run_workload(w, key, steps, warmup, op_timing=True, pmc_calibration=False, w
     T = w["batch"] * w["seq"]
     lora = w["lora"] or dict(rank=0, alpha=0.0, mask=0)
     cfg = tr.model_config(w["hidden"], w["layers"], w["heads"], w["kv_heads"], w["head_dim"], w["ffn"], w["vocab"],
-                          w["rms_eps"], w["rope_theta"], lora["rank"], lora["alpha"], lora["mask"])
+                          w["rms_eps"], w["rope_theta"], lora["rank"], lora["alpha"], lora["mask"], 1 if w.get("qk_norm") else 0)
     opt = tr.optim_config(w["lr"], clip=w["clip"])
     n = tr.param_count(cfg)
 
@@ -299,7 +299,7 @@ def run_workload(w, key, steps, warmup, op_timing=True, pmc_calibration=False, w
         "ms_per_step": round(1000.0 * elapsed / steps, 3),
         "config": {"workload": w["name"], "tokens_per_step": T, "batch": w["batch"], "seq_len": w["seq"],
                    "params": n, "device_bytes": t.device_bytes + sum(x.numel() * 4 for x in ext if x is not None),
-                   "rms_eps": w["rms_eps"], "adamw_clip": w["clip"], "qk_norm": False, "seed": 1234},
+                   "rms_eps": w["rms_eps"], "adamw_clip": w["clip"], "qk_norm": bool(w.get("qk_norm")), "seed": 1234},
         "loss_first_last": [round(losses[0], 5), round(losses[-1], 5)],
         "phase_ms_last_step": {k: round(v, 3) for k, v in timing.items()},
         "roofline": roofline,
@@ -534,8 +534,13 @@ def main():
         # the rest of the metric: the 33M model and the LoRA configuration as whole steps, the single-op
         # configurations alone, and the unmodified reference step driver over the vulkan_* symbols
         others = {}
-        for key, steps, warmup in (("c1", 30, 5), ("c4", 8, 2)):
-            r = run_workload(WORKLOADS[key], key, steps, warmup, op_timing=not args.no_op_timing, wgrad_overlap=not args.one_stream)
+        # The two 1.7B configurations again with qk_norm on: the reference's text-mode step never applies it
+        # (src/train.c:4687-4689 acts only with the video flag), so the headline leaves it off; these lines say what
+        # the RMS over all heads after RoPE and its backward cost when the option is used.
+        extra = {"c5_with_qk_norm": dict(WORKLOADS["c5"], qk_norm=1, name=WORKLOADS["c5"]["name"] + ", qk_norm on"),
+                 "c4_with_qk_norm": dict(WORKLOADS["c4"], qk_norm=1, name=WORKLOADS["c4"]["name"] + ", qk_norm on")}
+        for key, steps, warmup in (("c1", 30, 5), ("c4", 8, 2), ("c5_with_qk_norm", 2, 1), ("c4_with_qk_norm", 4, 1)):
+            r = run_workload(WORKLOADS.get(key) or extra[key], key, steps, warmup, op_timing=not args.no_op_timing, wgrad_overlap=not args.one_stream)
             others[key] = {k: r[k] for k in ("value", "unit", "ms_per_step", "steps", "warmup", "config", "loss_first_last", "roofline")}
             top = sorted(r["kernels"].items(), key=lambda kv: -kv[1]["share"])[:6]
             others[key]["kernels"] = dict(top)
