@@ -165,9 +165,9 @@ struct TileOrder {
     }
 };
 template <typename LenFn>
-__device__ __forceinline__ TileOrder rank_tiles_by_length(int* lens, int* order, int n, bool descending, LenFn len) {
+__device__ __forceinline__ TileOrder rank_tiles_by_length(int* lens, int* order, int n, bool descending, bool all_at_once, LenFn len) {
     TileOrder t{nullptr, n, descending};
-    if (n > kMaxOrder || n < kMinOrder) return t;
+    if (n > kMaxOrder || n < kMinOrder || all_at_once) return t;       // every item starts at once: any order will do
     for (int i = threadIdx.x; i < n; i += (int)blockDim.x) lens[i] = len(i);
     __syncthreads();
     for (int i = threadIdx.x; i < n; i += (int)blockDim.x) {
@@ -244,7 +244,7 @@ __global__ __launch_bounds__(kAttnThreads, (KSPLIT ? 1 : 2)) void attn_fwd_kerne
     TileQueue tq_{queue, &sItem, nqt * H};
     __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
     // key tiles a query tile runs over: from the start of its first query's sequence to its last query
-    const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, [&](int q) {
+    const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, tq_.one_each(), [&](int q) {
         const int64_t a = (int64_t)q * QROWS, z = (a + QROWS - 1 < T - 1) ? a + QROWS - 1 : T - 1;
         return (int)((z + 1 - (seqs.start_of((int)a) / 32) * 32 + 31) / 32);
     });
@@ -490,7 +490,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void attn_bwd_dkv_kernel(const flo
     TileQueue tq_{queue, &sItem, nkt * KVH * split};
     __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
     // query tiles a 128-key tile is visible to: up to the end of its last key's sequence
-    const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nkt, false, [&](int k) {
+    const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nkt, false, tq_.one_each(), [&](int k) {
         const int64_t a = (int64_t)k * 128, z = (a + 127 < T - 1) ? a + 127 : T - 1;
         return (int)((seqs.end_of((int)z) - a + 31) / 32);
     });
@@ -1129,7 +1129,7 @@ __global__ __launch_bounds__(kAttnThreads, (D <= 64 ? 2 : 1)) void attn_bwd_dq_k
     const int nqt = (int)((T + 127) / 128);
     TileQueue tq_{queue, &sItem, nqt * H};
     __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
-    const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, [&](int q) {
+    const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, tq_.one_each(), [&](int q) {
         const int64_t a = (int64_t)q * 128, z = (a + 127 < T - 1) ? a + 127 : T - 1;
         return (int)((z + 1 - (seqs.start_of((int)a) / 32) * 32 + 31) / 32);
     });
@@ -1254,7 +1254,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_dq_ds_kernel(const f
     const int64_t nqt32 = (T + 31) >> 5;
     TileQueue tq_{queue, &sItem, nqt * H, red.blocks};
     __shared__ int sLen[kMaxOrder], sOrd[kMaxOrder];
-    const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, [&](int q) {
+    const TileOrder by_len = rank_tiles_by_length(sLen, sOrd, nqt, true, tq_.one_each(), [&](int q) {
         const int64_t a = (int64_t)q * QROWS, z = (a + QROWS - 1 < T - 1) ? a + QROWS - 1 : T - 1;
         return (int)((z + 1 - (seqs.start_of((int)a) / 32) * 32 + 31) / 32);
     });
