@@ -213,6 +213,17 @@ void hip_add_rmsnorm(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffe
 void hip_rmsnorm_backward_residual(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* scale,
                                    vulkan_buffer_t* grad_output, vulkan_buffer_t* residual, vulkan_buffer_t* grad_input,
                                    vulkan_buffer_t* grad_scale, int rows, int cols, float eps);
+/* vulkan_rmsnorm_backward_batch in two halves, for a step whose norms are small enough that each column-sum launch
+ * counts: hip_rmsnorm_backward_rows is the row pass (grad_input complete; residual may be NULL; the column sums behind
+ * grad_scale stay in `partial`, a buffer of hip_rmsnorm_backward_partial_bytes(rows, cols) bytes kept per norm) and
+ * returns the number of partial rows (0 on error); one hip_rmsnorm_colsum_multi after the last layer then adds every
+ * norm's column sums into its grad_scale (src/train.c:5071-5355: 2 L + 1 norms), bit-identically to the one-call op. */
+size_t hip_rmsnorm_backward_partial_bytes(int rows, int cols);
+int hip_rmsnorm_backward_rows(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* scale, vulkan_buffer_t* grad_output,
+                              vulkan_buffer_t* residual, vulkan_buffer_t* grad_input, vulkan_buffer_t* partial,
+                              int rows, int cols, float eps);
+void hip_rmsnorm_colsum_multi(vulkan_context_t* ctx, int count, vulkan_buffer_t* const* partial, const int* nparts,
+                              vulkan_buffer_t* const* grad_scale, int cols);
 /* C (+)= alpha * op(A) op(B): vulkan_matmul_transpose followed by vulkan_scale of the product, the pair the
  * LoRA path issues (src/train.c:5785-5792, :5815-5841), as one op.  accumulate with alpha != 1 is only possible
  * for the shapes the library computes through its scratch (small output, long K); otherwise the op reports an

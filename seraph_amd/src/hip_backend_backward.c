@@ -5,6 +5,7 @@
  * arguments ignored, outputs that the reference accumulates into are accumulated into.
  */
 #include <math.h>
+#include <stdlib.h>
 
 #include "hip_backend_internal.h"
 
@@ -60,6 +61,42 @@ void hip_rmsnorm_backward_residual(vulkan_context_t* ctx, vulkan_buffer_t* input
     HIP_OP(ctx, "rmsnorm_backward_residual", seraph_rmsnorm_backward_residual(FPTR(input), FPTR(scale), FPTR(grad_output), FPTR(residual),
                                                                               FPTR(grad_input), FPTR(grad_scale), rows, cols, eps, ws,
                                                                               st->ws_bytes, st->stream));
+}
+
+/* The row pass of vulkan_rmsnorm_backward_batch alone (residual may be NULL): grad_input is complete, and the column
+ * sums behind grad_scale stay in `partial`, a buffer of hip_rmsnorm_backward_partial_bytes(rows, cols) bytes that the
+ * caller keeps for this norm until hip_rmsnorm_colsum_multi has run.  Returns the number of partial rows, 0 on error. */
+size_t hip_rmsnorm_backward_partial_bytes(int rows, int cols) { return seraph_rmsnorm_backward_ws_bytes(rows, cols); }
+
+int hip_rmsnorm_backward_rows(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* scale, vulkan_buffer_t* grad_output,
+                              vulkan_buffer_t* residual, vulkan_buffer_t* grad_input, vulkan_buffer_t* partial,
+                              int rows, int cols, float eps) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || !input || !scale || !grad_output || !grad_input || !partial) return 0;
+    int nparts = 0;
+    HIP_OP(ctx, "rmsnorm_backward_rows", seraph_rmsnorm_backward_rows(FPTR(input), FPTR(scale), FPTR(grad_output),
+                                                                      residual ? FPTR(residual) : NULL, FPTR(grad_input), rows, cols, eps,
+                                                                      DPTR(partial), partial->size, &nparts, st->stream));
+    return nparts;
+}
+
+/* grad_scale[i] += column sums of partial[i] (nparts[i] rows as hip_rmsnorm_backward_rows returned them), for `count`
+ * norms of one width in one recorded op: the 2 L + 1 norms of a step (src/train.c:5071-5355) folded after the last
+ * layer.  Bit-identical to vulkan_rmsnorm_backward_batch's grad_scale. */
+void hip_rmsnorm_colsum_multi(vulkan_context_t* ctx, int count, vulkan_buffer_t* const* partial, const int* nparts,
+                              vulkan_buffer_t* const* grad_scale, int cols) {
+    hip_state_t* st = hip_state(ctx);
+    if (!st || count <= 0 || !partial || !nparts || !grad_scale) return;
+    seraph_colsum_job_t* jobs = (seraph_colsum_job_t*)malloc((size_t)count * sizeof(*jobs));
+    if (!jobs) { hip_backend_report(ctx, "rmsnorm_colsum_multi", SERAPH_ERR_INVALID); return; }
+    int k = 0;
+    for (int i = 0; i < count; i++) {
+        if (!partial[i] || !grad_scale[i] || nparts[i] <= 0) continue;                 /* skipped silently, like a NULL op argument */
+        jobs[k].partial = FPTR(partial[i]); jobs[k].nparts = nparts[i]; jobs[k].grad_scale = FPTR(grad_scale[i]);
+        k++;
+    }
+    HIP_OP(ctx, "rmsnorm_colsum_multi", seraph_rmsnorm_colsum_multi(jobs, k, cols, st->stream));
+    free(jobs);
 }
 
 /* src/vulkan_backend_backward.c:931-1045 */

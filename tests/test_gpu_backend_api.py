@@ -184,6 +184,44 @@ def test_lora_products_through_the_backend(vk, orc):
     assert lib.hip_backend_error_count(ctx) == 0
 
 
+def test_norm_column_sums_deferred_through_the_backend(vk):
+    """Three norms' backward as vulkan_rmsnorm_backward_batch issues them, and as row passes followed by one
+    hip_rmsnorm_colsum_multi over the kept partial rows: the same bits in grad_input and grad_scale."""
+    lib, ctx = vk
+    lib.hip_rmsnorm_backward_partial_bytes.restype = C.c_size_t
+    r = rng(23)
+    rows, cols, eps = 300, 512, C.c_float(1e-5)
+    s = (1 + 0.02 * r.standard_normal(cols)).astype(np.float32)
+    bs = up(vk, s)
+    nbytes = lib.hip_rmsnorm_backward_partial_bytes(rows, cols)
+    assert nbytes > 0
+    keep, parts, nparts, gs_new, want = [], [], [], [], []
+    assert lib.vulkan_cmd_begin(ctx) == 1
+    for i in range(3):
+        x, dy = (r.standard_normal((rows, cols)).astype(np.float32) for _ in range(2))
+        g0 = r.standard_normal(cols).astype(np.float32)
+        bx, bdy = up(vk, x), up(vk, dy)
+        dx1, dx2 = up(vk, np.zeros((rows, cols), np.float32)), up(vk, np.zeros((rows, cols), np.float32))
+        gs1, gs2 = up(vk, g0), up(vk, g0)
+        part = lib.vulkan_buffer_create(ctx, C.c_size_t(nbytes))
+        lib.vulkan_rmsnorm_backward_batch(ctx, bx, bs, bdy, dx1, gs1, rows, cols, eps)
+        n = lib.hip_rmsnorm_backward_rows(ctx, bx, bs, bdy, None, dx2, part, rows, cols, eps)
+        assert n > 0
+        parts.append(part); nparts.append(n); gs_new.append(gs2); want.append((dx1, dx2, gs1))
+        keep += [bx, bdy]
+    P = (C.c_void_p * 3)(*[C.cast(b, C.c_void_p) for b in parts])
+    G = (C.c_void_p * 3)(*[C.cast(b, C.c_void_p) for b in gs_new])
+    N = (C.c_int * 3)(*nparts)
+    lib.hip_rmsnorm_colsum_multi(ctx, 3, P, N, G, cols)
+    assert lib.vulkan_cmd_end_submit(ctx) == 1
+    for (dx1, dx2, gs1), gs2 in zip(want, gs_new):
+        assert (down(vk, dx1, (rows, cols)) == down(vk, dx2, (rows, cols))).all()
+        assert (down(vk, gs1, cols) == down(vk, gs2, cols)).all()
+    for buf in keep + parts + gs_new + [b for w in want for b in w] + [bs]:
+        lib.vulkan_buffer_free(ctx, buf)
+    assert lib.hip_backend_error_count(ctx) == 0
+
+
 def test_residual_adds_folded_into_the_norms(vk):
     """hip_add_rmsnorm and hip_rmsnorm_backward_residual against the reference's op pairs, bit for bit."""
     lib, ctx = vk
