@@ -64,6 +64,17 @@ def test_argument_validation_needs_no_device(libs):
                           C.c_float(0), C.c_float(0), 1, C.c_float(0), None) == 0           # empty tensor: no-op
     k.seraph_attention_backward_ws_bytes.restype = C.c_size_t
     assert k.seraph_attention_backward_ws_bytes(C.c_int64(1024), 16, 8, 128) >= 1024 * 16 * 128 * 4
+    # the norm backward in two halves: an empty pass reports no partial rows, a missing scratch is refused before
+    # any launch, an empty job list is a no-op and a list without its array is an error
+    n = C.c_int(7)
+    assert k.seraph_rmsnorm_backward_rows(None, None, None, None, None, C.c_int64(0), C.c_int64(512), C.c_float(1e-5),
+                                          None, C.c_size_t(0), C.byref(n), None) == 0 and n.value == 0
+    p = C.c_void_p(256)                                  # never dereferenced: the scratch check comes first
+    assert k.seraph_rmsnorm_backward_rows(p, p, p, None, p, C.c_int64(64), C.c_int64(512), C.c_float(1e-5),
+                                          None, C.c_size_t(0), C.byref(n), None) == -3
+    assert b"scratch" in k.seraph_hip_last_error()
+    assert k.seraph_rmsnorm_colsum_multi(None, 0, C.c_int64(512), None) == 0
+    assert k.seraph_rmsnorm_colsum_multi(None, 3, C.c_int64(512), None) == -1
 
 
 def test_param_count_matches_reference_shapes(libs):
