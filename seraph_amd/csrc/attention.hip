@@ -315,6 +315,11 @@ __global__ __launch_bounds__(kAttnThreads, (KSPLIT ? 1 : 2)) void attn_fwd_kerne
                 if (s8 + 1 < D / 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
             }
+            // The softmax between the two runs of matrix instructions is this wave's only stretch of plain vector
+            // work; beside a wave of the co-resident workgroup that always has a matrix instruction ready it is
+            // served slowly.  Raised priority for just this stretch lets it through (the neighbour's matrix
+            // instructions have 64 cycles of slack each): forward 207 -> 200 us at 8 x 1024 tokens, 16 heads of 64.
+            __builtin_amdgcn_s_setprio(3);
             float mloc = -INFINITY;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
@@ -343,6 +348,7 @@ __global__ __launch_bounds__(kAttnThreads, (KSPLIT ? 1 : 2)) void attn_fwd_kerne
             for (int v = 0; v < 16; v++) { s[v] = fast_exp2(s[v] - msafe); lsum += s[v]; }
             lsum += __shfl_xor(lsum, 32, 64);
             l += lsum;
+            __builtin_amdgcn_s_setprio(0);
             DVec<DB> vb[2];
             vb[0] = lds_dvec<DB>(&sVt[acc_row(0, h) * LD], r);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
