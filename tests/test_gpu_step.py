@@ -132,6 +132,36 @@ def test_full_step_gradient_accumulation(tr, orc):
     t.close()
 
 
+def test_twelve_optimizer_steps_follow_the_oracle(tr, orc):
+    """A short training run: every step a new batch, the warm-up schedule moving, Adam's moments and bias corrections
+    carried from step to step, clipping on.  Per-step loss, then weights and both moments at the end, against the
+    oracle's step and AdamW applied in the same order."""
+    case = dict(CASES[0])
+    starts = np.array(case.pop("starts"), np.int32)
+    ocfg = orc.make_config(**case)
+    cfg = tr.model_config(**case)
+    p = init_params(orc, ocfg, 11)
+    T, base_lr, clip = int(starts[-1]), 1e-2, 1.0
+    t = tr.Trainer(cfg, tr.optim_config(base_lr, clip=clip), max_tokens=T, max_batch=len(starts) - 1)
+    t.upload(tr.PARAMS, p)
+    w, m, v = p.copy(), np.zeros_like(p), np.zeros_like(p)
+    for step in range(1, 13):
+        tok = rng(100 + step).integers(0, case["vocab"], T).astype(np.int32)
+        ref_loss, g = orc.step_full(ocfg, w, tok, starts)
+        lr = orc.lr_schedule(base_lr, step, 1)
+        w, m, v = orc.adamw(w, g, m, v, lr, 0.9, 0.999, 0.01, 1e-8, step, clip)
+        loss = t.step(tok, starts)
+        assert t.optimizer_step == step and abs(t.last_lr - lr) < 1e-12
+        assert abs(loss - ref_loss) < 2e-5 * max(1.0, abs(ref_loss)), (step, loss, ref_loss)
+    sl = tensor_slices(ocfg)
+    check_tensors(t.download(tr.PARAMS), w, sl, "weight after 12 steps")
+    check_tensors(t.download(tr.ADAM_M), m, sl, "adam m after 12 steps")
+    got_v, ref_v = t.download(tr.ADAM_V), v
+    assert np.abs(got_v - ref_v).max() <= 1e-9 + 1e-3 * np.abs(ref_v).max()
+    assert np.abs(w - p).max() > 1e-3                    # the run did move the weights
+    t.close()
+
+
 def test_weight_gradients_on_the_second_stream_change_no_bit(tr, orc):
     """Three optimizer steps with the weight gradients beside the input-gradient chain (default) and with everything on
     one stream: every product is one kernel either way, so weights, gradients and moments must be identical; a missing
