@@ -253,6 +253,44 @@ def test_lora_step(tr, orc, b_zero, mask):
     t.close()
 
 
+def test_eight_lora_steps_from_the_initial_state_follow_the_oracle(tr, orc):
+    """From B = 0 (the adapters' initial state, src/lora.c:76-78): the first step moves only B, the later ones both
+    factors, with the forward's kept x A^T feeding every backward.  Per-step loss, then the adapters and Adam's first
+    moment after eight steps, against the oracle."""
+    mask = 0b1111111
+    case = dict(hidden=64, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=96, vocab=101, lora_rank=16,
+                lora_alpha=32.0, lora_mask=mask)
+    starts = np.array([0, 41, 90], np.int32)
+    ocfg = orc.make_config(**case)
+    cfg = tr.model_config(**case)
+    p = init_params(orc, ocfg, 6)
+    lo = (0.05 * rng(8).standard_normal(orc.lora_param_count(ocfg))).astype(np.float32)
+    h, qd, kv, f, rk = 64, 128, 64, 96, 16
+    o = 0
+    for _ in range(2):
+        for i, oo in ((h, qd), (h, kv), (h, kv), (qd, h), (h, f), (h, f), (f, h)):
+            o += rk * i
+            lo[o:o + oo * rk] = 0
+            o += oo * rk
+    base_lr = 2e-2
+    t = tr.Trainer(cfg, tr.optim_config(base_lr), max_tokens=90, max_batch=2)
+    t.upload(tr.PARAMS, p)
+    t.upload(tr.LORA_PARAMS, lo)
+    w, m, v = lo.copy(), np.zeros_like(lo), np.zeros_like(lo)
+    for step in range(1, 9):
+        tok = rng(200 + step).integers(0, 101, 90).astype(np.int32)
+        ref_loss, g = orc.step_lora(ocfg, p, w, tok, starts)
+        w, m, v = orc.adamw(w, g.astype(np.float32), m, v, orc.lr_schedule(base_lr, step), 0.9, 0.999, 0.01, 1e-8, step)
+        loss = t.step(tok, starts)
+        assert abs(loss - ref_loss) < 2e-5 * max(1.0, abs(ref_loss)), (step, loss, ref_loss)
+    got = t.download(tr.LORA_PARAMS).astype(np.float64)
+    assert (np.abs(got - w) <= ATOL + RTOL * np.abs(w)).all(), np.abs(got - w).max()
+    gm = t.download(tr.LORA_M).astype(np.float64)
+    assert (np.abs(gm - m) <= ATOL + RTOL * np.abs(m)).all(), np.abs(gm - m).max()
+    assert np.abs(w - lo).max() > 1e-3 and (t.download(tr.PARAMS) == p).all()
+    t.close()
+
+
 @pytest.mark.parametrize("lora", [False, True])
 def test_step_with_qk_norm(tr, orc, lora):
     """use_qk_norm = 1 in both step drivers: forward after RoPE, derivative before the RoPE backward (the reference's
