@@ -33,13 +33,13 @@ def tr():
     return trainer
 
 
-def make_model_dir(path, orc, shape, seed):
+def make_model_dir(path, orc, shape, seed, std=0.05):
     from safetensors.torch import save_file
     from seraph_amd.trainer import model_config
     os.makedirs(path, exist_ok=True)
     ocfg = orc.make_config(**shape, rms_eps=1e-5, rope_theta=10000.0)
     cfg = model_config(**shape, rms_eps=1e-5, rope_theta=10000.0)
-    p = init_params(orc, ocfg, seed)
+    p = init_params(orc, ocfg, seed, std)
     p = torch.from_numpy(p).to(torch.bfloat16).to(torch.float32).numpy()             # what a BF16 file can hold
     save_file({k: v.to(torch.bfloat16).contiguous() for k, v in named_tensors(cfg, p).items()},
               os.path.join(path, "model.safetensors"))
@@ -321,6 +321,46 @@ def test_reference_batched_trainer_runs_unmodified_and_matches_oracle(tmp_path, 
     rc, mine, err = run_cli(args[:-1] if flash else args)
     assert rc == 0, err[-1500:]
     assert np.allclose([l for _, l in step_losses(mine)], got, atol=1.1e-4)
+
+
+C1_SHAPE = dict(hidden=512, layers=8, heads=8, kv_heads=8, head_dim=64, ffn=1408, vocab=8192)
+
+
+@needs_ref
+def test_reference_batched_trainer_at_the_33m_shape_8_x_256(tmp_path, orc):
+    """The 33M model exactly, eight packed sequences of 256 tokens per step, three optimizer steps through the
+    reference's own cuda_train_step_gpu_full_batch (src/train_cuda.c:1966-2326) over the cuda_train_* symbols:
+    the printed losses step by step and the final checkpoint against the oracle's step + AdamW."""
+    mdir, ckpt = str(tmp_path / "model"), str(tmp_path / "ckpt")
+    ocfg, cfg, p0 = make_model_dir(mdir, orc, C1_SHAPE, seed=81, std=0.02)
+    add_tokenizer(mdir, C1_SHAPE["vocab"])
+    r = np.random.default_rng(82)
+    samples = [r.integers(0, C1_SHAPE["vocab"], 256).astype(np.int32) for _ in range(24)]
+    ttok = os.path.join(mdir, "train.ttok")
+    write_ttok(ttok, samples, vocab=C1_SHAPE["vocab"])
+    args = [mdir, ttok, "--full-training", "--batch", 8, "--max-seq", 256, "--lr", 3.14e-4, "--log-every", 1,
+            "--save-every", 0, "--checkpoint", ckpt]
+    rc, out, err = run_ref(args)
+    assert rc == 0, (out[-1500:], err[-1500:])
+    tokens = np.concatenate(samples)
+    offsets = np.concatenate([[0], np.cumsum([len(s) for s in samples])]).tolist()
+    batches = reference_pack(tokens.tolist(), offsets, 8, 256)
+    assert len(batches) == 3 and all(len(b[1]) == 9 and b[1][-1] == 2048 for b in batches)
+    ref_losses, rp, _, _ = oracle_run(orc, ocfg, p0.copy(), batches, 3.14e-4)
+    got = [l for _, l in step_losses(out)]
+    assert len(got) == 3
+    assert np.allclose(got, ref_losses, atol=1.5e-4), (got, ref_losses)
+    from seraph_amd import io as sio
+    saved = sio.checkpoint_load(os.path.join(ckpt, "checkpoint_final.safetensors"), cfg)
+    assert np.all(np.abs(saved - rp) <= 2.0 ** -7 * np.abs(rp) + 1e-6)
+    assert np.abs(rp - p0).max() > 1e-6                              # the weights moved, so the bound above says something
+    # this repository's own front end (the fused step) on the same files
+    rc, mine, err = run_cli(args)
+    assert rc == 0, err[-1500:]
+    assert np.allclose([l for _, l in step_losses(mine)], ref_losses, atol=1.5e-4)
+    gp, gm, gv = read_optim(os.path.join(ckpt, "checkpoint_final.safetensors"))
+    sl = tensor_slices(ocfg)
+    check_tensors(gp, rp, sl, "weight (33M shape, fused front end)")
 
 
 @needs_ref

@@ -39,7 +39,7 @@ def run_driver(tmp_path, case, steps, T, lr0, theta, p, tok, rank=0, mask=0, alp
             lora.tofile(f)
         tok.tofile(f)
     print(f"running {BIN} case={case} T={T} steps={steps} rank={rank} mask={mask:#b}", flush=True)
-    r = subprocess.run([BIN, str(fin), str(fout)], capture_output=True, text=True, timeout=100)
+    r = subprocess.run([BIN, str(fin), str(fout)], capture_output=True, text=True, timeout=170)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     return np.fromfile(fout, np.float32)
 
@@ -69,6 +69,43 @@ def test_reference_driver_matches_oracle(orc, case, tmp_path):
     sl = tensor_slices(ocfg)
     check_tensors(g, ref_g, sl, "reference-driver grad")
     check_tensors(w, rw, sl, "reference-driver weight")
+
+
+C1 = dict(hidden=512, layers=8, heads=8, kv_heads=8, head_dim=64, ffn=1408, vocab=8192)
+
+
+@needs_bin
+@pytest.mark.parametrize("T", [256, 2048])
+def test_reference_driver_at_the_33m_shape(orc, T, tmp_path):
+    """The 33M model exactly (512 wide, 8 layers, 8 heads of 64, FFN 1408, vocabulary 8192) through the reference's own
+    train_step_gpu_full over the vulkan_* symbols, one sequence of 256 and of 2048 tokens, two optimizer steps: the
+    op-by-op path at the sizes where it takes the banded attention backward, K runs in vulkan_matmul_transpose and
+    the 512-fan-in vulkan_reduce_sum over more than one pass.  Loss per step, every gradient tensor of the last step
+    and every weight tensor after it against the oracle's step + AdamW, element-wise 1e-5 + 1e-4 |ref|."""
+    case, steps, lr0, theta = dict(C1), 2, 3.14e-4, 10000.0
+    ocfg = orc.make_config(**case, rms_eps=1e-5, rope_theta=theta)
+    r = np.random.default_rng(31)
+    p = (0.02 * r.standard_normal(orc.param_count(ocfg))).astype(np.float32)
+    sl = tensor_slices(ocfg)
+    for name, a, b in sl:
+        if name.endswith("norm"):
+            p[a:b] = 1.0
+    tok = r.integers(0, case["vocab"], steps * T).astype(np.int32)
+    out = run_driver(tmp_path, case, steps, T, lr0, theta, p, tok)
+    n = p.size
+    assert out.size == steps + 2 * n
+    loss, g, w = out[:steps], out[steps:steps + n], out[steps + n:]
+    rw, rm, rv = p.copy(), np.zeros_like(p), np.zeros_like(p)
+    starts = np.array([0, T], np.int32)
+    for s in range(steps):
+        ref_loss, ref_g = orc.step_full(ocfg, rw, tok[s * T:(s + 1) * T], starts)
+        assert abs(loss[s] - ref_loss) < 1e-5 * max(1.0, abs(ref_loss)), (s, loss[s], ref_loss)
+        rw, rm, rv = orc.adamw(rw, ref_g, rm, rv, orc.lr_schedule(lr0, s + 1, 1), 0.9, 0.999, 0.01, 1e-8, s + 1)
+    check_tensors(g, ref_g, sl, "reference-driver grad")
+    check_tensors(w, rw, sl, "reference-driver weight")
+    rel = max(np.linalg.norm(g[a:b] - ref_g[a:b]) / (np.linalg.norm(ref_g[a:b]) + 1e-30) for _, a, b in sl)
+    assert rel <= 1e-4, rel
+    print(f"\n  T={T}: losses {loss.tolist()}, worst per-tensor rel-L2 of the gradients {rel:.2e}")
 
 
 @needs_bin

@@ -145,6 +145,7 @@ def test_twelve_optimizer_steps_follow_the_oracle(tr, orc):
     t = tr.Trainer(cfg, tr.optim_config(base_lr, clip=clip), max_tokens=T, max_batch=len(starts) - 1)
     t.upload(tr.PARAMS, p)
     w, m, v = p.copy(), np.zeros_like(p), np.zeros_like(p)
+    worst_loss = 0.0
     for step in range(1, 13):
         tok = rng(100 + step).integers(0, case["vocab"], T).astype(np.int32)
         ref_loss, g = orc.step_full(ocfg, w, tok, starts)
@@ -152,12 +153,15 @@ def test_twelve_optimizer_steps_follow_the_oracle(tr, orc):
         w, m, v = orc.adamw(w, g, m, v, lr, 0.9, 0.999, 0.01, 1e-8, step, clip)
         loss = t.step(tok, starts)
         assert t.optimizer_step == step and abs(t.last_lr - lr) < 1e-12
-        assert abs(loss - ref_loss) < 2e-5 * max(1.0, abs(ref_loss)), (step, loss, ref_loss)
+        worst_loss = max(worst_loss, abs(loss - ref_loss) / max(1.0, abs(ref_loss)))
     sl = tensor_slices(ocfg)
     check_tensors(t.download(tr.PARAMS), w, sl, "weight after 12 steps")
     check_tensors(t.download(tr.ADAM_M), m, sl, "adam m after 12 steps")
     got_v, ref_v = t.download(tr.ADAM_V), v
-    assert np.abs(got_v - ref_v).max() <= 1e-9 + 1e-3 * np.abs(ref_v).max()
+    check_tensors(got_v, ref_v, sl, "adam v after 12 steps")
+    rel_v = max(np.linalg.norm(got_v[a:b] - ref_v[a:b]) / (np.linalg.norm(ref_v[a:b]) + 1e-30) for _, a, b in sl)
+    print(f"\n  [margin] twelve steps: worst loss difference {worst_loss:.2e} (bar 1e-5), adam v worst rel-L2 {rel_v:.2e} (bar 1e-4)")
+    assert worst_loss <= 1e-5 and rel_v <= 1e-4
     assert np.abs(w - p).max() > 1e-3                    # the run did move the weights
     t.close()
 
@@ -277,12 +281,15 @@ def test_eight_lora_steps_from_the_initial_state_follow_the_oracle(tr, orc):
     t.upload(tr.PARAMS, p)
     t.upload(tr.LORA_PARAMS, lo)
     w, m, v = lo.copy(), np.zeros_like(lo), np.zeros_like(lo)
+    worst_loss = 0.0
     for step in range(1, 9):
         tok = rng(200 + step).integers(0, 101, 90).astype(np.int32)
         ref_loss, g = orc.step_lora(ocfg, p, w, tok, starts)
         w, m, v = orc.adamw(w, g.astype(np.float32), m, v, orc.lr_schedule(base_lr, step), 0.9, 0.999, 0.01, 1e-8, step)
         loss = t.step(tok, starts)
-        assert abs(loss - ref_loss) < 2e-5 * max(1.0, abs(ref_loss)), (step, loss, ref_loss)
+        worst_loss = max(worst_loss, abs(loss - ref_loss) / max(1.0, abs(ref_loss)))
+    print(f"\n  [margin] eight LoRA steps: worst loss difference {worst_loss:.2e} (bar 1e-5)")
+    assert worst_loss <= 1e-5
     got = t.download(tr.LORA_PARAMS).astype(np.float64)
     assert (np.abs(got - w) <= ATOL + RTOL * np.abs(w)).all(), np.abs(got - w).max()
     gm = t.download(tr.LORA_M).astype(np.float64)

@@ -248,6 +248,20 @@ def test_qwen3_shape_full_step_2_x_4096_two_layers(tr, orc):
     run_full_case(tr, orc, QWEN, np.array([0, 4096, 8192], np.int32), 3.14e-4, 0.0, seed=51)
 
 
+def test_qwen3_shape_lora_step_with_qk_norm(tr, orc):
+    """The LoRA configuration as it is worded ("with qk_norm"): use_qk_norm = 1 at head_dim 128 over 16 / 8 heads, B != 0
+    so that both adapter matrices receive a gradient through the normalised queries and keys.  Forward after RoPE as
+    src/train.c:4687-4689; the derivative (saved rms, before the RoPE backward) is this build's own, pinned by
+    float64 autograd in the oracle's tests."""
+    c = dict(QWEN, lora_rank=16, lora_alpha=32.0, lora_mask=0b1111, use_qk_norm=1)
+    run_lora_case(tr, orc, c, np.array([0, 2048], np.int32), 3.14e-4, seed=43, b_zero=False)
+
+
+def test_qwen3_shape_full_step_with_qk_norm(tr, orc):
+    """Full-weight training at full width and vocabulary, depth 2, 2 x 4096 packed, use_qk_norm = 1."""
+    run_full_case(tr, orc, dict(QWEN, use_qk_norm=1), np.array([0, 4096, 8192], np.int32), 3.14e-4, 0.0, seed=53)
+
+
 # ------------------------------------------------------------------ the full 28-layer model, through properties
 def test_qwen3_shape_full_depth_step_properties(tr):
     """28 layers, 4 x 4096 tokens, 1.72 G parameters.  (1) The step is deterministic: the same state and batch give
