@@ -73,10 +73,12 @@ int  seraph_hip_device_sync(void);
 int  seraph_hip_event_create(void** out);
 int  seraph_hip_event_create_sync(void** out);                         /* orders streams of one device only: no timestamps, not for the host to wait on */
 int  seraph_hip_event_destroy(void* ev);
-/* Arms `ev` for the calling thread: the next op of this library that supports it (SwiGLU backward, RoPE, RMSNorm backward,
- * reduce_sum) completes the event with its last kernel, which is what hipEventRecord after the op would give, minus the
- * marker packet that a record puts between that kernel and the next.  seraph_hip_event_armed() tells afterwards whether
- * the event is still waiting for such an op (then record it the ordinary way; calling seraph_hip_event_on_next_op(NULL) disarms). */
+/* Arms `ev` for the calling thread: the next op of this library that supports it completes the event with its last
+ * kernel, which is what hipEventRecord after the op would give, minus the marker packet that a record puts between that
+ * kernel and the next.  The ops that take the event: every one-pass element-wise op (fill, add, mul, scale, silu, SwiGLU,
+ * their backward forms, AdamW), RoPE, RMSNorm backward and the column sums, reduce_sum - so arm it directly before the op
+ * it is meant for.  An op that returns an error disarms it.  seraph_hip_event_armed() tells afterwards whether the event
+ * is still waiting for such an op (then record it the ordinary way; seraph_hip_event_on_next_op(NULL) disarms). */
 int  seraph_hip_event_on_next_op(void* ev);
 int  seraph_hip_event_armed(void);
 int  seraph_hip_event_record(void* ev, seraph_stream_t s);
@@ -239,9 +241,11 @@ int seraph_rmsnorm_colsum_multi(const seraph_colsum_job_t* jobs, int count, int6
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  The partial rows of the column reduction live in an array built into the
  * library (seraph_rmsnorm_backward_static_max_bytes() = 16 MiB on every GPU the library runs on, held until
- * the process ends); the call allocates nothing.  Shapes whose seraph_rmsnorm_backward_ws_bytes exceeds
- * that size are refused with SERAPH_ERR_WORKSPACE (16384 x 2048 needs 4 MiB; rows of up to 8192 columns
- * fit at any row count when 16-byte aligned).  Results are bit-identical to the workspace form.  Every
+ * the process ends); the call allocates nothing.  The requirement is that of the kernel the operands
+ * select: 16-byte aligned rows of 516 to 8192 columns write one partial row per workgroup (two workgroups
+ * per compute unit: 16384 x 2048 needs 4 MiB, and such rows fit at any row count), aligned rows of up to
+ * 512 columns likewise, anything else one partial row per wavefront.  A call that needs more is refused
+ * with SERAPH_ERR_WORKSPACE before anything is touched.  Results are bit-identical to the workspace form.  Every
  * call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race. */
 size_t seraph_rmsnorm_backward_static_max_bytes(void);
 int seraph_rmsnorm_backward_static(const float* x, const float* scale, const float* dy, const float* residual, float* dx,

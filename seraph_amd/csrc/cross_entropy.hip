@@ -198,24 +198,27 @@ __device__ __forceinline__ float block_reduce(float v, float* lds) {
 // each workgroup combines its row's P records itself, in part order, so all of them derive the same maximum and total.
 //
 // The grid is persistent (a multiple of P workgroups, at most four per CU); workgroup g takes units g, g + G, ...
-// where unit u = (row u / P, part u % P): the P partners of a row work on it in the same round.  Records are
-// double-buffered by round parity and tagged (launch, round): a workgroup can only be one round ahead of a partner
-// it exchanges with, and a tag from another launch or round never matches.  The wait for a partner is bounded: past
-// the limit (a partner that has not been scheduled yet) the workgroup computes that part's statistics itself from
-// the logits, and takes the published ones instead if they have appeared meanwhile (the partner may by then be
-// overwriting its logits with the gradient when the call is in place; it publishes before it stores).
+// where unit u = (row u / P, part u % P): the P partners of a row work on it in the same round.  Every unit of a
+// launch has a record of its own, written once and never overwritten while the launch runs, tagged (launch, round):
+// a tag from another launch never matches.  The wait for a partner is bounded: past the limit (a partner that has
+// not been scheduled yet) the workgroup forms that part's statistics itself from the logits, with the owner's own
+// slots per lane, order of additions and reductions, so it arrives at the owner's bits; and it takes the published
+// pair instead if that has appeared meanwhile (in place the partner may by then be overwriting its logits with the
+// gradient: it publishes before it stores, and what it published stays readable however far ahead it runs).
+// Whichever way a workgroup learns a part's statistics, it learns the same two floats.
 constexpr int kCoopBlock = 256;
 constexpr int kCoopVpt = 19;                         // float4 per lane: 76 of the 128 registers a lane has at four workgroups per CU
 constexpr int kCoopWgsPerCu = 4;
 constexpr int kCoopMaxParts = 64;                     // one lane of the first wave per partner
 constexpr int kCoopMaxGrid = 2048;
-constexpr int kCoopLaunchSlots = 16;
+constexpr int kCoopLaunchSlots = 4;                   // launches that may be in flight on one device at a time
+constexpr int kCoopMaxUnits = 1 << 18;                // (row, part) units per launch; longer inputs go in several launches
 
 // Each word of a record validates itself: (statistic, half of a 64-bit hash of (launch, round)).  No ordering between
 // the two stores or the two loads is needed, hence no release/acquire fence (at device scope those write back and
 // invalidate whole caches on this part); the accesses are relaxed device-scope atomics, which go past the per-XCD L2s.
 struct CoopRec { unsigned long long max_word; unsigned long long sum_word; };
-static __device__ CoopRec g_ce_records[kCoopLaunchSlots][2][kCoopMaxGrid];
+static __device__ CoopRec g_ce_records[kCoopLaunchSlots][kCoopMaxUnits];
 
 __device__ __forceinline__ unsigned long long coop_tag(unsigned launch, unsigned round) {
     unsigned long long z = (((unsigned long long)launch << 32) | round) + 0x9e3779b97f4a7c15ull;      // splitmix64
@@ -240,32 +243,30 @@ __global__ __launch_bounds__(kCoopBlock, kCoopWgsPerCu) void ce_coop_kernel(cons
                                                                const uint32_t* __restrict__ targets,
                                                                float* __restrict__ grad, float* __restrict__ loss_rows,
                                                                const uint32_t* __restrict__ seq_starts, int batch,
-                                                               int64_t rows, int64_t cols, float scale, int P,
+                                                               int64_t row_begin, int64_t row_end, int64_t cols, float scale, int P,
                                                                CoopRec* __restrict__ recs, unsigned launch, int spin_limit,
                                                                int in_place) {
     __shared__ float red[2][kCoopBlock / 64];
-    __shared__ MaxSum redms[kCoopBlock / 64];
     __shared__ MaxSum parts[kCoopMaxParts];
     __shared__ unsigned long long missing;
     __shared__ float bcast[2];
     constexpr int kChunkBytes = kCoopBlock * 16;                   // one slot of every lane: 4 KB of the row
     const int G = gridDim.x;
     const int n4 = (int)(cols >> 2);
-    const int nchunks = (n4 + kCoopBlock - 1) / kCoopBlock;
-    const int part = (int)(blockIdx.x % P), base_wg = (int)blockIdx.x - part;
+    const int part = (int)(blockIdx.x % P);
     // Chunk c of the row belongs to part c % P: the P partners sweep the row side by side, and slot k of this
     // workgroup is chunk k P + part.  A slot whose chunk lies past the end of the row reads zeros and its store is
     // dropped (the row is addressed as a buffer), so no slot needs a test of its own.
     const int lane_off = threadIdx.x * 16;
     const int step_bytes = P * kChunkBytes, first_bytes = part * kChunkBytes;
     const float4 pad = make_float4(kNegBig, kNegBig, kNegBig, kNegBig);
-    const int64_t units = rows * P;
-    auto is_live = [&](int64_t r) { return r < rows && (int64_t)targets[r] < cols && row_live(seq_starts, batch, r); };
+    const int64_t unit0 = row_begin * P, units = row_end * P;     // this launch's units: records are indexed by u - unit0
+    auto is_live = [&](int64_t r) { return r < row_end && (int64_t)targets[r] < cols && row_live(seq_starts, batch, r); };
 
     float4 v[kCoopVpt];
     bool loaded = false;
     unsigned round = 0;
-    for (int64_t u = blockIdx.x; u < units; u += G, round++) {
+    for (int64_t u = unit0 + blockIdx.x; u < units; u += G, round++) {
         const int64_t row = u / P;
         const RowBuf x(logits + row * cols, cols), g(grad + row * cols, cols);
         if (!is_live(row)) {
@@ -310,17 +311,17 @@ __global__ __launch_bounds__(kCoopBlock, kCoopWgsPerCu) void ce_coop_kernel(cons
         float m = mine.m, total = mine.s;
         if (P > 1) {
             const unsigned long long tag = coop_tag(launch, round);
-            CoopRec* mine_rec = recs + (size_t)(round & 1u) * kCoopMaxGrid;
+            CoopRec* row_recs = recs + (row - row_begin) * P;     // the row's P records, one per part
             if (threadIdx.x == 0) {
                 missing = 0ull;
-                coop_publish(mine_rec + blockIdx.x, mine.m, mine.s, tag);
+                coop_publish(row_recs + part, mine.m, mine.s, tag);
                 // In place the gradient will overwrite this part's logits: the record has to be out before that, for a
                 // partner that gave up waiting and is reading these logits (it looks at the record again afterwards).
                 if (in_place) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             }
             __syncthreads();
             if (threadIdx.x < (unsigned)P) {                      // one lane per partner (its own part included)
-                const CoopRec* rec = mine_rec + base_wg + threadIdx.x;
+                const CoopRec* rec = row_recs + threadIdx.x;
                 MaxSum got;
                 bool ok = coop_try_read(rec, tag, &got);
                 for (int spin = 0; !ok && spin < spin_limit; spin++) {
@@ -335,23 +336,29 @@ __global__ __launch_bounds__(kCoopBlock, kCoopWgsPerCu) void ce_coop_kernel(cons
             while (todo) {                                        // uniform across the workgroup
                 const int p = __builtin_ctzll(todo);
                 todo &= todo - 1;
-                // that part's statistics from its logits, with the whole workgroup
+                // That part's statistics from its logits, formed as its owner forms them: lane t takes the same
+                // slots (chunks p, p + P, ...) in the same order, and the two reductions are the owner's.  Two sweeps
+                // over memory: the registers hold this workgroup's own part.
                 const float4* src = reinterpret_cast<const float4*>(logits + row * cols);
-                MaxSum ms;
-                ms.m = kNegBig; ms.s = 0.0f;
-                for (int c = p; c < nchunks; c += P) {
-                    const int i4 = c * kCoopBlock + (int)threadIdx.x;
-                    if (i4 < n4) {
-                        const float4 a = src[i4];
-                        const float cm = max4(a);
-                        if (cm > ms.m) { ms.s *= __expf(ms.m - cm); ms.m = cm; }
-                        ms.s += sumexp4(a, ms.m);
-                    }
+                float pm = kNegBig;
+#pragma unroll 1
+                for (int k = 0; k < kCoopVpt; k++) {
+                    const int i4 = (p + k * P) * kCoopBlock + (int)threadIdx.x;
+                    if (i4 < n4) pm = fmaxf(pm, max4(src[i4]));
                 }
-                ms = block_combine<kCoopBlock>(ms, redms);
-                if (threadIdx.x == 0) {                           // (the barrier inside block_combine: every lane's loads have returned)
+                MaxSum ms;
+                ms.m = block_reduce<kCoopBlock, true>(pm, red[0]);
+                const float pmc = ms.m * kLog2e;
+                float ps = 0.0f;
+#pragma unroll 1
+                for (int k = 0; k < kCoopVpt; k++) {
+                    const int i4 = (p + k * P) * kCoopBlock + (int)threadIdx.x;
+                    ps += sum4(exp4(i4 < n4 ? src[i4] : pad, pmc));
+                }
+                ms.s = block_reduce<kCoopBlock, false>(ps, red[1]);
+                if (threadIdx.x == 0) {                           // (after the reductions' barriers: every lane's loads have returned)
                     MaxSum got;
-                    parts[p] = coop_try_read(mine_rec + base_wg + p, tag, &got) ? got : ms;
+                    parts[p] = coop_try_read(row_recs + p, tag, &got) ? got : ms;
                 }
                 __syncthreads();
             }
@@ -521,16 +528,20 @@ extern "C" int seraph_cross_entropy_grad(const float* logits, const uint32_t* ta
         int64_t G = (int64_t)num_compute_units() * kCoopWgsPerCu;
         if (G > kCoopMaxGrid) G = kCoopMaxGrid;
         G = (G / P) * P;
-        if (G > rows * P) G = rows * P;
         static std::atomic<unsigned> launches{0};
-        unsigned launch = launches.fetch_add(1) + 1;
-        if (launch == 0) launch = launches.fetch_add(1) + 1;      // a zeroed record must never look published
-        CoopRec* recs = nullptr;
-        int rc = coop_records(&recs);
+        CoopRec* all_recs = nullptr;
+        int rc = coop_records(&all_recs);
         if (rc != SERAPH_OK) return rc;
-        recs += (size_t)(launch % kCoopLaunchSlots) * 2 * kCoopMaxGrid;
-        hipLaunchKernelGGL(ce_coop_kernel, dim3((unsigned)G), dim3(kCoopBlock), 0, st, logits, targets, grad, loss_rows,
-                           seq_starts, batch, rows, cols, scale, P, recs, launch, g_ce_spin_limit, grad == logits ? 1 : 0);
+        const int64_t rows_per_launch = kCoopMaxUnits / P;        // every unit of a launch keeps a record of its own
+        for (int64_t r0 = 0; r0 < rows; r0 += rows_per_launch) {
+            const int64_t r1 = r0 + rows_per_launch < rows ? r0 + rows_per_launch : rows;
+            const int64_t g = G > (r1 - r0) * P ? (r1 - r0) * P : G;
+            unsigned launch = launches.fetch_add(1) + 1;
+            if (launch == 0) launch = launches.fetch_add(1) + 1;  // a zeroed record must never look published
+            CoopRec* recs = all_recs + (size_t)(launch % kCoopLaunchSlots) * kCoopMaxUnits;
+            hipLaunchKernelGGL(ce_coop_kernel, dim3((unsigned)g), dim3(kCoopBlock), 0, st, logits, targets, grad, loss_rows,
+                               seq_starts, batch, r0, r1, cols, scale, P, recs, launch, g_ce_spin_limit, grad == logits ? 1 : 0);
+        }
     } else if (vec) {
         // Rows in flight are re-read by the second sweep: keep their total under the last-level cache.
         // Two 1024-lane workgroups fit a CU; when that many long rows would overflow the cache, an

@@ -650,6 +650,14 @@ int seraph_add_rmsnorm(const float* x, const float* addend, float* sum, const fl
     return SERAPH_OK;
 }
 
+// Partial rows that rmsnorm_backward_launch writes for a shape, by the kernel it will pick (`aligned`: every
+// operand on a 16-byte boundary).
+static size_t bwd_partial_rows(int64_t rows, int64_t cols, bool aligned) {
+    if (aligned && pick_block_vpl(cols)) return (size_t)bwd_block_grid(rows);                  // one per workgroup
+    if (aligned && cols <= 512 && pick_vpl(cols)) return (size_t)bwd_grid(rows);               // one per workgroup
+    return (size_t)bwd_grid(rows) * kWavesPerBlock;                                            // one per wave
+}
+
 size_t seraph_rmsnorm_backward_ws_bytes(int64_t rows, int64_t cols) {
     if (rows <= 0 || cols <= 0) return 0;
     // the generic path needs one partial row per wave, the register path one per block
@@ -775,16 +783,19 @@ int seraph_rmsnorm_backward_static(const float* x, const float* scale, const flo
     if (rows == 0 || cols == 0) return SERAPH_OK;
     SERAPH_REQUIRE(x && scale && dy && dx && grad_scale, "rmsnorm_backward_static: NULL pointer");
     SERAPH_REQUIRE(rows > 0 && cols > 0, "rmsnorm_backward_static: bad shape");
-    const size_t need = seraph_rmsnorm_backward_ws_bytes(rows, cols);
+    float* partial = nullptr;
+    int rc = static_scratch(&partial);
+    if (rc != SERAPH_OK) return rc;
+    // what the kernel that these operands select will write (the workspace query answers for any alignment)
+    const bool aligned = aligned16(x) && aligned16(scale) && aligned16(dy) && aligned16(dx) && aligned16(partial) &&
+                         (!residual || aligned16(residual));
+    const size_t need = bwd_partial_rows(rows, cols, aligned) * (size_t)cols * sizeof(float);
     if (need > kStaticScratchBytes) {
         set_error("rmsnorm_backward_static: %lld x %lld needs %zu bytes of scratch, the built-in array holds %zu; "
                   "use seraph_rmsnorm_backward_residual with a workspace", (long long)rows, (long long)cols, need,
                   kStaticScratchBytes);
         return SERAPH_ERR_WORKSPACE;
     }
-    float* partial = nullptr;
-    int rc = static_scratch(&partial);
-    if (rc != SERAPH_OK) return rc;
     return rmsnorm_backward_launch(x, scale, dy, residual, dx, grad_scale, rows, cols, eps, partial, s);
 }
 

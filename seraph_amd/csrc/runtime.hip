@@ -18,7 +18,10 @@ hipEvent_t take_armed_event() {
 }
 static int g_cu_count = 0;
 
+// Every error path of the library goes through here: an op that fails before its last launch must not leave its
+// caller's event armed for whatever op the thread calls next.
 void set_error(const char* fmt, ...) {
+    g_armed_event = nullptr;
     va_list ap;
     va_start(ap, fmt);
     vsnprintf(g_err, sizeof(g_err), fmt, ap);

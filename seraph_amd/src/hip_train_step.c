@@ -732,6 +732,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
     seraph_stream_t s = t->stream;
     const float* P = t->P;
 
+    seraph_hip_event_on_next_op(NULL);      /* an event this thread armed before the step belongs to none of its ops */
     if (upload_batch(t, tokens, total_tokens, seq_starts, batch)) return -1.0f;
     const uint32_t* starts = t->d_starts;
 

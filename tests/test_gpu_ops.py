@@ -649,22 +649,45 @@ def test_cross_entropy_long_rows_when_partners_are_not_waited_for(ops, orc, spin
     would for a partner that has not been scheduled: same results, also in place and with unsupervised rows."""
     from seraph_amd._lib import kernels
     r = rng(91)
-    try:
-        kernels().seraph_cross_entropy_exchange_spins(spins)
-        for rows, cols in ((5, 40000), (9, 151936), (1100, 36000)):
-            x = (2 * r.standard_normal((rows, cols))).astype(np.float32)
-            t = r.integers(0, cols, rows).astype(np.uint32)
-            t[1] = cols
-            starts = np.array([0, 3, rows], np.uint32)
-            rg, rl = orc.cross_entropy_grad_packed(x, t, starts, rows - 3)
-            sd = dev(starts.view(np.int32))
+    for rows, cols in ((5, 40000), (9, 151936), (1100, 36000)):
+        x = (2 * r.standard_normal((rows, cols))).astype(np.float32)
+        t = r.integers(0, cols, rows).astype(np.uint32)
+        t[1] = cols
+        starts = np.array([0, 3, rows], np.uint32)
+        rg, rl = orc.cross_entropy_grad_packed(x, t, starts, rows - 3)
+        sd = dev(starts.view(np.int32))
+        g_waited, l_waited = ops.cross_entropy_grad(dev(x), dev(t.view(np.int32)), rows - 3, seq_starts=sd)
+        try:
+            kernels().seraph_cross_entropy_exchange_spins(spins)
             g, l = ops.cross_entropy_grad(dev(x), dev(t.view(np.int32)), rows - 3, seq_starts=sd)
-            parity(g, rg, "grad", atol=1e-7); parity(l, rl, "loss")
             X = dev(x)
             g2, l2 = ops.cross_entropy_grad(X, dev(t.view(np.int32)), rows - 3, seq_starts=sd, grad=X)
-            parity(g2, rg, "grad in place", atol=1e-7); parity(l2, rl, "loss in place")
-    finally:
-        kernels().seraph_cross_entropy_exchange_spins(1 << 16)
+            torch.cuda.synchronize()
+        finally:
+            kernels().seraph_cross_entropy_exchange_spins(1 << 16)
+        parity(g, rg, "grad", atol=1e-7); parity(l, rl, "loss")
+        parity(g2, rg, "grad in place", atol=1e-7); parity(l2, rl, "loss in place")
+        # a part's statistics formed by a partner are the owner's own bits: whoever waited for whom, nothing changes
+        assert torch.equal(g, g_waited) and torch.equal(l, l_waited)
+        assert torch.equal(g2, g_waited) and torch.equal(l2, l_waited)
+
+
+def test_cross_entropy_long_rows_in_more_than_one_launch(ops, orc):
+    """Every (row, part) unit of a launch has an exchange record of its own (2^18 per launch); 140000 rows in two parts
+    need two launches.  Sampled rows against the oracle, row sums, and the in-place form bit for bit."""
+    rows, cols = 140000, 33792
+    torch.manual_seed(5)
+    x = torch.randn(rows, cols, device="cuda") * 2
+    t = torch.randint(0, cols, (rows,), device="cuda", dtype=torch.int32)
+    g, l = ops.cross_entropy_grad(x, t, rows)
+    pick = np.array([0, 1, 131071, 131072, 131073, rows - 1])
+    xs, ts = x[pick].cpu().numpy(), t[pick].cpu().numpy().astype(np.uint32)
+    rg, rl = orc.cross_entropy_grad(xs, ts, len(pick))
+    parity(g[pick] * (rows / len(pick)), rg, "grad of sampled rows", atol=1e-7)
+    parity(l[pick], rl, "loss of sampled rows")
+    assert float(g.sum(dim=1).abs().max()) < 1e-9
+    g2, l2 = ops.cross_entropy_grad(x, t, rows, grad=x)
+    assert torch.equal(g2, g) and torch.equal(l2, l)
 
 
 @pytest.mark.parametrize("rows,cols", [(4, 40000), (3, 151936), (300, 151936), (2100, 77828), (40, 1000000)])
@@ -694,10 +717,10 @@ def test_cross_entropy_long_rows_are_deterministic_and_alias_safe(ops, rows, col
 @pytest.mark.parametrize("case", ["one token", "few tokens", "pairs", "mixed"])
 def test_embedding_backward_repeated_tokens(ops, orc, case, h):
     """Groups of every size: a batch that is one token repeated (a padding-dominated batch), a handful of tokens, every
-    token twice, and a mixture whose groups straddle the lengths at which the gathering changes method (16), at which a
-    group is cut along the row's width (128, for rows of more than 256 columns: 520 has a ragged third slab, 2048 has
-    eight) and the batch size of the gather list (1024).  Integer-valued gradients: the sums are exact, so the check is
-    bit-exact."""
+    token twice, and a mixture whose groups straddle the length from which a group is cut along the row's width (16, for
+    rows of more than 256 columns: 520 has a ragged third slab, 2048 has eight; narrower rows are gathered by one
+    wavefront at any length) and the batch size of the gather list (1024).  Integer-valued gradients: the sums are
+    exact, so the check is bit-exact."""
     r = rng(15)
     T, V = 5000, 3000
     if case == "one token":
@@ -723,3 +746,23 @@ def test_embedding_backward_repeated_tokens(ops, orc, case, h):
     b = ops.embedding_backward(dev(tok.view(np.int32)), dev(dF), dev(base))
     assert torch.equal(a, b)
     parity(a, orc.embedding_backward(tok, dF, base), "embedding backward", atol=1e-4)
+
+
+def test_embedding_backward_more_column_slabs_than_positions(ops, orc):
+    """Rows of 9000 floats are 36 column slabs; a token that occurs 16 to 35 times has fewer positions than slabs, so its
+    takers have to come back for more than one slab each.  Also repeated calls: the tables that the library keeps between
+    calls carry the call's number, so what an earlier call left in them must count as empty."""
+    r = rng(17)
+    T, V, h = 700, 500, 9000
+    sizes = [16, 17, 20, 35, 36, 37, 100]
+    tok = np.concatenate([np.full(n, 3 + 7 * i, np.uint32) for i, n in enumerate(sizes)] +
+                         [r.integers(100, V, T - sum(sizes)).astype(np.uint32)])
+    tok = tok[r.permutation(T)]
+    dH = r.integers(-8, 9, (T, h)).astype(np.float32)
+    base = r.integers(-3, 4, (V, h)).astype(np.float32)
+    ref = orc.embedding_backward(tok, dH, base)
+    for _ in range(6):                                         # more calls than the library has tables
+        got = host(ops.embedding_backward(dev(tok.view(np.int32)), dev(dH), dev(base)))
+        assert (got == ref).all()
+    tok2 = tok[::-1].copy()                                    # other owners, other chains, the same tables
+    assert (host(ops.embedding_backward(dev(tok2.view(np.int32)), dev(dH), dev(base))) == orc.embedding_backward(tok2, dH, base)).all()

@@ -44,6 +44,13 @@ def test_static_scratch_matches_workspace_form_on_two_calls_in_a_row(ops):
     _case(ops, 5, 333, 5, residual=False)
 
 
+def test_static_scratch_takes_the_training_shape(ops):
+    """16384 x 2048 with the residual: 512 partial rows of 8 KiB, a quarter of the array (the workspace query, which
+    answers for any alignment, asks for 32 MiB here), then a smaller call on the same array."""
+    _case(ops, 16384, 2048, 6, residual=True)
+    _case(ops, 2000, 1024, 7, residual=False)
+
+
 def test_static_scratch_refuses_shapes_beyond_its_size(ops):
     from seraph_amd._lib import kernels
     k = kernels()
