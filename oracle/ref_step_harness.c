@@ -11,7 +11,9 @@
  * for the ops (those are this build's kernels); it cross-checks the op ORDER of the
  * oracle's step against the reference's own driver.
  *
- * usage: ref_step_hip [--cpu] [--time] <in.bin> <out.bin>
+ * usage: ref_step_hip [--cpu] [--time] [--profile] <in.bin> <out.bin>
+ *   --profile : the backend's vulkan_profiler_* is switched on around every step (nothing in the reference calls it;
+ *            it is the interface of include/vulkan_backend.h:638-642) and prints its report to stdout
  *   --cpu  : no backend is created, so train_step takes the reference's CPU path (src/train.c:6842-6983:
  *            train_forward_fp32, the scalar loss loops, train_backward, the CPU AdamW); full-weight mode only.
  *            This is the timed "reference" CPU baseline; its gradients are NOT those of the GPU path
@@ -47,10 +49,11 @@ static double now_s(void) {
 }
 
 int main(int argc, char** argv) {
-    int cpu_only = 0, timed = 0;
+    int cpu_only = 0, timed = 0, profile = 0;
     while (argc > 1 && argv[1][0] == '-' && argv[1][1] == '-') {
         if (!strcmp(argv[1], "--cpu")) cpu_only = 1;
         else if (!strcmp(argv[1], "--time")) timed = 1;
+        else if (!strcmp(argv[1], "--profile")) profile = 1;
         else { fprintf(stderr, "unknown option %s\n", argv[1]); return 2; }
         argv++; argc--;
     }
@@ -170,11 +173,14 @@ int main(int argc, char** argv) {
 
     float* loss = malloc((size_t)steps * sizeof(float));
     double t_first = 0.0, t_rest = 0.0;
+    if (profile) vulkan_profiler_enable(ctx);
     for (int s = 0; s < steps; s++) {                    /* train_step returns after its submit-and-wait and loss download */
+        if (profile) vulkan_profiler_begin_step(ctx);
         const double t0 = now_s();
         loss[s] = train_step(&st, tokens + (size_t)s * T, T);
         const double dt = now_s() - t0;
         if (s == 0) t_first = dt; else t_rest += dt;
+        if (profile) vulkan_profiler_end_step(ctx, s + 1, T, loss[s]);
     }
     if (timed) printf("seconds_per_step %.6f\n", steps > 1 ? t_rest / (steps - 1) : t_first);
 

@@ -651,8 +651,12 @@ void cuda_download_lora_weights(cuda_train_context_t* ctx, void* lora_ptr) {
 /* Every device buffer the trainer created through cuda_train_buffer_create is on the live list:
  * releasing the list releases the context's weights, moments, caches and LoRA state whatever
  * fields they hang from.  The small host arrays of pointers are released through the list below. */
+/* hip_fused_step.c, when it is part of the link: the fused trainer that serves this context goes first */
+__attribute__((weak)) void hip_fused_step_release(cuda_train_context_t* ctx);
+
 void cuda_train_free(cuda_train_context_t* ctx) {
     if (!ctx) return;
+    if (hip_fused_step_release) hip_fused_step_release(ctx);
     hc_state_t* st = state_of(ctx);
     if (st) {
         seraph_hip_stream_sync(st->stream);

@@ -9,6 +9,7 @@
  * gets from its barrier after every recorded op (src/vulkan_backend_backward.c:124-142).
  */
 #include <math.h>
+#include <stdarg.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -47,8 +48,8 @@ void* hip_backend_scratch(vulkan_context_t* ctx, size_t bytes) {
 }
 
 /* ------------------------------------------------------------------ profiler
- * hipEvent pairs per op; vulkan_profiler_end_step prints the per-op table and a roll-up
- * by op-name substring, like src/vulkan_backend.c:105-210. */
+ * hipEvent pairs per op, named as the reference names its ops; vulkan_profiler_end_step prints the
+ * reference's report (src/vulkan_backend.c:105-207). */
 void hip_prof_begin(vulkan_context_t* ctx, const char* name) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !ctx->profiling || st->prof_count >= HIP_PROF_MAX_OPS) return;
@@ -59,7 +60,8 @@ void hip_prof_begin(vulkan_context_t* ctx, const char* name) {
         if (seraph_hip_event_create(&op->ev_start) != SERAPH_OK || seraph_hip_event_create(&op->ev_stop) != SERAPH_OK) return;
         st->prof_events_made = st->prof_count + 1;
     }
-    op->name = name;
+    strncpy(op->name, name, sizeof(op->name) - 1);
+    op->name[sizeof(op->name) - 1] = '\0';
     seraph_hip_event_record(op->ev_start, st->stream);
 }
 
@@ -82,28 +84,86 @@ void vulkan_profiler_begin_step(vulkan_context_t* ctx) {
     ctx->prof_num_ops = 0;
 }
 
+/* Both to stdout and to the log file, as the reference's PROF_LOG (src/vulkan_backend.c:25-28). */
+static void prof_log(vulkan_context_t* ctx, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vprintf(fmt, ap);
+    va_end(ap);
+    if (ctx->prof_log) {
+        va_start(ap, fmt);
+        vfprintf((FILE*)ctx->prof_log, fmt, ap);
+        va_end(ap);
+        fflush((FILE*)ctx->prof_log);
+    }
+}
+
+/* The report of src/vulkan_backend.c:105-207: header, nine categories found by substrings of the op names, one line
+ * per op.  The Grid / Block column stays empty (as it does in the reference for an op that records no launch shape):
+ * the kernel library chooses its launches itself and an op may be several of them. */
 void vulkan_profiler_end_step(vulkan_context_t* ctx, int step, int seq_len, float loss) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !ctx->profiling || st->prof_count == 0) return;
-    FILE* out = ctx->prof_log ? (FILE*)ctx->prof_log : stderr;
-    static const char* cats[] = {"matmul", "attention", "rmsnorm", "rope", "cross_entropy", "adamw", "embed", "silu", "mul", "add", "copy", "fill"};
-    enum { NCAT = sizeof(cats) / sizeof(cats[0]) };
-    double cat_ms[NCAT + 1] = {0}, total = 0.0;
+    if (!st || !ctx->profiling || !st->prof_ops || st->prof_count == 0) return;
+    const int nops = st->prof_count;
     seraph_hip_stream_sync(st->stream);
-    fprintf(out, "[HIP PROFILE] step=%d seq=%d loss=%.6f ops=%d\n", step, seq_len, loss, st->prof_count);
-    for (int i = 0; i < st->prof_count; i++) {
+    float* ms_of = (float*)calloc((size_t)nops, sizeof(float));
+    if (!ms_of) return;
+    double total_ms = 0;
+    double cat_matmul = 0, cat_attn = 0, cat_attn_bwd = 0, cat_rmsnorm = 0, cat_rmsnorm_bwd = 0;
+    double cat_cross_entropy = 0, cat_adamw = 0, cat_copy = 0, cat_other = 0;
+    for (int i = 0; i < nops; i++) {
         float ms = 0.f;
         seraph_hip_event_elapsed_ms(st->prof_ops[i].ev_start, st->prof_ops[i].ev_stop, &ms);
-        total += ms;
-        int c = NCAT;
-        for (int k = 0; k < NCAT; k++) if (strstr(st->prof_ops[i].name, cats[k])) { c = k; break; }
-        cat_ms[c] += ms;
-        fprintf(out, "  %4d %-32s %9.3f ms\n", i, st->prof_ops[i].name, ms);
+        ms_of[i] = ms;
+        total_ms += ms;
+        const char* n = st->prof_ops[i].name;
+        if (strstr(n, "matmul"))           cat_matmul += ms;
+        else if (strstr(n, "attn_bwd"))    cat_attn_bwd += ms;
+        else if (strstr(n, "attn"))        cat_attn += ms;
+        else if (strstr(n, "rmsnorm_bwd")) cat_rmsnorm_bwd += ms;
+        else if (strstr(n, "rmsnorm"))     cat_rmsnorm += ms;
+        else if (strstr(n, "cross_ent"))   cat_cross_entropy += ms;
+        else if (strstr(n, "adamw"))       cat_adamw += ms;
+        else if (strstr(n, "copy") || strstr(n, "fill") || strstr(n, "barrier")) cat_copy += ms;
+        else                               cat_other += ms;
     }
-    for (int k = 0; k <= NCAT; k++)
-        if (cat_ms[k] > 0) fprintf(out, "  [%s] %.3f ms (%.1f%%)\n", k < NCAT ? cats[k] : "other", cat_ms[k], 100.0 * cat_ms[k] / total);
-    fprintf(out, "  [total] %.3f ms\n", total);
-    fflush(out);
+    if (total_ms <= 0) total_ms = 1e-6;
+
+    prof_log(ctx, "\n");
+    prof_log(ctx, "  ══════════════════════════════════════════════════════════════════\n");
+    prof_log(ctx, "  SERAPH VULKAN STEP PROFILER (step %d, seq=%d, loss=%.4f)\n", step, seq_len, loss);
+    prof_log(ctx, "  %d operations, %.2f ms total\n", nops, total_ms);
+    prof_log(ctx, "  ══════════════════════════════════════════════════════════════════\n");
+    prof_log(ctx, "\n  ── CATEGORY BREAKDOWN ──\n\n");
+    prof_log(ctx, "  %-24s %10s  %6s  %s\n", "Category", "Time (ms)", "%", "Bar");
+    prof_log(ctx, "  %-24s %10s  %6s  %s\n", "------------------------", "----------", "------",
+             "----------------------------------------");
+    const struct { const char* name; double ms; } cats[] = {
+        {"matmul (all)", cat_matmul}, {"attention fwd", cat_attn}, {"attention bwd", cat_attn_bwd},
+        {"rmsnorm fwd", cat_rmsnorm}, {"rmsnorm bwd", cat_rmsnorm_bwd}, {"cross_entropy", cat_cross_entropy},
+        {"adamw", cat_adamw}, {"copy/fill", cat_copy}, {"other", cat_other},
+    };
+    for (size_t i = 0; i < sizeof(cats) / sizeof(cats[0]); i++) {
+        const double pct = 100.0 * cats[i].ms / total_ms;
+        int bar_len = (int)(pct * 0.4);
+        if (bar_len > 40) bar_len = 40;
+        char bar[41];
+        memset(bar, '#', (size_t)bar_len);
+        bar[bar_len] = '\0';
+        prof_log(ctx, "  %-24s %10.3f  %5.1f%%  %s\n", cats[i].name, cats[i].ms, pct, bar);
+    }
+    prof_log(ctx, "\n  ── PER-OPERATION DETAIL ──\n\n");
+    prof_log(ctx, "  %4s  %-60s %10s  %5s  %s\n", "#", "Operation", "Time (ms)", "%", "Grid / Block");
+    prof_log(ctx, "  %4s  %-60s %10s  %5s  %s\n", "----", "------------------------------------------------------------",
+             "----------", "-----", "------------------");
+    for (int i = 0; i < nops; i++) {
+        const double pct = 100.0 * ms_of[i] / total_ms;
+        const char* marker = (pct > 5.0) ? " <<<" : (pct > 1.0) ? " <<" : "";
+        prof_log(ctx, "  %4d  %-60s %10.3f  %4.1f%%  %-20s%s\n", i, st->prof_ops[i].name, ms_of[i], pct, "", marker);
+    }
+    prof_log(ctx, "\n");
+    fflush(stdout);
+    free(ms_of);
 }
 
 /* ------------------------------------------------------------------ init / free */
@@ -278,7 +338,8 @@ static void backend_gemm(vulkan_context_t* ctx, hip_state_t* st, const char* wha
                          int M, int N, int K, int tA, int tB, int accumulate) {
     const size_t need = seraph_gemm_scaled_ws_bytes(M, N, K, tA, tB);
     void* ws = need ? hip_backend_scratch(ctx, need) : NULL;
-    HIP_OP(ctx, what, seraph_gemm_scaled(A, B, C, M, N, K, tA, tB, accumulate, 1.0f, ws, ws ? need : 0, st->stream));
+    HIP_OPF(ctx, seraph_gemm_scaled(A, B, C, M, N, K, tA, tB, accumulate, 1.0f, ws, ws ? need : 0, st->stream),
+            "%s [%dx%d K=%d]", what, M, N, K);                        /* src/vulkan_backend.c:1674, :1848 */
 }
 
 void hip_matmul_scaled(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C,
@@ -287,8 +348,8 @@ void hip_matmul_scaled(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_
     if (!st || !A || !B || !C) return;
     const size_t need = seraph_gemm_scaled_ws_bytes(M, N, K, transpose_A, transpose_B);
     void* ws = need ? hip_backend_scratch(ctx, need) : NULL;
-    HIP_OP(ctx, "matmul_scaled", seraph_gemm_scaled(FPTR(A), FPTR(B), FPTR(C), M, N, K, transpose_A, transpose_B, accumulate, alpha,
-                                                    ws, ws ? need : 0, st->stream));
+    HIP_OPF(ctx, seraph_gemm_scaled(FPTR(A), FPTR(B), FPTR(C), M, N, K, transpose_A, transpose_B, accumulate, alpha,
+                                    ws, ws ? need : 0, st->stream), "matmul_scaled [%dx%d K=%d]", M, N, K);
 }
 
 void vulkan_matmul(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C, int M, int N, int K) {
@@ -301,7 +362,7 @@ void vulkan_matmul_transpose(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_b
                              int M, int N, int K, int transpose_A, int transpose_B, int accumulate) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !A || !B || !C) return;
-    backend_gemm(ctx, st, "matmul_transpose", FPTR(A), FPTR(B), FPTR(C), M, N, K, transpose_A, transpose_B, accumulate);
+    backend_gemm(ctx, st, "matmul_t", FPTR(A), FPTR(B), FPTR(C), M, N, K, transpose_A, transpose_B, accumulate);
 }
 
 void vulkan_add(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C, size_t count) {
@@ -338,7 +399,7 @@ void vulkan_rmsnorm(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer
                     int rows, int cols, float eps) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !input || !scale || !output) return;
-    HIP_OP(ctx, "rmsnorm", seraph_rmsnorm(FPTR(input), FPTR(scale), FPTR(output), rows, cols, eps, st->stream));
+    HIP_OPF(ctx, seraph_rmsnorm(FPTR(input), FPTR(scale), FPTR(output), rows, cols, eps, st->stream), "rmsnorm [%dx%d] %u-thr", rows, cols, ctx->wg_size_1d);
 }
 
 /* vulkan_add of a residual branch and the vulkan_rmsnorm that reads the sum (src/train.c:4705-4711): sum = input + addend,
@@ -347,21 +408,21 @@ void hip_add_rmsnorm(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffe
                      vulkan_buffer_t* scale, vulkan_buffer_t* output, int rows, int cols, float eps) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !input || !addend || !sum || !scale || !output) return;
-    HIP_OP(ctx, "add_rmsnorm", seraph_add_rmsnorm(FPTR(input), FPTR(addend), FPTR(sum), FPTR(scale), FPTR(output), rows, cols, eps, st->stream));
+    HIP_OPF(ctx, seraph_add_rmsnorm(FPTR(input), FPTR(addend), FPTR(sum), FPTR(scale), FPTR(output), rows, cols, eps, st->stream), "add+rmsnorm [%dx%d] %u-thr", rows, cols, ctx->wg_size_1d);
 }
 
 void vulkan_rope(vulkan_context_t* ctx, vulkan_buffer_t* x_in, vulkan_buffer_t* x_out,
                  int seq_len, int num_heads, int head_dim, float rope_theta) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !x_in || !x_out) return;
-    HIP_OP(ctx, "rope", seraph_rope(FPTR(x_in), FPTR(x_out), NULL, 1, seq_len, num_heads, head_dim, rope_theta, 0, st->stream));
+    HIP_OP(ctx, "rope_fwd", seraph_rope(FPTR(x_in), FPTR(x_out), NULL, 1, seq_len, num_heads, head_dim, rope_theta, 0, st->stream));
 }
 
 void hip_rope_packed(vulkan_context_t* ctx, vulkan_buffer_t* x_in, vulkan_buffer_t* x_out, vulkan_buffer_t* seq_starts,
                      int total_tokens, int batch_size, int num_heads, int head_dim, float rope_theta) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !x_in || !x_out || !seq_starts) return;
-    HIP_OP(ctx, "rope_packed", seraph_rope(FPTR(x_in), FPTR(x_out), UPTR(seq_starts), batch_size, total_tokens, num_heads, head_dim, rope_theta, 0, st->stream));
+    HIP_OP(ctx, "rope_fwd_packed", seraph_rope(FPTR(x_in), FPTR(x_out), UPTR(seq_starts), batch_size, total_tokens, num_heads, head_dim, rope_theta, 0, st->stream));
 }
 
 void vulkan_batch_attention(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulkan_buffer_t* K, vulkan_buffer_t* V,
@@ -369,8 +430,8 @@ void vulkan_batch_attention(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulkan_bu
     hip_state_t* st = hip_state(ctx);
     if (!st || !Q || !K || !V || !out) return;
     float scale = 1.0f / sqrtf((float)head_dim);          /* src/vulkan_backend.c:2980-2984 */
-    HIP_OP(ctx, "batch_attention", seraph_attention_forward(FPTR(Q), FPTR(K), FPTR(V), FPTR(out), NULL, NULL, 1, seq_len,
-                                                            num_heads, kv_heads, head_dim, scale, st->stream));
+    HIP_OPF(ctx, seraph_attention_forward(FPTR(Q), FPTR(K), FPTR(V), FPTR(out), NULL, NULL, 1, seq_len,
+                                                            num_heads, kv_heads, head_dim, scale, st->stream), "attn_fwd [seq=%d h=%d hd=%d]", seq_len, num_heads, head_dim);
 }
 
 void hip_batch_attention_packed(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulkan_buffer_t* K, vulkan_buffer_t* V,
@@ -379,9 +440,9 @@ void hip_batch_attention_packed(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulka
     hip_state_t* st = hip_state(ctx);
     if (!st || !Q || !K || !V || !out || !seq_starts) return;
     float scale = 1.0f / sqrtf((float)head_dim);
-    HIP_OP(ctx, "batch_attention_packed", seraph_attention_forward(FPTR(Q), FPTR(K), FPTR(V), FPTR(out), lse_out ? FPTR(lse_out) : NULL,
+    HIP_OPF(ctx, seraph_attention_forward(FPTR(Q), FPTR(K), FPTR(V), FPTR(out), lse_out ? FPTR(lse_out) : NULL,
                                                                    UPTR(seq_starts), batch_size, total_tokens,
-                                                                   num_heads, kv_heads, head_dim, scale, st->stream));
+                                                                   num_heads, kv_heads, head_dim, scale, st->stream), "attn_fwd_packed [tok=%d seqs=%d h=%d hd=%d]", total_tokens, batch_size, num_heads, head_dim);
 }
 
 void vulkan_embed_lookup(vulkan_context_t* ctx, vulkan_buffer_t* tokens_u32, vulkan_buffer_t* embed_weight,
@@ -403,7 +464,7 @@ void hip_adamw_update_clipped(vulkan_context_t* ctx, vulkan_buffer_t* weight, vu
                               int step, size_t size, float clip) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !weight || !grad || !m || !v || size == 0) return;
-    HIP_OP(ctx, "adamw", seraph_adamw(FPTR(weight), FPTR(grad), FPTR(m), FPTR(v), size, lr, beta1, beta2, weight_decay, eps, step, clip, st->stream));
+    HIP_OPF(ctx, seraph_adamw(FPTR(weight), FPTR(grad), FPTR(m), FPTR(v), size, lr, beta1, beta2, weight_decay, eps, step, clip, st->stream), "adamw [%zu] %u-thr", (size_t)size, ctx->wg_size_1d);
 }
 
 void hip_adamw_update_multi(vulkan_context_t* ctx, int count, vulkan_buffer_t* const* weights, vulkan_buffer_t* const* grads,
@@ -420,7 +481,7 @@ void hip_adamw_update_multi(vulkan_context_t* ctx, int count, vulkan_buffer_t* c
         list[k].n = sizes[i];
         k++;
     }
-    HIP_OP(ctx, "adamw", seraph_adamw_multi(list, k, lr, beta1, beta2, weight_decay, eps, step, clip, st->stream));
+    HIP_OPF(ctx, seraph_adamw_multi(list, k, lr, beta1, beta2, weight_decay, eps, step, clip, st->stream), "adamw [%d tensors] %u-thr", k, ctx->wg_size_1d);
     free(list);
 }
 

@@ -14,8 +14,8 @@ void vulkan_cross_entropy_grad(vulkan_context_t* ctx, vulkan_buffer_t* logits, v
                                vulkan_buffer_t* grad_logits, vulkan_buffer_t* loss_rows, int rows, int cols, int valid_rows) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !logits || !targets_u32 || !grad_logits || !loss_rows) return;
-    HIP_OP(ctx, "cross_entropy_grad", seraph_cross_entropy_grad(FPTR(logits), UPTR(targets_u32), FPTR(grad_logits), FPTR(loss_rows),
-                                                               NULL, 1, rows, cols, valid_rows, st->stream));
+    HIP_OPF(ctx, seraph_cross_entropy_grad(FPTR(logits), UPTR(targets_u32), FPTR(grad_logits), FPTR(loss_rows),
+                                                               NULL, 1, rows, cols, valid_rows, st->stream), "cross_entropy_grad [%dx%d] %u-thr", rows, cols, ctx->wg_size_1d);
 }
 
 void hip_cross_entropy_grad_packed(vulkan_context_t* ctx, vulkan_buffer_t* logits, vulkan_buffer_t* targets_u32,
@@ -23,9 +23,9 @@ void hip_cross_entropy_grad_packed(vulkan_context_t* ctx, vulkan_buffer_t* logit
                                    int total_tokens, int batch_size, int vocab_size, int num_valid_predictions) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !logits || !targets_u32 || !grad_logits || !loss_rows || !seq_starts) return;
-    HIP_OP(ctx, "cross_entropy_grad_packed", seraph_cross_entropy_grad(FPTR(logits), UPTR(targets_u32), FPTR(grad_logits), FPTR(loss_rows),
+    HIP_OPF(ctx, seraph_cross_entropy_grad(FPTR(logits), UPTR(targets_u32), FPTR(grad_logits), FPTR(loss_rows),
                                                                       UPTR(seq_starts), batch_size, total_tokens, vocab_size,
-                                                                      num_valid_predictions, st->stream));
+                                                                      num_valid_predictions, st->stream), "cross_entropy_grad_packed [%dx%d] %u-thr", total_tokens, vocab_size, ctx->wg_size_1d);
 }
 
 /* src/vulkan_backend_backward.c:691-800: 512 inputs per output (src/train.c:4906-4913) */
@@ -44,8 +44,8 @@ void vulkan_rmsnorm_backward_batch(vulkan_context_t* ctx, vulkan_buffer_t* input
     size_t need = seraph_rmsnorm_backward_ws_bytes(rows, cols);
     void* ws = hip_backend_scratch(ctx, need);
     if (!ws) return;
-    HIP_OP(ctx, "rmsnorm_backward_batch", seraph_rmsnorm_backward(FPTR(input), FPTR(scale), FPTR(grad_output), FPTR(grad_input),
-                                                                  FPTR(grad_scale), rows, cols, eps, ws, st->ws_bytes, st->stream));
+    HIP_OPF(ctx, seraph_rmsnorm_backward(FPTR(input), FPTR(scale), FPTR(grad_output), FPTR(grad_input),
+                                                                  FPTR(grad_scale), rows, cols, eps, ws, st->ws_bytes, st->stream), "rmsnorm_bwd [%dx%d] %u-thr", rows, cols, ctx->wg_size_1d);
 }
 
 /* vulkan_rmsnorm_backward_batch and the vulkan_add of the residual gradient that follows it (src/train.c:5180-5193):
@@ -58,9 +58,9 @@ void hip_rmsnorm_backward_residual(vulkan_context_t* ctx, vulkan_buffer_t* input
     size_t need = seraph_rmsnorm_backward_ws_bytes(rows, cols);
     void* ws = hip_backend_scratch(ctx, need);
     if (!ws) return;
-    HIP_OP(ctx, "rmsnorm_backward_residual", seraph_rmsnorm_backward_residual(FPTR(input), FPTR(scale), FPTR(grad_output), FPTR(residual),
+    HIP_OPF(ctx, seraph_rmsnorm_backward_residual(FPTR(input), FPTR(scale), FPTR(grad_output), FPTR(residual),
                                                                               FPTR(grad_input), FPTR(grad_scale), rows, cols, eps, ws,
-                                                                              st->ws_bytes, st->stream));
+                                                                              st->ws_bytes, st->stream), "rmsnorm_bwd+add [%dx%d] %u-thr", rows, cols, ctx->wg_size_1d);
 }
 
 /* The row pass of vulkan_rmsnorm_backward_batch alone (residual may be NULL): grad_input is complete, and the column
@@ -74,9 +74,9 @@ int hip_rmsnorm_backward_rows(vulkan_context_t* ctx, vulkan_buffer_t* input, vul
     hip_state_t* st = hip_state(ctx);
     if (!st || !input || !scale || !grad_output || !grad_input || !partial) return 0;
     int nparts = 0;
-    HIP_OP(ctx, "rmsnorm_backward_rows", seraph_rmsnorm_backward_rows(FPTR(input), FPTR(scale), FPTR(grad_output),
+    HIP_OPF(ctx, seraph_rmsnorm_backward_rows(FPTR(input), FPTR(scale), FPTR(grad_output),
                                                                       residual ? FPTR(residual) : NULL, FPTR(grad_input), rows, cols, eps,
-                                                                      DPTR(partial), partial->size, &nparts, st->stream));
+                                                                      DPTR(partial), partial->size, &nparts, st->stream), "rmsnorm_bwd_rows [%dx%d] %u-thr", rows, cols, ctx->wg_size_1d);
     return nparts;
 }
 
@@ -95,7 +95,7 @@ void hip_rmsnorm_colsum_multi(vulkan_context_t* ctx, int count, vulkan_buffer_t*
         jobs[k].partial = FPTR(partial[i]); jobs[k].nparts = nparts[i]; jobs[k].grad_scale = FPTR(grad_scale[i]);
         k++;
     }
-    HIP_OP(ctx, "rmsnorm_colsum_multi", seraph_rmsnorm_colsum_multi(jobs, k, cols, st->stream));
+    HIP_OP(ctx, "rmsnorm_bwd_colsum", seraph_rmsnorm_colsum_multi(jobs, k, cols, st->stream));
     free(jobs);
 }
 
@@ -104,14 +104,14 @@ void vulkan_rope_backward(vulkan_context_t* ctx, vulkan_buffer_t* x_in, vulkan_b
                           int seq_len, int num_heads, int head_dim, float rope_theta) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !x_in || !x_out) return;
-    HIP_OP(ctx, "rope_backward", seraph_rope(FPTR(x_in), FPTR(x_out), NULL, 1, seq_len, num_heads, head_dim, rope_theta, 1, st->stream));
+    HIP_OP(ctx, "rope_bwd", seraph_rope(FPTR(x_in), FPTR(x_out), NULL, 1, seq_len, num_heads, head_dim, rope_theta, 1, st->stream));
 }
 
 void hip_rope_backward_packed(vulkan_context_t* ctx, vulkan_buffer_t* x_in, vulkan_buffer_t* x_out, vulkan_buffer_t* seq_starts,
                               int total_tokens, int batch_size, int num_heads, int head_dim, float rope_theta) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !x_in || !x_out || !seq_starts) return;
-    HIP_OP(ctx, "rope_backward_packed", seraph_rope(FPTR(x_in), FPTR(x_out), UPTR(seq_starts), batch_size, total_tokens, num_heads,
+    HIP_OP(ctx, "rope_bwd_packed", seraph_rope(FPTR(x_in), FPTR(x_out), UPTR(seq_starts), batch_size, total_tokens, num_heads,
                                                     head_dim, rope_theta, 1, st->stream));
 }
 
@@ -128,9 +128,9 @@ void vulkan_batch_attention_backward(vulkan_context_t* ctx, vulkan_buffer_t* Q, 
     void* ws = hip_backend_scratch(ctx, need);
     if (!ws) return;
     float scale = 1.0f / sqrtf((float)head_dim);          /* :1168 */
-    HIP_OP(ctx, "batch_attention_backward", seraph_attention_backward_banded(FPTR(Q), FPTR(K), FPTR(V), FPTR(grad_out), NULL, NULL,
+    HIP_OPF(ctx, seraph_attention_backward_banded(FPTR(Q), FPTR(K), FPTR(V), FPTR(grad_out), NULL, NULL,
                                                                      FPTR(grad_Q), FPTR(grad_K), FPTR(grad_V), NULL, 1, seq_len,
-                                                                     num_heads, kv_heads, head_dim, scale, seq_len, ws, need, st->stream));
+                                                                     num_heads, kv_heads, head_dim, scale, seq_len, ws, need, st->stream), "attn_bwd [seq=%d h=%d hd=%d]", seq_len, num_heads, head_dim);
 }
 
 void hip_batch_attention_backward_packed(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulkan_buffer_t* K, vulkan_buffer_t* V,
@@ -144,10 +144,9 @@ void hip_batch_attention_backward_packed(vulkan_context_t* ctx, vulkan_buffer_t*
     void* ws = hip_backend_scratch(ctx, need);
     if (!ws) return;
     float scale = 1.0f / sqrtf((float)head_dim);
-    HIP_OP(ctx, "batch_attention_backward_packed",
-           seraph_attention_backward(FPTR(Q), FPTR(K), FPTR(V), FPTR(grad_out), attn_out ? FPTR(attn_out) : NULL, lse ? FPTR(lse) : NULL,
+    HIP_OPF(ctx, seraph_attention_backward(FPTR(Q), FPTR(K), FPTR(V), FPTR(grad_out), attn_out ? FPTR(attn_out) : NULL, lse ? FPTR(lse) : NULL,
                                      FPTR(grad_Q), FPTR(grad_K), FPTR(grad_V), UPTR(seq_starts), batch_size, total_tokens,
-                                     num_heads, kv_heads, head_dim, scale, ws, st->ws_bytes, st->stream));
+                                     num_heads, kv_heads, head_dim, scale, ws, st->ws_bytes, st->stream), "attn_bwd_packed [tok=%d seqs=%d h=%d hd=%d]", total_tokens, batch_size, num_heads, head_dim);
 }
 
 /* src/vulkan_backend_backward.c:1185-1300 */
@@ -158,7 +157,7 @@ void vulkan_embedding_backward(vulkan_context_t* ctx, vulkan_buffer_t* tokens_u3
     size_t need = seraph_embedding_backward_ws_bytes(seq_len, vocab_size);
     void* ws = hip_backend_scratch(ctx, need);
     if (!ws) return;
-    HIP_OP(ctx, "embedding_backward", seraph_embedding_backward(UPTR(tokens_u32), FPTR(grad_hidden), FPTR(grad_embed), seq_len,
+    HIP_OP(ctx, "embed_bwd", seraph_embedding_backward(UPTR(tokens_u32), FPTR(grad_hidden), FPTR(grad_embed), seq_len,
                                                                 hidden_size, vocab_size, ws, st->ws_bytes, st->stream));
 }
 
@@ -167,7 +166,7 @@ void vulkan_silu_backward(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_
                           vulkan_buffer_t* grad_input, size_t count) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !input || !grad_output || !grad_input) return;
-    HIP_OP(ctx, "silu_backward", seraph_silu_backward(FPTR(input), FPTR(grad_output), FPTR(grad_input), count, st->stream));
+    HIP_OP(ctx, "silu_bwd", seraph_silu_backward(FPTR(input), FPTR(grad_output), FPTR(grad_input), count, st->stream));
 }
 
 /* src/vulkan_backend_backward.c:300-452 */
@@ -175,19 +174,19 @@ void vulkan_elementwise_mul_backward(vulkan_context_t* ctx, vulkan_buffer_t* A, 
                                      vulkan_buffer_t* grad_A, vulkan_buffer_t* grad_B, size_t count) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !A || !B || !grad_C || !grad_A || !grad_B) return;
-    HIP_OP(ctx, "elementwise_mul_backward", seraph_mul_backward(FPTR(A), FPTR(B), FPTR(grad_C), FPTR(grad_A), FPTR(grad_B), count, st->stream));
+    HIP_OP(ctx, "mul_bwd", seraph_mul_backward(FPTR(A), FPTR(B), FPTR(grad_C), FPTR(grad_A), FPTR(grad_B), count, st->stream));
 }
 
 void hip_swiglu_backward(vulkan_context_t* ctx, vulkan_buffer_t* gate, vulkan_buffer_t* up, vulkan_buffer_t* grad_hidden,
                          vulkan_buffer_t* grad_gate, vulkan_buffer_t* grad_up, size_t count) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !gate || !up || !grad_hidden || !grad_gate || !grad_up) return;
-    HIP_OP(ctx, "silu_mul_backward", seraph_swiglu_backward(FPTR(gate), FPTR(up), FPTR(grad_hidden), FPTR(grad_gate), FPTR(grad_up), count, st->stream));
+    HIP_OP(ctx, "silu_mul_bwd", seraph_swiglu_backward(FPTR(gate), FPTR(up), FPTR(grad_hidden), FPTR(grad_gate), FPTR(grad_up), count, st->stream));
 }
 
 void hip_qk_norm_backward(vulkan_context_t* ctx, vulkan_buffer_t* qk_pre, vulkan_buffer_t* grad_out, vulkan_buffer_t* grad_in,
                           int seq_len, int num_heads, int head_dim, float eps) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !qk_pre || !grad_out || !grad_in) return;
-    HIP_OP(ctx, "qk_norm_backward", seraph_qk_norm_backward(FPTR(qk_pre), FPTR(grad_out), FPTR(grad_in), seq_len, num_heads, head_dim, eps, st->stream));
+    HIP_OP(ctx, "qk_norm_bwd", seraph_qk_norm_backward(FPTR(qk_pre), FPTR(grad_out), FPTR(grad_in), seq_len, num_heads, head_dim, eps, st->stream));
 }

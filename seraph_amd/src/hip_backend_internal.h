@@ -10,7 +10,7 @@
 #define HIP_PROF_MAX_OPS 8192
 
 typedef struct {
-    const char* name;
+    char name[128];              /* as the reference names the op (src/vulkan_backend.c:31-43): its report sorts ops by substrings */
     void* ev_start;
     void* ev_stop;
 } hip_prof_op_t;
@@ -42,6 +42,14 @@ void hip_prof_end(vulkan_context_t* ctx);
         int rc_ = (call);                             \
         hip_prof_end((ctx));                          \
         if (rc_ != SERAPH_OK) hip_backend_report((ctx), (name), rc_); \
+    } while (0)
+
+/* The same with a formatted name, e.g. HIP_OPF(ctx, call, "matmul [%dx%d K=%d]", M, N, K). */
+#define HIP_OPF(ctx, call, ...)                       \
+    do {                                              \
+        char pn_[128];                                \
+        snprintf(pn_, sizeof(pn_), __VA_ARGS__);      \
+        HIP_OP((ctx), pn_, (call));                   \
     } while (0)
 
 #define DPTR(buf) ((buf)->buffer)

@@ -284,15 +284,24 @@ def add_tokenizer(mdir, vocab):
         f.write("t 0\n")
 
 
-def run_ref(args, timeout=170):
-    print("seraph-train-cuda-hip", " ".join(map(str, args)), flush=True)
-    p = subprocess.run([REF_BIN] + [str(a) for a in args], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=timeout)
+# The same front end with seraph_amd/seraph_tree/hip_fused_step.c behind its step functions (the reference's
+# src/train_cuda.c still compiled in, unmodified, as the op-by-op fallback).
+FUSED_BIN = os.path.join(ROOT, "oracle", "_ref", "seraph-train-cuda-hip-fused")
+BINARIES = [pytest.param(REF_BIN, id="op-by-op"),
+            pytest.param(FUSED_BIN, id="fused", marks=pytest.mark.skipif(not os.path.exists(FUSED_BIN), reason="fused front end not built"))]
+
+
+def run_ref(args, timeout=170, binary=REF_BIN, env=None):
+    print(os.path.basename(binary), " ".join(map(str, args)), flush=True)
+    p = subprocess.run([binary] + [str(a) for a in args], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=timeout,
+                       env=dict(os.environ, **env) if env else None)
     return p.returncode, p.stdout, p.stderr
 
 
 @needs_ref
+@pytest.mark.parametrize("binary", BINARIES)
 @pytest.mark.parametrize("flash", [False, True])
-def test_reference_batched_trainer_runs_unmodified_and_matches_oracle(tmp_path, orc, flash):
+def test_reference_batched_trainer_runs_unmodified_and_matches_oracle(tmp_path, orc, flash, binary):
     mdir, ckpt = str(tmp_path / "model"), str(tmp_path / "ckpt")
     ocfg, cfg, p0 = make_model_dir(mdir, orc, SHAPE, seed=61)
     add_tokenizer(mdir, SHAPE["vocab"])
@@ -303,8 +312,9 @@ def test_reference_batched_trainer_runs_unmodified_and_matches_oracle(tmp_path, 
     write_ttok(ttok, samples, vocab=SHAPE["vocab"])
     args = [mdir, ttok, "--full-training", "--batch", 3, "--max-seq", 24, "--lr", 2e-3, "--log-every", 1,
             "--save-every", 0, "--checkpoint", ckpt] + (["--flash"] if flash else [])
-    rc, out, err = run_ref(args)
+    rc, out, err = run_ref(args, binary=binary)
     assert rc == 0, (out[-1500:], err[-1500:])
+    assert ("[HIP] fused training step" in err) == (binary == FUSED_BIN)
     tokens = np.concatenate(samples)
     offsets = np.concatenate([[0], np.cumsum([len(s) for s in samples])]).tolist()
     batches = reference_pack(tokens.tolist(), offsets, 3, 24)
@@ -327,7 +337,8 @@ C1_SHAPE = dict(hidden=512, layers=8, heads=8, kv_heads=8, head_dim=64, ffn=1408
 
 
 @needs_ref
-def test_reference_batched_trainer_at_the_33m_shape_8_x_256(tmp_path, orc):
+@pytest.mark.parametrize("binary", BINARIES)
+def test_reference_batched_trainer_at_the_33m_shape_8_x_256(tmp_path, orc, binary):
     """The 33M model exactly, eight packed sequences of 256 tokens per step, three optimizer steps through the
     reference's own cuda_train_step_gpu_full_batch (src/train_cuda.c:1966-2326) over the cuda_train_* symbols:
     the printed losses step by step and the final checkpoint against the oracle's step + AdamW."""
@@ -340,7 +351,7 @@ def test_reference_batched_trainer_at_the_33m_shape_8_x_256(tmp_path, orc):
     write_ttok(ttok, samples, vocab=C1_SHAPE["vocab"])
     args = [mdir, ttok, "--full-training", "--batch", 8, "--max-seq", 256, "--lr", 3.14e-4, "--log-every", 1,
             "--save-every", 0, "--checkpoint", ckpt]
-    rc, out, err = run_ref(args)
+    rc, out, err = run_ref(args, binary=binary)
     assert rc == 0, (out[-1500:], err[-1500:])
     tokens = np.concatenate(samples)
     offsets = np.concatenate([[0], np.cumsum([len(s) for s in samples])]).tolist()
@@ -469,3 +480,37 @@ def test_bench_line_contract():
     assert d["value"] > 0 and abs(d["value"] - d["config"]["tokens_per_step"] / d["ms_per_step"] * 1e3) < 1e-3 * d["value"]
     rf = d["roofline"]
     assert rf["bound"] in ("hbm", "mfma") and abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-3
+
+
+@pytest.mark.skipif(not os.path.exists(FUSED_BIN), reason="fused front end not built")
+def test_fused_front_end_validation_accumulation_and_the_switch_back(tmp_path, orc):
+    """The reference's front end over the fused step: validation losses (cuda_evaluate), gradient accumulation over two
+    micro-steps (the state's counters travel through the fused step), and SERAPH_HIP_FUSED_STEP=0, which makes the same
+    binary run the reference's op-by-op step: all three print the oracle's numbers."""
+    mdir = str(tmp_path / "model")
+    ocfg, cfg, p0 = make_model_dir(mdir, orc, SHAPE, seed=91)
+    add_tokenizer(mdir, SHAPE["vocab"])
+    samples = make_samples(92, 12, SHAPE["vocab"], lo=6, hi=24)
+    val = make_samples(93, 5, SHAPE["vocab"], lo=2, hi=24)
+    ttok, vtok = os.path.join(mdir, "train.ttok"), os.path.join(mdir, "val.ttok")
+    write_ttok(ttok, samples, vocab=SHAPE["vocab"])
+    write_ttok(vtok, val, vocab=SHAPE["vocab"])
+    args = [mdir, ttok, "--full-training", "--batch", 2, "--max-seq", 32, "--lr", 2e-3, "--log-every", 1, "--save-every", 0,
+            "--accum", 2, "--val", vtok, "--eval-every", 2, 0]
+    tokens = np.concatenate(samples)
+    offsets = np.concatenate([[0], np.cumsum([len(s) for s in samples])]).tolist()
+    batches = reference_pack(tokens.tolist(), offsets, 2, 32)
+    ref_losses, rp, _, _ = oracle_run(orc, ocfg, p0.copy(), batches, 2e-3, accum=2)
+    outs = {}
+    for name, env in (("fused", None), ("switched back", {"SERAPH_HIP_FUSED_STEP": "0"})):
+        rc, out, err = run_ref(args + ["--checkpoint", tmp_path / name.replace(" ", "_")], binary=FUSED_BIN, env=env)
+        assert rc == 0, (out[-1500:], err[-1500:])
+        assert ("[HIP] fused training step" in err) == (env is None)
+        got = [l for _, l in step_losses(out)]
+        assert len(got) == len(batches) and np.allclose(got, ref_losses, atol=1.5e-4), (name, got, ref_losses)
+        outs[name] = [float(x) for x in re.findall(r"Val Loss: ([0-9.]+)", out)]
+        assert len(outs[name]) >= 1
+    assert np.allclose(outs["fused"], outs["switched back"], atol=1.5e-4), outs
+    from seraph_amd import io as sio
+    saved = sio.checkpoint_load(str(tmp_path / "fused" / "checkpoint_final.safetensors"), cfg)
+    assert np.all(np.abs(saved - rp) <= 2.0 ** -7 * np.abs(rp) + 1e-6)

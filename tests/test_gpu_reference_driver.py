@@ -28,7 +28,7 @@ CASES = [
 needs_bin = pytest.mark.skipif(not os.path.exists(BIN), reason="oracle/_ref/ref_step_hip not built (needs the Seraph tree)")
 
 
-def run_driver(tmp_path, case, steps, T, lr0, theta, p, tok, rank=0, mask=0, alpha=0.0, lora=None):
+def run_driver(tmp_path, case, steps, T, lr0, theta, p, tok, rank=0, mask=0, alpha=0.0, lora=None, flags=(), stdout=None):
     fin, fout = tmp_path / "in.bin", tmp_path / "out.bin"
     with open(fin, "wb") as f:
         np.array([case["hidden"], case["layers"], case["heads"], case["kv_heads"], case["head_dim"], case["ffn"],
@@ -39,8 +39,10 @@ def run_driver(tmp_path, case, steps, T, lr0, theta, p, tok, rank=0, mask=0, alp
             lora.tofile(f)
         tok.tofile(f)
     print(f"running {BIN} case={case} T={T} steps={steps} rank={rank} mask={mask:#b}", flush=True)
-    r = subprocess.run([BIN, str(fin), str(fout)], capture_output=True, text=True, timeout=170)
+    r = subprocess.run([BIN, *flags, str(fin), str(fout)], capture_output=True, text=True, timeout=170)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    if stdout is not None:
+        stdout.append(r.stdout)
     return np.fromfile(fout, np.float32)
 
 
@@ -137,3 +139,41 @@ def test_reference_lora_driver_matches_oracle(orc, mask, tmp_path):
         bad = np.abs(got.astype(np.float64) - ref) > 1e-5 + 1e-4 * np.abs(ref)
         assert not bad.any(), f"{name}: {bad.sum()}/{bad.size} outside tolerance, max {np.abs(got - ref).max():.3e}"
     assert np.abs(w - lo).max() > 1e-5            # the adapters did move
+
+
+@needs_bin
+def test_profiler_report_has_the_reference_layout(orc, tmp_path):
+    """vulkan_profiler_end_step prints what src/vulkan_backend.c:152-207 prints: the header, the nine categories in
+    order, the per-operation table, with the ops under the reference's names (src/vulkan_backend.c:1674-3482,
+    src/vulkan_backend_backward.c:164-1191), so that the substring roll-up fills the same rows: attention backward
+    apart from forward, RMSNorm backward apart from forward, cross entropy, AdamW."""
+    import re
+    case = dict(CASES[0])
+    T, steps = case.pop("T"), case.pop("steps")
+    ocfg = orc.make_config(**case, rms_eps=1e-5, rope_theta=10000.0)
+    p = init_params(orc, ocfg, 41)
+    tok = np.random.default_rng(42).integers(0, case["vocab"], steps * T).astype(np.int32)
+    text = []
+    out = run_driver(tmp_path, case, steps, T, 1e-3, 10000.0, p, tok, flags=("--profile",), stdout=text)
+    text = text[0]
+    assert text.count("SERAPH VULKAN STEP PROFILER (step ") == steps
+    m = re.search(r"SERAPH VULKAN STEP PROFILER \(step 2, seq=%d, loss=([0-9.]+)\)\n  (\d+) operations, ([0-9.]+) ms total" % T, text)
+    assert m and abs(float(m.group(1)) - out[1]) < 1e-3 and int(m.group(2)) > 50
+    report = text[text.rindex("SERAPH VULKAN STEP PROFILER"):]
+    cats = re.findall(r"^  (matmul \(all\)|attention fwd|attention bwd|rmsnorm fwd|rmsnorm bwd|cross_entropy|adamw|copy/fill|other) +([0-9.]+) +([0-9.]+)%", report, re.M)
+    assert [c[0] for c in cats] == ["matmul (all)", "attention fwd", "attention bwd", "rmsnorm fwd", "rmsnorm bwd", "cross_entropy",
+                                    "adamw", "copy/fill", "other"]
+    ms = {c[0]: float(c[1]) for c in cats}
+    assert all(ms[k] > 0 for k in ("matmul (all)", "attention fwd", "attention bwd", "rmsnorm fwd", "rmsnorm bwd", "cross_entropy", "adamw", "copy/fill", "other"))
+    assert abs(sum(ms.values()) - float(m.group(3))) < 0.05 * float(m.group(3)) + 0.01
+    assert "── CATEGORY BREAKDOWN ──" in report and "── PER-OPERATION DETAIL ──" in report
+    assert re.search(r"^     #  Operation +Time \(ms\) +%  Grid / Block", report, re.M)
+    L, h, qd, kv, f, V = case["layers"], case["hidden"], case["heads"] * case["head_dim"], case["kv_heads"] * case["head_dim"], case["ffn"], case["vocab"]
+    for needle in (f"matmul_t [{T}x{qd} K={h}]", f"matmul [{T}x{h} K={f}]", f"attn_fwd [seq={T} h={case['heads']} hd={case['head_dim']}]",
+                   f"attn_bwd [seq={T} h={case['heads']} hd={case['head_dim']}]", f"rmsnorm [{T}x{h}] 256-thr", f"rmsnorm_bwd [{T}x{h}] 256-thr",
+                   f"cross_entropy_grad [{T - 1}x{V}] 256-thr", f"adamw [{V * h}] 256-thr", "rope_fwd", "rope_bwd", "silu_bwd", "mul_bwd",
+                   "embed_lookup", "embed_bwd", "reduce_sum"):
+        assert needle in report, needle
+    ops = re.findall(r"^ +(\d+)  (\S.*?) +([0-9.]+) +([0-9.]+)%", report[report.index("PER-OPERATION DETAIL"):], re.M)
+    assert len(ops) == int(m.group(2)) and [int(o[0]) for o in ops] == list(range(len(ops)))
+    assert sum(1 for o in ops if o[1].startswith("attn_bwd")) == L and sum(1 for o in ops if o[1].startswith("rmsnorm_bwd")) == 2 * L + 1
