@@ -154,6 +154,17 @@ int seraph_gemm_scaled(const float* A, const float* B, float* C, int64_t M, int6
                        int transpose_A, int transpose_B, int accumulate, float alpha,
                        void* ws, size_t ws_bytes, seraph_stream_t s);
 
+/* Several such products in one launch each: the rank-sized products of the LoRA adapters of a layer (four adapters
+ * times x A^T, then B^T onto the output, and three gradient products each: src/train.c:5778-5845 runs them one by one).
+ * The products share the orientations, alpha and the accumulate flag, not their shapes.  Every product is computed
+ * exactly as seraph_gemm_scaled computes it alone (same runs of K, same order of additions); a list that cannot share
+ * launches is run as single calls.  `problems` is a HOST array of at most 4; the outputs must not overlap; the scratch
+ * holds the runs of all products at once. */
+typedef struct { const float* A; const float* B; float* C; int64_t M, N, K; } seraph_gemm_scaled_problem_t;
+size_t seraph_gemm_scaled_grouped_ws_bytes(const seraph_gemm_scaled_problem_t* problems, int count, int transpose_A, int transpose_B);
+int seraph_gemm_scaled_grouped(const seraph_gemm_scaled_problem_t* problems, int count, int transpose_A, int transpose_B,
+                               int accumulate, float alpha, void* ws, size_t ws_bytes, seraph_stream_t s);
+
 /* ---------------------------------------------------------------- attention */
 /* vulkan_batch_attention (include/vulkan_backend.h:485-488, shaders/batch_attention_stream.comp)
  * and cuda_train_batch_attention_packed (include/cuda_train_context.h:273): causal, GQA,

@@ -520,7 +520,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_group
 template <bool A_KC, bool B_KC>
 __device__ __forceinline__ void splitk_body(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
                                             int64_t M, int64_t N, int64_t K, int accumulate, int nbn, int tile,
-                                            int slices, float* __restrict__ part) {
+                                            int slices, int slice, float* __restrict__ part) {
     constexpr int BT = 32;
     constexpr int A_FLOATS = lds_floats<BT, A_KC>(), B_FLOATS = lds_floats<BT, B_KC>();
     __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
@@ -543,7 +543,7 @@ __device__ __forceinline__ void splitk_body(const float* __restrict__ A, const f
     FastLoader<BT, B_KC, R> lb;
     la.init(lda, m0, M);
     lb.init(ldb, n0, N);
-    const int64_t k_run = K / slices, k0 = (int64_t)blockIdx.y * k_run;          // whole stages: the launcher sees to it
+    const int64_t k_run = K / slices, k0 = (int64_t)slice * k_run;               // whole stages: the launcher sees to it
     const float* ta = A_KC ? A + m0 * lda + k0 : A + m0 + k0 * lda;
     const float* tb = B_KC ? B + n0 * ldb + k0 : B + n0 + k0 * ldb;
     const int64_t step_a = A_KC ? kBK : kBK * lda, step_b = B_KC ? kBK : kBK * ldb;
@@ -615,7 +615,7 @@ __device__ __forceinline__ void splitk_body(const float* __restrict__ A, const f
         if (row < M && col < N) {
             const float v = ((red[0][e] + red[1][e]) + red[2][e]) + red[3][e];
             if (slices > 1) {
-                part[(int64_t)blockIdx.y * M * N + row * N + col] = v;
+                part[(int64_t)slice * M * N + row * N + col] = v;
             } else {
                 float* dst = C + row * N + col;
                 *dst = accumulate ? *dst + v : v;
@@ -632,7 +632,7 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_kernel(c
                                                                                int accumulate, int nbm, int nbn,
                                                                                int slices, float* __restrict__ part) {
     (void)nbm;
-    splitk_body<A_KC, B_KC>(A, B, C, M, N, K, accumulate, nbn, (int)blockIdx.x, slices, part);
+    splitk_body<A_KC, B_KC>(A, B, C, M, N, K, accumulate, nbn, (int)blockIdx.x, slices, (int)blockIdx.y, part);
 }
 
 // the grouped form of the above (one run of K, no slices); nbm / nbn / first count 32 x 32 tiles here
@@ -641,7 +641,7 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_grouped_
     const int tile = (int)blockIdx.x;
     int i = 0;
     while (i + 1 < g.count && tile >= g.first[i + 1]) i++;
-    splitk_body<A_KC, B_KC>(g.A[i], g.B[i], g.C[i], g.M[i], g.N[i], K, accumulate, g.nbn[i], tile - g.first[i], 1, nullptr);
+    splitk_body<A_KC, B_KC>(g.A[i], g.B[i], g.C[i], g.M[i], g.N[i], K, accumulate, g.nbn[i], tile - g.first[i], 1, 0, nullptr);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -649,11 +649,69 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_grouped_
 // matrix instructions.  A lane keeps its four columns' rows of B in registers, a wave walks down rows of A,
 // whose K values are the same for all lanes (scalar loads), and adds in ascending k.
 template <int K4>
+__device__ __forceinline__ void smallk_body(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
+                                            int64_t M, int64_t N, int accumulate, int rows_per_wave, int block_x, int block_y);
+
+template <int K4>
 __global__ __launch_bounds__(256) void gemm_smallk_kernel(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
                                                           int64_t M, int64_t N, int accumulate, int rows_per_wave) {
+    smallk_body<K4>(A, B, C, M, N, accumulate, rows_per_wave, (int)blockIdx.x, (int)blockIdx.y);
+}
+
+// C (+)= alpha * (part[0] + part[1] + ... ), the runs added in index order
+__global__ __launch_bounds__(256) void gemm_slices_sum_kernel(const float* __restrict__ part, float* __restrict__ C, int64_t n,
+                                                              int slices, float alpha, int accumulate) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float v = part[i];
+    for (int p = 1; p < slices; p++) v += part[(int64_t)p * n + i];
+    v *= alpha;
+    C[i] = accumulate ? C[i] + v : v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The rank-sized products of several LoRA adapters of one layer in one launch each.  Every product keeps its own K and
+// its own number of runs, a workgroup is one (product, run, tile) and does what the single-product kernels above do
+// for it: the results are the single calls' bits.
+struct GemmRuns {
+    const float* A[kMaxGroup]; const float* B[kMaxGroup]; float* C[kMaxGroup]; float* part[kMaxGroup];
+    int64_t M[kMaxGroup], N[kMaxGroup], K[kMaxGroup];
+    int nbn[kMaxGroup], tiles[kMaxGroup], slices[kMaxGroup];
+    int first[kMaxGroup + 1];                                      // first workgroup of product i (runs kernel) / first block (sum kernel)
+    int count;
+};
+
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_runs_grouped_kernel(const GemmRuns g) {
+    const int wg = (int)blockIdx.x;
+    int i = 0;
+    while (i + 1 < g.count && wg >= g.first[i + 1]) i++;           // uniform
+    const int local = wg - g.first[i];
+    splitk_body<A_KC, B_KC>(g.A[i], g.B[i], g.C[i], g.M[i], g.N[i], g.K[i], 0, g.nbn[i], local % g.tiles[i], g.slices[i],
+                            local / g.tiles[i], g.part[i]);
+}
+
+__global__ __launch_bounds__(256) void gemm_slices_sum_grouped_kernel(const GemmRuns g, float alpha, int accumulate) {
+    const int b = (int)blockIdx.x;
+    int i = 0;
+    while (i + 1 < g.count && b >= g.first[i + 1]) i++;
+    const int64_t n = g.M[i] * g.N[i];
+    const int64_t e = (int64_t)(b - g.first[i]) * 256 + threadIdx.x;
+    if (e >= n) return;
+    const float* part = g.part[i];
+    float v = part[e];
+    for (int p = 1; p < g.slices[i]; p++) v += part[(int64_t)p * n + e];
+    v *= alpha;
+    float* C = g.C[i];
+    C[e] = accumulate ? C[e] + v : v;
+}
+
+template <int K4>
+__device__ __forceinline__ void smallk_body(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
+                                            int64_t M, int64_t N, int accumulate, int rows_per_wave, int block_x, int block_y) {
     constexpr int K = 4 * K4;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int64_t n = ((int64_t)blockIdx.x * 64 + lane) * 4;
+    const int64_t n = ((int64_t)block_x * 64 + lane) * 4;
     const bool col_ok = n < N;                                  // N is a multiple of 4
     float4 b[4][K4];
 #pragma unroll
@@ -661,7 +719,7 @@ __global__ __launch_bounds__(256) void gemm_smallk_kernel(const float* __restric
 #pragma unroll
         for (int q = 0; q < K4; q++)
             b[j][q] = col_ok ? *reinterpret_cast<const float4*>(B + (n + j) * K + 4 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
-    const int64_t m0 = ((int64_t)blockIdx.y * 4 + wave) * rows_per_wave;
+    const int64_t m0 = ((int64_t)block_y * 4 + wave) * rows_per_wave;
     for (int r = 0; r < rows_per_wave && m0 + r < M; r++) {
         const float* a = A + (m0 + r) * K;
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -686,15 +744,13 @@ __global__ __launch_bounds__(256) void gemm_smallk_kernel(const float* __restric
     }
 }
 
-// C (+)= alpha * (part[0] + part[1] + ... ), the runs added in index order
-__global__ __launch_bounds__(256) void gemm_slices_sum_kernel(const float* __restrict__ part, float* __restrict__ C, int64_t n,
-                                                              int slices, float alpha, int accumulate) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    float v = part[i];
-    for (int p = 1; p < slices; p++) v += part[(int64_t)p * n + i];
-    v *= alpha;
-    C[i] = accumulate ? C[i] + v : v;
+// grid x: the column blocks of all products one after the other; grid y: row blocks (of the tallest product)
+template <int K4>
+__global__ __launch_bounds__(256) void gemm_smallk_grouped_kernel(const GemmRuns g, int accumulate, int rows_per_wave) {
+    const int b = (int)blockIdx.x;
+    int i = 0;
+    while (i + 1 < g.count && b >= g.first[i + 1]) i++;
+    smallk_body<K4>(g.A[i], g.B[i], g.C[i], g.M[i], g.N[i], accumulate, rows_per_wave, b - g.first[i], (int)blockIdx.y);
 }
 
 // The pipelined kernel needs whole K stages, and every per-lane offset inside a tile panel
@@ -1034,4 +1090,115 @@ extern "C" int seraph_gemm_scaled(const float* A, const float* B, float* C, int6
     int rc = seraph_gemm(A, B, C, M, N, K, transpose_A, transpose_B, accumulate, s);
     if (rc != SERAPH_OK || alpha == 1.0f) return rc;
     return seraph_scale(C, (size_t)(M * N), alpha, s);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Several seraph_gemm_scaled products that share the orientations, alpha and the accumulate flag: one pair of launches
+// when every product is cut into runs of K, one launch when every product has the same rank-sized K, else one call each.
+static int scaled_group_kind(const seraph_gemm_scaled_problem_t* p, int count, int tA, int tB, float alpha, int* slices, size_t* need) {
+    if (count < 2 || count > kMaxGroup) return 0;
+    bool runs = true, small = alpha == 1.0f;
+    size_t bytes = 0;
+    for (int i = 0; i < count; i++) {
+        const int64_t M = p[i].M, N = p[i].N, K = p[i].K, lda = tA ? M : K, ldb = tB ? K : N;
+        if (M <= 0 || N <= 0 || K <= 0 || !p[i].A || !p[i].B || !p[i].C) return 0;
+        const bool vec = lda % 4 == 0 && ldb % 4 == 0 && aligned16(p[i].A) && aligned16(p[i].B);
+        slices[i] = vec ? slice_count(M, N, K, tA, tB) : 1;
+        runs = runs && slices[i] > 1 && ceil_div(M, 32) * ceil_div(N, 32) * slices[i] < (1 << 24);
+        small = small && use_smallk(p[i].A, p[i].B, p[i].C, M, N, K, tA, tB) && K == p[0].K && ceil_div(N, 256) < (1 << 24);
+        bytes += (((size_t)slices[i] * (size_t)M * (size_t)N + 3) & ~(size_t)3) * 4;     // every product's runs start on a 16-byte boundary
+    }
+    *need = runs ? bytes : 0;
+    return runs ? 1 : small ? 2 : 0;
+}
+
+extern "C" size_t seraph_gemm_scaled_grouped_ws_bytes(const seraph_gemm_scaled_problem_t* problems, int count,
+                                                      int transpose_A, int transpose_B) {
+    if (!problems || count <= 0) return 0;
+    int slices[kMaxGroup];
+    size_t need = 0;
+    if (scaled_group_kind(problems, count, transpose_A, transpose_B, 0.5f, slices, &need) == 1) return need;
+    for (int i = 0; i < count; i++) {                      // run one by one: the largest single requirement
+        const size_t one = seraph_gemm_scaled_ws_bytes(problems[i].M, problems[i].N, problems[i].K, transpose_A, transpose_B);
+        if (one > need) need = one;
+    }
+    return need;
+}
+
+extern "C" int seraph_gemm_scaled_grouped(const seraph_gemm_scaled_problem_t* problems, int count, int transpose_A, int transpose_B,
+                                          int accumulate, float alpha, void* ws, size_t ws_bytes, seraph_stream_t s) {
+    if (count <= 0) return SERAPH_OK;
+    SERAPH_REQUIRE(problems, "gemm_scaled_grouped: NULL problem list");
+    int slices[kMaxGroup];
+    size_t need = 0;
+    int kind = scaled_group_kind(problems, count, transpose_A, transpose_B, alpha, slices, &need);
+    if (kind == 1 && (!ws || !aligned16(ws) || ws_bytes < need)) kind = 0;
+    hipStream_t st = as_stream(s);
+    if (kind == 0) {                                       // exactly as the single calls
+        for (int i = 0; i < count; i++) {
+            int rc = seraph_gemm_scaled(problems[i].A, problems[i].B, problems[i].C, problems[i].M, problems[i].N, problems[i].K,
+                                        transpose_A, transpose_B, accumulate, alpha, ws, ws_bytes, s);
+            if (rc != SERAPH_OK) return rc;
+        }
+        return SERAPH_OK;
+    }
+    GemmRuns g;
+    g.count = count;
+    if (kind == 1) {
+        float* part = (float*)ws;
+        int total = 0;
+        for (int i = 0; i < kMaxGroup; i++) {
+            const int j = i < count ? i : count - 1;
+            g.A[i] = problems[j].A; g.B[i] = problems[j].B; g.C[i] = problems[j].C;
+            g.M[i] = problems[j].M; g.N[i] = problems[j].N; g.K[i] = problems[j].K;
+            g.nbn[i] = (int)ceil_div(g.N[i], 32); g.tiles[i] = (int)(ceil_div(g.M[i], 32) * ceil_div(g.N[i], 32)); g.slices[i] = slices[j];
+            g.first[i] = total;
+            if (i < count) {
+                g.part[i] = part;
+                part += ((size_t)slices[i] * (size_t)g.M[i] * (size_t)g.N[i] + 3) & ~(size_t)3;
+                total += g.tiles[i] * g.slices[i];
+            } else {
+                g.part[i] = g.part[count - 1];
+            }
+        }
+        g.first[kMaxGroup] = total;
+        for (int i = count; i <= kMaxGroup; i++) g.first[i] = total;
+        const dim3 grid((unsigned)total), block(kGemmThreads);
+        const int form = (transpose_A ? 2 : 0) + (transpose_B ? 1 : 0);
+        switch (form) {
+            case 0: hipLaunchKernelGGL((gemm_f32_mfma_splitk_runs_grouped_kernel<true, false>), grid, block, 0, st, g); break;
+            case 1: hipLaunchKernelGGL((gemm_f32_mfma_splitk_runs_grouped_kernel<true, true>), grid, block, 0, st, g); break;
+            case 2: hipLaunchKernelGGL((gemm_f32_mfma_splitk_runs_grouped_kernel<false, false>), grid, block, 0, st, g); break;
+            default: hipLaunchKernelGGL((gemm_f32_mfma_splitk_runs_grouped_kernel<false, true>), grid, block, 0, st, g); break;
+        }
+        SERAPH_LAUNCH_CHECK();
+        int blocks = 0;
+        for (int i = 0; i < count; i++) { g.first[i] = blocks; blocks += (int)ceil_div(g.M[i] * g.N[i], 256); }
+        for (int i = count; i <= kMaxGroup; i++) g.first[i] = blocks;
+        hipLaunchKernelGGL(gemm_slices_sum_grouped_kernel, dim3((unsigned)blocks), dim3(256), 0, st, g, alpha, accumulate);
+        SERAPH_LAUNCH_CHECK();
+        return SERAPH_OK;
+    }
+    // rank-sized K: the column blocks of all products side by side
+    const int rows_per_wave = 8;
+    int blocks = 0;
+    int64_t max_m = 0;
+    for (int i = 0; i < kMaxGroup; i++) {
+        const int j = i < count ? i : count - 1;
+        g.A[i] = problems[j].A; g.B[i] = problems[j].B; g.C[i] = problems[j].C; g.part[i] = nullptr;
+        g.M[i] = problems[j].M; g.N[i] = problems[j].N; g.K[i] = problems[j].K;
+        g.nbn[i] = 0; g.tiles[i] = 0; g.slices[i] = 1;
+        g.first[i] = blocks;
+        if (i < count) { blocks += (int)ceil_div(g.N[i], 256); if (g.M[i] > max_m) max_m = g.M[i]; }
+    }
+    for (int i = count; i <= kMaxGroup; i++) g.first[i] = blocks;
+    const dim3 grid((unsigned)blocks, (unsigned)ceil_div(max_m, 4 * rows_per_wave));
+    SERAPH_REQUIRE(grid.y <= 65535u * 1024u, "gemm_scaled_grouped: too many rows");
+    switch (problems[0].K / 4) {
+#define GOK(K4) case K4: hipLaunchKernelGGL(gemm_smallk_grouped_kernel<K4>, grid, dim3(256), 0, st, g, accumulate, rows_per_wave); break;
+        GOK(1) GOK(2) GOK(3) GOK(4) GOK(5) GOK(6) GOK(7) GOK(8)
+#undef GOK
+    }
+    SERAPH_LAUNCH_CHECK();
+    return SERAPH_OK;
 }

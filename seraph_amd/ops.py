@@ -136,6 +136,23 @@ def gemm_scaled(A, B, M, N, K, tA=0, tB=0, out=None, accumulate=False, alpha=1.0
     return out
 
 
+class GemmScaledProblem(C.Structure):
+    _fields_ = [("A", C.c_void_p), ("B", C.c_void_p), ("C", C.c_void_p), ("M", C.c_int64), ("N", C.c_int64), ("K", C.c_int64)]
+
+
+def gemm_scaled_grouped(problems, tA=0, tB=0, accumulate=False, alpha=1.0):
+    """problems: list of (A, B, out, M, N, K) sharing the orientations, alpha and the accumulate flag; one launch each."""
+    k = kernels()
+    arr = (GemmScaledProblem * len(problems))(*[GemmScaledProblem(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, n, kk)
+                                                 for a, b, c, m, n, kk in problems])
+    k.seraph_gemm_scaled_grouped_ws_bytes.restype = C.c_size_t
+    nbytes = k.seraph_gemm_scaled_grouped_ws_bytes(arr, C.c_int(len(problems)), C.c_int(tA), C.c_int(tB))
+    ws = torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=problems[0][0].device)
+    check(k.seraph_gemm_scaled_grouped(arr, C.c_int(len(problems)), C.c_int(tA), C.c_int(tB), C.c_int(1 if accumulate else 0),
+                                       f32(alpha), _p(ws), C.c_size_t(int(nbytes)), _stream()), "gemm_scaled_grouped")
+    return [p[2] for p in problems]
+
+
 def attention_forward(Q, K, V, heads, kv_heads, head_dim, seq_starts=None, scale=None, want_lse=True):
     T = Q.shape[0]
     out = torch.empty_like(Q)

@@ -374,7 +374,7 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
         const size_t per_layer = 4 * up256(T * h * 4) + 2 * up256(T * qd * 4) + 2 * up256(T * kv * 4) +
                                  up256(T * cfg->heads * 4) + 3 * up256(T * f * 4) + (cfg->use_qk_norm ? 2 * up256(T * 4) : 0) +
                                  adapters * up256(T * r * 4);
-        const size_t rest = 2 * up256(T * h * 4) + up256(T * Vv * 4) + 3 * up256(T * 4) + up256(T * h * 4) + 2 * up256(T * r * 4) +
+        const size_t rest = 2 * up256(T * h * 4) + up256(T * Vv * 4) + 3 * up256(T * 4) + up256(T * h * 4) + up256(4 * T * r * 4) + up256(T * r * 4) +
                             3 * up256(T * h * 4) + 3 * up256(T * f * 4) + 2 * up256(T * qd * 4) + 2 * up256(T * kv * 4) +
                             2 * up256(T * 4) + up256(((size_t)max_batch + 1) * 4);
         t->act_bytes = per_layer * (size_t)cfg->layers + rest;
@@ -394,7 +394,7 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
         }
         TAKE(t->final_in, T * h * 4); TAKE(t->xn_final, T * h * 4); TAKE(t->logits, T * Vv * 4);
         TAKE(t->loss_rows, T * 4); TAKE(t->red_a, T * 4); TAKE(t->red_b, T * 4);
-        TAKE(t->tmp_h, T * h * 4); TAKE(t->lora_tmp, T * r * 4); TAKE(t->lora_tmp2, T * r * 4);
+        TAKE(t->tmp_h, T * h * 4); TAKE(t->lora_tmp, 4 * T * r * 4); TAKE(t->lora_tmp2, T * r * 4);
         TAKE(t->g_hidden, T * h * 4); TAKE(t->g_tmp, T * h * 4); TAKE(t->g_xn, T * h * 4);
         TAKE(t->g_ffn, T * f * 4); TAKE(t->g_gate, T * f * 4); TAKE(t->g_up, T * f * 4);
         TAKE(t->g_attn, T * qd * 4); TAKE(t->g_q, T * qd * 4); TAKE(t->g_k, T * kv * 4); TAKE(t->g_v, T * kv * 4);
@@ -417,6 +417,7 @@ hip_trainer_t* hip_trainer_create(const hip_model_config_t* cfg, const hip_optim
                 t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(dims[i], r, Tm, 1, 0));
                 t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(r, dims[i], Tm, 1, 0));
                 t->ws2_bytes = t->ws_bytes;
+                if (i == 3) t->ws_bytes = 4 * t->ws_bytes + 64;    /* the adapters of a layer share launches: all their runs at once */
             } else {
                 for (int j = 0; j < 4; j++) {
                     t->ws_bytes = max_sz(t->ws_bytes, seraph_gemm_scaled_ws_bytes(dims[i], dims[j], Tm, 1, 0));
@@ -582,6 +583,50 @@ static int lora_backward(hip_trainer_t* t, const float* dY, const float* x, cons
     LGEMM(dY, B, tmp, T, r, outd, 0, 0, 0, s);
     LGEMM(tmp, x, gA, r, in, T, 1, 0, 1, 1.0f);
 #undef LGEMM
+    return 0;
+}
+
+/* The same for the adapters of one layer that are due at the same point of the step (q, k, v; gate, up; in the backward
+ * also o with q, k, v and down with gate, up, whose operands are still in place then): each kind of product is one
+ * launch for all of them (seraph_gemm_scaled_grouped), every product computed exactly as the single call computes it. */
+typedef struct { const float* x; float* out; const float* A; const float* B; int64_t in, outd; float* xa; } lora_fwd_item_t;
+typedef struct { const float* dY; const float* x; const float* xa; const float* B; float* gA; float* gB; int64_t in, outd; } lora_bwd_item_t;
+
+static int lora_forward_group(hip_trainer_t* t, const lora_fwd_item_t* it, int n, int64_t T) {
+    if (n <= 0) return 0;
+    const int r = t->cfg.lora_rank;
+    const float s = t->cfg.lora_alpha / (float)r;
+    seraph_gemm_scaled_problem_t p1[4], p2[4];
+    double fl = 0.0;
+    for (int i = 0; i < n; i++) {
+        p1[i] = (seraph_gemm_scaled_problem_t){it[i].x, it[i].A, it[i].xa, T, r, it[i].in};
+        p2[i] = (seraph_gemm_scaled_problem_t){it[i].xa, it[i].B, it[i].out, T, it[i].outd, r};
+        fl += 2.0 * (double)T * r * (double)it[i].in;
+    }
+    OP("gemm_scaled", fl, 0.0, seraph_gemm_scaled_grouped(p1, n, 0, 1, 0, s, t->ws, t->ws_bytes, t->stream));
+    fl = 0.0;
+    for (int i = 0; i < n; i++) fl += 2.0 * (double)T * r * (double)it[i].outd;
+    OP("gemm_scaled", fl, 0.0, seraph_gemm_scaled_grouped(p2, n, 0, 1, 1, 1.0f, t->ws, t->ws_bytes, t->stream));
+    return 0;
+}
+
+static int lora_backward_group(hip_trainer_t* t, const lora_bwd_item_t* it, int n, int64_t T) {
+    if (n <= 0) return 0;
+    const int r = t->cfg.lora_rank;
+    const float s = t->cfg.lora_alpha / (float)r;
+    seraph_gemm_scaled_problem_t pb[4], pt[4], pa[4];
+    double fb = 0.0, fa = 0.0;
+    for (int i = 0; i < n; i++) {
+        float* tmp = t->lora_tmp + (size_t)i * (size_t)T * (size_t)r;
+        pb[i] = (seraph_gemm_scaled_problem_t){it[i].dY, it[i].xa, it[i].gB, it[i].outd, r, T};     /* src/train.c:5823-5829 */
+        pt[i] = (seraph_gemm_scaled_problem_t){it[i].dY, it[i].B, tmp, T, r, it[i].outd};           /* :5831-5836 */
+        pa[i] = (seraph_gemm_scaled_problem_t){tmp, it[i].x, it[i].gA, r, it[i].in, T};             /* :5837-5841 */
+        fb += 2.0 * (double)T * r * (double)it[i].outd;
+        fa += 2.0 * (double)T * r * (double)it[i].in;
+    }
+    OP("gemm_scaled", fb, 0.0, seraph_gemm_scaled_grouped(pb, n, 1, 0, 1, 1.0f, t->ws, t->ws_bytes, t->stream));
+    OP("gemm_scaled", fb, 0.0, seraph_gemm_scaled_grouped(pt, n, 0, 0, 0, s, t->ws, t->ws_bytes, t->stream));
+    OP("gemm_scaled", fa, 0.0, seraph_gemm_scaled_grouped(pa, n, 1, 0, 1, 1.0f, t->ws, t->ws_bytes, t->stream));
     return 0;
 }
 
@@ -766,9 +811,15 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
                                                   {a->xn_attn, W + t->L.v, a->v, T, kv}};
             GEMM_GROUP(qkv, 3, h, 0, 1, 0);
         }
-        if (lora && t->LL.A[0] >= 0 && lora_forward_add(t, a->xn_attn, a->q, LW + t->LL.A[0], LW + t->LL.B[0], T, h, qd, a->xa[0])) return -1.0f;
-        if (lora && t->LL.A[1] >= 0 && lora_forward_add(t, a->xn_attn, a->k, LW + t->LL.A[1], LW + t->LL.B[1], T, h, kv, a->xa[1])) return -1.0f;
-        if (lora && t->LL.A[2] >= 0 && lora_forward_add(t, a->xn_attn, a->v, LW + t->LL.A[2], LW + t->LL.B[2], T, h, kv, a->xa[2])) return -1.0f;
+        if (lora) {                                                        /* the q, k and v adapters in one launch per product */
+            float* outs[3] = {a->q, a->k, a->v};
+            const int64_t od[3] = {qd, kv, kv};
+            lora_fwd_item_t it[3];
+            int n = 0;
+            for (int p = 0; p < 3; p++)
+                if (t->LL.A[p] >= 0) it[n++] = (lora_fwd_item_t){a->xn_attn, outs[p], LW + t->LL.A[p], LW + t->LL.B[p], h, od[p], a->xa[p]};
+            if (lora_forward_group(t, it, n, T)) return -1.0f;
+        }
         OP("rope", 0.0, 8.0 * (double)(T * (qd + kv)), seraph_rope_qk(a->q, a->q, H, a->k, a->k, KVH, starts, batch, T, D, theta, 0, s));
         if (c->use_qk_norm) {                                              /* after RoPE, before the attention: src/train.c:4687-4689 */
             OP("qk_norm", 0.0, 8.0 * (double)(T * qd), seraph_qk_norm_saved(a->q, a->rms_q, T, H, D, eps, s));
@@ -782,8 +833,14 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
             const seraph_gemm_problem_t gu[2] = {{a->xn_ffn, W + t->L.gate, a->gate, T, f}, {a->xn_ffn, W + t->L.up, a->up, T, f}};
             GEMM_GROUP(gu, 2, h, 0, 1, 0);
         }
-        if (lora && t->LL.A[4] >= 0 && lora_forward_add(t, a->xn_ffn, a->gate, LW + t->LL.A[4], LW + t->LL.B[4], T, h, f, a->xa[4])) return -1.0f;
-        if (lora && t->LL.A[5] >= 0 && lora_forward_add(t, a->xn_ffn, a->up, LW + t->LL.A[5], LW + t->LL.B[5], T, h, f, a->xa[5])) return -1.0f;
+        if (lora) {
+            float* outs[2] = {a->gate, a->up};
+            lora_fwd_item_t it[2];
+            int n = 0;
+            for (int p = 4; p < 6; p++)
+                if (t->LL.A[p] >= 0) it[n++] = (lora_fwd_item_t){a->xn_ffn, outs[p - 4], LW + t->LL.A[p], LW + t->LL.B[p], h, f, a->xa[p]};
+            if (lora_forward_group(t, it, n, T)) return -1.0f;
+        }
         OP("swiglu", 0.0, 12.0 * (double)(T * f), seraph_swiglu(a->gate, a->up, a->ffn_h, (size_t)(T * f), s));
         GEMM(a->ffn_h, W + t->L.down, t->tmp_h, T, h, f, 0, 1, 0);
         if (lora && t->LL.A[6] >= 0 && lora_forward_add(t, a->ffn_h, t->tmp_h, LW + t->LL.A[6], LW + t->LL.B[6], T, f, h, a->xa[6])) return -1.0f;
@@ -851,7 +908,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         /* what leaves the chain at each fork: the weight gradient of the projection, or (LoRA) its adapter's gradients */
         SIDE_FORK();
         if (!lora) WGEMM(t->g_hidden, a->ffn_h, GW + t->L.down, h, f, T);
-        else if (t->LL.A[6] >= 0 &&                                          /* src/train.c:6422-6429 */
+        else if (ov && t->LL.A[6] >= 0 &&                                    /* src/train.c:6422-6429 */
                  lora_backward(t, t->g_hidden, a->ffn_h, a->xa[6], LW + t->LL.B[6], LGW + t->LL.A[6], LGW + t->LL.B[6], T, f, h, ov)) return -1.0f;
         SIDE_MARK(MK_DOWN);
         GEMM(t->g_hidden, W + t->L.down, t->g_ffn, T, f, h, 0, 0, 0);
@@ -862,11 +919,23 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         if (!lora) {
             const seraph_gemm_problem_t gu[2] = {{t->g_gate, a->xn_ffn, GW + t->L.gate, f, h}, {t->g_up, a->xn_ffn, GW + t->L.up, f, h}};
             WGEMM_GROUP(gu, 2, T);
-        } else {                                                             /* src/train.c:6446-6461 */
+        } else if (ov) {                                                     /* src/train.c:6446-6461 */
             if (t->LL.A[4] >= 0 &&
                 lora_backward(t, t->g_gate, a->xn_ffn, a->xa[4], LW + t->LL.B[4], LGW + t->LL.A[4], LGW + t->LL.B[4], T, h, f, ov)) return -1.0f;
             if (t->LL.A[5] >= 0 &&
                 lora_backward(t, t->g_up, a->xn_ffn, a->xa[5], LW + t->LL.B[5], LGW + t->LL.A[5], LGW + t->LL.B[5], T, h, f, ov)) return -1.0f;
+        } else {
+            /* gate, up and the down adapter left over from above (g_hidden is not rewritten before the norm backward
+             * below, ffn_h stays): one launch per kind of product */
+            const float* dYs[3] = {t->g_gate, t->g_up, t->g_hidden};
+            const float* xs[3] = {a->xn_ffn, a->xn_ffn, a->ffn_h};
+            const int64_t ind[3] = {h, h, f}, od[3] = {f, f, h};
+            lora_bwd_item_t it[3];
+            int n = 0;
+            for (int p = 4; p < 7; p++)
+                if (t->LL.A[p] >= 0)
+                    it[n++] = (lora_bwd_item_t){dYs[p - 4], xs[p - 4], a->xa[p], LW + t->LL.B[p], LGW + t->LL.A[p], LGW + t->LL.B[p], ind[p - 4], od[p - 4]};
+            if (lora_backward_group(t, it, n, T)) return -1.0f;
         }
         SIDE_MARK(MK_GU);
         {   /* grad_x_norm_ffn = grad_gate Wgate + grad_up Wup (src/train.c:5162-5179) */
@@ -881,7 +950,7 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
         /* attention */
         SIDE_FORK();
         if (!lora) WGEMM(t->g_hidden, a->attn_out, GW + t->L.o, h, qd, T);
-        else if (t->LL.A[3] >= 0 &&
+        else if (ov && t->LL.A[3] >= 0 &&
                  lora_backward(t, t->g_hidden, a->attn_out, a->xa[3], LW + t->LL.B[3], LGW + t->LL.A[3], LGW + t->LL.B[3], T, qd, h, ov)) return -1.0f;
         SIDE_MARK(MK_O);
         GEMM(t->g_hidden, W + t->L.o, t->g_attn, T, qd, h, 0, 0, 0);
@@ -906,12 +975,23 @@ static float run_step(hip_trainer_t* t, const int* tokens, int total_tokens, con
             const seraph_gemm_problem_t qkv[3] = {{t->g_q, a->xn_attn, GW + t->L.q, qd, h}, {t->g_k, a->xn_attn, GW + t->L.k, kv, h},
                                                   {t->g_v, a->xn_attn, GW + t->L.v, kv, h}};
             WGEMM_GROUP(qkv, 3, T);
-        } else {
+        } else if (ov) {
             float* gs[3] = {t->g_q, t->g_k, t->g_v};
             int64_t outs[3] = {qd, kv, kv};
             for (int p = 0; p < 3; p++)
                 if (t->LL.A[p] >= 0 &&
                     lora_backward(t, gs[p], a->xn_attn, a->xa[p], LW + t->LL.B[p], LGW + t->LL.A[p], LGW + t->LL.B[p], T, h, outs[p], ov)) return -1.0f;
+        } else {
+            /* q, k, v and the o adapter left over from above (g_hidden and attn_out are still what they were there) */
+            const float* dYs[4] = {t->g_q, t->g_k, t->g_v, t->g_hidden};
+            const float* xs[4] = {a->xn_attn, a->xn_attn, a->xn_attn, a->attn_out};
+            const int64_t ind[4] = {h, h, h, qd}, od[4] = {qd, kv, kv, h};
+            lora_bwd_item_t it[4];
+            int n = 0;
+            for (int p = 0; p < 4; p++)
+                if (t->LL.A[p] >= 0)
+                    it[n++] = (lora_bwd_item_t){dYs[p], xs[p], a->xa[p], LW + t->LL.B[p], LGW + t->LL.A[p], LGW + t->LL.B[p], ind[p], od[p]};
+            if (lora_backward_group(t, it, n, T)) return -1.0f;
         }
         SIDE_MARK(MK_QKV);
         {   /* grad_x_norm = grad_q Wq + grad_k Wk + grad_v Wv (src/train.c:5294-5339) */

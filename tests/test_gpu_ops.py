@@ -246,6 +246,34 @@ def test_gemm_grouped(ops, orc, tA, tB, shapes, K):
         parity(o, orc.matmul(host(a), host(b), m, n, K, tA, tB), "grouped gemm, overwrite", atol=1e-4)
 
 
+@pytest.mark.parametrize("tA,tB,shapes", [
+    (0, 1, [(2048, 16, 2048), (2048, 16, 2048), (2048, 16, 2048)]),                       # x A^T of the q, k and v adapters
+    (1, 0, [(2048, 16, 2048), (1024, 16, 2048), (1024, 16, 2048), (2048, 16, 2048)]),     # dY^T (x A^T): four adapters' B gradients
+    (0, 0, [(2048, 16, 2048), (2048, 16, 1024), (2048, 16, 1024), (2048, 16, 2048)]),     # dY B: every product its own K
+    (1, 0, [(16, 2048, 2048)] * 4),                                                       # (dY B)^T x: the A gradients
+    (0, 1, [(2048, 2048, 16), (2048, 1024, 16), (2048, 1024, 16)]),                       # (x A^T) B^T onto q, k, v: rank-sized K
+    (0, 1, [(300, 20, 1000), (64, 64, 64)]),                                              # shapes that share no launch: single calls
+])
+@pytest.mark.parametrize("accumulate,alpha", [(False, 2.0), (True, 1.0)])
+def test_gemm_scaled_grouped_equals_the_single_calls(ops, orc, tA, tB, shapes, accumulate, alpha):
+    """The rank-sized products of a layer's adapters in one launch each: every output has the bits of its own
+    seraph_gemm_scaled call, and is the oracle's product within the bar."""
+    r = rng(len(shapes) + 2 * tA + tB + int(alpha))
+    probs, singles, refs = [], [], []
+    for M, N, K in shapes:
+        A = (0.5 * r.standard_normal((K, M) if tA else (M, K))).astype(np.float32)
+        B = (0.5 * r.standard_normal((N, K) if tB else (K, N))).astype(np.float32)
+        C0 = r.standard_normal((M, N)).astype(np.float32)
+        probs.append((dev(A), dev(B), dev(C0), M, N, K))
+        singles.append(ops.gemm_scaled(dev(A), dev(B), M, N, K, tA, tB, out=dev(C0), accumulate=accumulate, alpha=alpha))
+        ref = alpha * orc.matmul(A, B, M, N, K, tA, tB).astype(np.float64)
+        refs.append(ref + C0 if accumulate else ref)
+    outs = ops.gemm_scaled_grouped(probs, tA, tB, accumulate=accumulate, alpha=alpha)
+    for o, single, ref, shape in zip(outs, singles, refs, shapes):
+        assert torch.equal(o, single), shape
+        parity(o, ref, f"grouped scaled gemm {shape}", atol=2e-4)
+
+
 @pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
 @pytest.mark.parametrize("M,N,Ks", [(2048, 512, (1408, 1408)), (2048, 512, (512, 512, 512)), (1024, 2048, (2048, 1024, 1024)),
                                     (4100, 2048, (512, 256)),            # 128x128 tiles with a ragged edge
