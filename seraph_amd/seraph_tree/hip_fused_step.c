@@ -41,6 +41,10 @@ float cuda_eval_forward_opbyop(train_state_t* state, int* tokens, int num_tokens
 float cuda_evaluate_opbyop(train_state_t* state, int* val_tokens, int num_val_tokens, int* offsets, int num_samples,
                            int max_seq_len, int max_eval_samples, cuda_train_context_t* ctx, float* out_perplexity);
 
+/* hip_cuda_backend.c: the front end's profiler when it is attached and recording this step, and an entry with a known time */
+cuda_profiler_t* hip_cuda_active_profiler(cuda_train_context_t* ctx);
+void hip_cuda_profiler_add(cuda_profiler_t* p, const char* name, float elapsed_ms, size_t flops, size_t bytes);
+
 /* one fused trainer per process: the front end drives one model */
 static struct {
     cuda_train_context_t* ctx;
@@ -177,7 +181,27 @@ float cuda_train_step_gpu_full_batch(train_state_t* state, int* tokens_packed, i
     if (total_tokens - batch_size <= 0) return 0.0f;                                 /* :1990-1991 */
     /* the state's counters and learning rate are the truth (a resume sets them): src/train_cuda.c:2287-2303 */
     hip_trainer_set_schedule(t, state->learning_rate, state->optimizer_step, state->accumulation_counter);
+    /* --profile: the fused step has no per-call ops to bracket; its kernels are timed per class (event pairs around
+     * every kernel-library call of this one step) and each class goes to the front end's profiler as one entry, named so
+     * that the profiler's substring categories (src/cuda_profiler.cu:152-172) file it where the op-by-op step's ops go */
+    cuda_profiler_t* prof = hip_cuda_active_profiler(ctx);
+    if (prof) { hip_trainer_enable_op_timing(t, 1); hip_trainer_reset_op_stats(t); }
     const float loss = hip_train_step_full_batch(t, tokens_packed, total_tokens, seq_starts, batch_size, 1);
+    if (prof) {
+        static hip_op_stat_t stats[64];
+        const int n = hip_trainer_op_stats(t, stats, 64);
+        for (int i = 0; i < n; i++) {
+            const char* nm = stats[i].name ? stats[i].name : "";
+            const char* cat = strstr(nm, "gemm") ? "matmul " : !strcmp(nm, "attention_backward") ? "attn_bwd " :
+                              !strcmp(nm, "attention_forward") ? "attn_fwd " : !strcmp(nm, "rmsnorm_backward") ? "rmsnorm_bwd " :
+                              !strcmp(nm, "fill") ? "memset " : "";
+            const char* shortn = strncmp(nm, "seraph::", 8) == 0 ? nm + 8 : nm;
+            char label[80];
+            snprintf(label, sizeof(label), "%s%.*s x%lld", cat, 58 - (int)strlen(cat), shortn, (long long)stats[i].launches);
+            hip_cuda_profiler_add(prof, label, (float)stats[i].ms, (size_t)stats[i].flops, (size_t)stats[i].bytes);
+        }
+        hip_trainer_enable_op_timing(t, 0);
+    }
     state->optimizer_step = hip_trainer_optimizer_step(t);
     state->accumulation_counter = hip_trainer_accumulation_counter(t);
     if ((state->current_step % 20) == 0) {                                           /* :2311-2320 */

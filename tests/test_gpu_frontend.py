@@ -375,7 +375,8 @@ def test_reference_batched_trainer_at_the_33m_shape_8_x_256(tmp_path, orc, binar
 
 
 @needs_ref
-def test_reference_batched_trainer_profile_and_lora(tmp_path, orc):
+@pytest.mark.parametrize("binary", BINARIES)
+def test_reference_batched_trainer_profile_and_lora(tmp_path, orc, binary):
     mdir = str(tmp_path / "model")
     ocfg, cfg, p0 = make_model_dir(mdir, orc, SHAPE, seed=71)
     add_tokenizer(mdir, SHAPE["vocab"])
@@ -383,17 +384,21 @@ def test_reference_batched_trainer_profile_and_lora(tmp_path, orc):
     ttok = os.path.join(mdir, "train.ttok")
     write_ttok(ttok, samples, vocab=SHAPE["vocab"])
     ckpt = tmp_path / "p"
-    rc, out, err = run_ref([mdir, ttok, "--full-training", "--batch", 2, "--max-seq", 32, "--profile", 2, "--checkpoint", ckpt])
+    rc, out, err = run_ref([mdir, ttok, "--full-training", "--batch", 2, "--max-seq", 32, "--profile", 2, "--checkpoint", ckpt], binary=binary)
     assert rc == 0, (out[-1500:], err[-1500:])
     plog = open(ckpt / "profile.log").read()
+    # the op-by-op step reports every op; the fused step one entry per kernel class, under names that land in the same categories
+    ops = ("matmul_Bt [", "attn_bwd_packed", "adamw ") if binary == REF_BIN else ("matmul gemm_f32_mfma", "attn_bwd attention_backward x2", "adamw x1")
     for needle in ("SERAPH STEP PROFILER", "CATEGORY BREAKDOWN", "matmul (all)", "attention bwd", "PER-OPERATION DETAIL",
-                   "PERFORMANCE METRICS", "TOP 20 SLOWEST OPERATIONS", "matmul_Bt [", "attn_bwd_packed", "adamw "):
+                   "PERFORMANCE METRICS", "TOP 20 SLOWEST OPERATIONS") + ops:
         assert needle in plog, needle
+    cats = dict(re.findall(r"^  (matmul \(all\)|attention fwd|attention bwd|rmsnorm fwd|rmsnorm bwd|cross_entropy|adamw) +([0-9.]+) ", plog, re.M))
+    assert len(cats) == 7 and all(float(v) > 0 for v in cats.values()), cats
     assert "PROFILE STEP 2 (batch=2" in out
     # LoRA through the reference's trainer: adapters start with B = 0, so the first loss is the base model's
     # (the adapter seed is the wall clock there, src/tools: srand(time(NULL)); later steps are not comparable)
     rc, out, err = run_ref([mdir, ttok, "--batch", 2, "--max-seq", 32, "--lr", 1e-3, "--log-every", 1, "--lora-rank", 4,
-                            "--checkpoint", tmp_path / "q"])
+                            "--checkpoint", tmp_path / "q"], binary=binary)
     assert rc == 0, (out[-1500:], err[-1500:])
     tokens = np.concatenate(samples)
     offsets = np.concatenate([[0], np.cumsum([len(s) for s in samples])]).tolist()
