@@ -517,10 +517,12 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_pipelined_group
 // timing.  Same loaders and staging as the pipelined kernel.
 // With `slices` > 1 the grid's y index also cuts K into that many equal runs of stages; a workgroup then
 // stores its tile of run y, unscaled, into part[y] (M x N each) and gemm_slices_sum_kernel adds the runs.
-template <bool A_KC, bool B_KC>
+// With CHAIN the tile is the sum of several products (one run of K each): the four partial accumulators go on from one
+// term to the next and meet in LDS once.
+template <bool A_KC, bool B_KC, bool CHAIN = false>
 __device__ __forceinline__ void splitk_body(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
                                             int64_t M, int64_t N, int64_t K, int accumulate, int nbn, int tile,
-                                            int slices, int slice, float* __restrict__ part) {
+                                            int slices, int slice, float* __restrict__ part, const GemmChain* chain = nullptr) {
     constexpr int BT = 32;
     constexpr int A_FLOATS = lds_floats<BT, A_KC>(), B_FLOATS = lds_floats<BT, B_KC>();
     __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
@@ -530,11 +532,15 @@ __device__ __forceinline__ void splitk_body(const float* __restrict__ A, const f
     const int64_t m0 = (int64_t)pm * BT, n0 = (int64_t)pn * BT;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
-    const int64_t lda = A_KC ? K : M, ldb = B_KC ? K : N;
 
     v16f acc;
 #pragma unroll
     for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+
+    const int terms = CHAIN ? chain->count : 1;
+    for (int term = 0; term < terms; term++) {                 // (a term's last stage ends with a barrier: its LDS reads are over)
+    if (CHAIN) { A = chain->A[term]; B = chain->B[term]; K = chain->K[term]; }
+    const int64_t lda = A_KC ? K : M, ldb = B_KC ? K : N;
 
     // Four stages of both operands in flight (two float4 per lane and stage): with one or two workgroups per
     // CU nothing else hides the memory latency, and two stages ahead is less than one round trip.
@@ -603,6 +609,7 @@ __device__ __forceinline__ void splitk_body(const float* __restrict__ A, const f
     if (kt < nk) stage(std::integral_constant<int, 0>{}, kt);
     if (kt + 1 < nk) stage(std::integral_constant<int, 1>{}, kt + 1);
     if (kt + 2 < nk) stage(std::integral_constant<int, 2>{}, kt + 2);
+    }   // term
 
     // fixed-order sum of the four partial tiles
 #pragma unroll
@@ -633,6 +640,13 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_kernel(c
                                                                                int slices, float* __restrict__ part) {
     (void)nbm;
     splitk_body<A_KC, B_KC>(A, B, C, M, N, K, accumulate, nbn, (int)blockIdx.x, slices, (int)blockIdx.y, part);
+}
+
+// the sum of up to three products into one C (one run of K each, no slices)
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kGemmThreads, 4) void gemm_f32_mfma_splitk_chain_kernel(const GemmChain chain, float* __restrict__ C,
+                                                                                     int64_t M, int64_t N, int accumulate, int nbn) {
+    splitk_body<A_KC, B_KC, true>(nullptr, nullptr, C, M, N, 0, accumulate, nbn, (int)blockIdx.x, 1, 0, nullptr, &chain);
 }
 
 // the grouped form of the above (one run of K, no slices); nbm / nbn / first count 32 x 32 tiles here
@@ -973,19 +987,25 @@ extern "C" int seraph_gemm_grouped(const seraph_gemm_problem_t* problems, int co
 }
 
 // ---------------------------------------------------------------------------------------------
-// C (+)= sum of products that share M and N: one launch when every term suits the pipelined kernel and the output has
-// enough 64x64 tiles for it, else one product after the other.
+// C (+)= sum of products that share M and N: one launch when every term suits the pipelined loaders (whole K stages,
+// 16-byte aligned operands), else one product after the other.
 static bool chain_ok(const seraph_gemm_term_t* t, int count, const float* C, int64_t M, int64_t N, int tA, int tB) {
     if (count < 2 || count > kMaxChain || M <= 0 || N <= 0 || !C) return false;
-    int64_t ksum = 0;
     for (int i = 0; i < count; i++) {
         const int64_t K = t[i].K, lda = tA ? M : K, ldb = tB ? K : N;
         if (!t[i].A || !t[i].B || lda % 4 || ldb % 4 || !aligned16(t[i].A) || !aligned16(t[i].B)) return false;
         if (!pipelined_ok(M, N, K, tA, tB)) return false;
-        ksum += K;
     }
-    // (no 32x32 form of the sum: with fewer 64x64 tiles than compute units the products run one after the other)
-    return ksum < 256 || use_big_tiles(M, N) || ceil_div(M, 64) * ceil_div(N, 64) >= num_compute_units();
+    return ceil_div(M, 32) * ceil_div(N, 32) <= 0x7fffffff;
+}
+// The sum on 32x32 tiles whose waves share out K: with fewer 64x64 tiles than compute units.  From there up to the
+// single product's limit (small_tiles_pay) the 32x32 form is 3 % ahead alone (2048 x 512 with K 1408 + 1408: 57 against
+// 59 us) but 2.4 % behind inside the 33M step, where its 1024 workgroups crowd the weight gradients on the second
+// stream (4.46 against 4.36 ms, alternating builds on one GPU): there the 64x64 form stays.
+static bool chain_splitk(const seraph_gemm_term_t* t, int count, int64_t M, int64_t N) {
+    int64_t ksum = 0;
+    for (int i = 0; i < count; i++) ksum += t[i].K;
+    return !use_big_tiles(M, N) && ksum >= 256 && ceil_div(M, 64) * ceil_div(N, 64) < num_compute_units();
 }
 
 extern "C" const char* seraph_gemm_chain_kernel_name(const seraph_gemm_term_t* terms, int count, const float* C, int64_t M, int64_t N,
@@ -996,6 +1016,9 @@ extern "C" const char* seraph_gemm_chain_kernel_name(const seraph_gemm_term_t* t
         {"seraph::gemm_f32_mfma_pipelined_chain_kernel<2, 2, true, false>", "seraph::gemm_f32_mfma_pipelined_chain_kernel<2, 2, true, true>",
          "seraph::gemm_f32_mfma_pipelined_chain_kernel<2, 2, false, false>", "seraph::gemm_f32_mfma_pipelined_chain_kernel<2, 2, false, true>"}};
     if (!terms || !chain_ok(terms, count, C, M, N, transpose_A, transpose_B)) return "gemm (chain run as single products)";
+    static const char* split[4] = {"seraph::gemm_f32_mfma_splitk_chain_kernel<true, false>", "seraph::gemm_f32_mfma_splitk_chain_kernel<true, true>",
+                                   "seraph::gemm_f32_mfma_splitk_chain_kernel<false, false>", "seraph::gemm_f32_mfma_splitk_chain_kernel<false, true>"};
+    if (chain_splitk(terms, count, M, N)) return split[(transpose_A ? 2 : 0) + (transpose_B ? 1 : 0)];
     return names[use_big_tiles(M, N) ? 1 : 0][(transpose_A ? 2 : 0) + (transpose_B ? 1 : 0)];
 }
 
@@ -1016,13 +1039,24 @@ extern "C" int seraph_gemm_chain(const seraph_gemm_term_t* terms, int count, flo
         const int j = i < count ? i : count - 1;
         ch.A[i] = terms[j].A; ch.B[i] = terms[j].B; ch.K[i] = terms[j].K;
     }
+    hipStream_t st = as_stream(s);
+    const int form = (transpose_A ? 2 : 0) + (transpose_B ? 1 : 0);
+    if (chain_splitk(terms, count, M, N)) {
+        const int64_t nbn = ceil_div(N, 32);
+        const dim3 grid((unsigned)(ceil_div(M, 32) * nbn)), block(kGemmThreads);
+        switch (form) {
+            case 0: hipLaunchKernelGGL((gemm_f32_mfma_splitk_chain_kernel<true, false>), grid, block, 0, st, ch, C, M, N, accumulate, (int)nbn); break;
+            case 1: hipLaunchKernelGGL((gemm_f32_mfma_splitk_chain_kernel<true, true>), grid, block, 0, st, ch, C, M, N, accumulate, (int)nbn); break;
+            case 2: hipLaunchKernelGGL((gemm_f32_mfma_splitk_chain_kernel<false, false>), grid, block, 0, st, ch, C, M, N, accumulate, (int)nbn); break;
+            default: hipLaunchKernelGGL((gemm_f32_mfma_splitk_chain_kernel<false, true>), grid, block, 0, st, ch, C, M, N, accumulate, (int)nbn); break;
+        }
+        SERAPH_LAUNCH_CHECK();
+        return SERAPH_OK;
+    }
     const bool big = use_big_tiles(M, N);
     const int tile = big ? 128 : 64;
     const int64_t nbm = ceil_div(M, tile), nbn = ceil_div(N, tile);
-    SERAPH_REQUIRE(nbm * nbn <= 0x7fffffff, "gemm_chain: too many tiles");
-    hipStream_t st = as_stream(s);
     const dim3 grid((unsigned)(nbm * nbn)), block(kGemmThreads);
-    const int form = (transpose_A ? 2 : 0) + (transpose_B ? 1 : 0);
 #define GOC(TMN) \
     switch (form) { \
         case 0: hipLaunchKernelGGL((gemm_f32_mfma_pipelined_chain_kernel<TMN, TMN, true, false>), grid, block, 0, st, ch, C, M, N, accumulate, (int)nbm, (int)nbn); break; \

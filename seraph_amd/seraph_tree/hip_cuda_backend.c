@@ -34,6 +34,7 @@
  * handle as their `stream` argument, which is what the reference's callers pass.
  */
 #include <math.h>
+#include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -58,6 +59,26 @@ static hc_state_t* state_of(cuda_train_context_t* ctx) { return ctx ? (hc_state_
 
 static void op_failed(hc_state_t* st, const char* what) {
     if (st->errors++ < 20) fprintf(stderr, "HIP: %s failed: %s\n", what, seraph_hip_last_error());
+}
+
+/* 1 when each of the `pairs` (buffer, number of 4-byte values) arguments fits its buffer (a NULL buffer is an optional
+ * operand the op goes without).  Otherwise the op is refused with a message and nothing is launched: a shape that
+ * reaches past the end of a buffer is a memory fault on this device, not the silent garbage it is elsewhere. */
+#define FIT(buf, n) (const cuda_buffer_t*)(buf), (size_t)(n)
+static int fits(hc_state_t* st, const char* op, int pairs, ...) {
+    va_list ap;
+    va_start(ap, pairs);
+    int ok = 1;
+    for (int i = 0; i < pairs; i++) {
+        const cuda_buffer_t* buf = va_arg(ap, const cuda_buffer_t*);
+        const size_t n = va_arg(ap, size_t);
+        if (!buf || n <= buf->size / 4) continue;
+        if (ok && st->errors++ < 20)
+            fprintf(stderr, "HIP: %s skipped: operand %d has %zu bytes, the shape needs %zu\n", op, i, buf->size, n * 4);
+        ok = 0;
+    }
+    va_end(ap);
+    return ok;
 }
 
 static void* scratch(hc_state_t* st, size_t bytes) {
@@ -420,56 +441,79 @@ static void gemm_op(cuda_train_context_t* ctx, const char* label, const float* A
         seraph_gemm_scaled(A, B, C, M, N, K, tA, tB, acc, 1.0f, ws, ws ? need : 0, st->stream));
 }
 
+/* (The reference's batched LoRA step hands every adapter the final hidden gradient as its output gradient,
+ * src/train_cuda.c:2596-2644, which is smaller than tokens x out_dim for any adapter whose out_dim exceeds hidden_size:
+ * the products check their operands like every other op here.) */
+static int gemm_fits(cuda_train_context_t* ctx, const char* label, const cuda_buffer_t* A, const cuda_buffer_t* B, const cuda_buffer_t* C,
+                     int M, int N, int K) {
+    hc_state_t* st = state_of(ctx);
+    if (!st || M < 0 || N < 0 || K < 0) return 0;
+    char name[80];
+    snprintf(name, sizeof(name), "%s [%dx%d K=%d]", label, M, N, K);
+    return fits(st, name, 3, FIT(A, (size_t)M * K), FIT(B, (size_t)N * K), FIT(C, (size_t)M * N));
+}
+static void gemm_bufs(cuda_train_context_t* ctx, const char* label, cuda_buffer_t* A, cuda_buffer_t* B, cuda_buffer_t* C,
+                      int M, int N, int K, int tA, int tB, int acc) {
+    if (A && B && C && gemm_fits(ctx, label, A, B, C, M, N, K)) gemm_op(ctx, label, A->data, B->data, C->data, M, N, K, tA, tB, acc);
+}
+
 void cuda_train_matmul(cuda_train_context_t* ctx, cuda_buffer_t* A, cuda_buffer_t* B, cuda_buffer_t* C, int M, int N, int K) {
-    if (A && B && C) gemm_op(ctx, "matmul", A->data, B->data, C->data, M, N, K, 0, 0, 0);
+    gemm_bufs(ctx, "matmul", A, B, C, M, N, K, 0, 0, 0);
 }
 void cuda_train_matmul_transpose(cuda_train_context_t* ctx, cuda_buffer_t* A, cuda_buffer_t* B, cuda_buffer_t* C, int M, int N, int K,
                                  int transpose_A, int transpose_B, int accumulate) {
-    if (!A || !B || !C) return;
     const char* label = (transpose_A && !transpose_B) ? "matmul_At" : (!transpose_A && transpose_B) ? "matmul_Bt" : "matmul";
-    gemm_op(ctx, label, A->data, B->data, C->data, M, N, K, transpose_A, transpose_B, accumulate);
+    gemm_bufs(ctx, label, A, B, C, M, N, K, transpose_A, transpose_B, accumulate);
 }
 
 void cuda_train_silu(cuda_train_context_t* ctx, cuda_buffer_t* input, cuda_buffer_t* output, size_t count) {
     hc_state_t* st = state_of(ctx);
-    if (st && input && output) RUN(st, "silu", 0, 8 * count, seraph_silu(input->data, output->data, count, st->stream));
+    if (st && input && output && fits(st, "silu", 2, FIT(input, count), FIT(output, count))) RUN(st, "silu", 0, 8 * count, seraph_silu(input->data, output->data, count, st->stream));
 }
 void cuda_train_rmsnorm(cuda_train_context_t* ctx, cuda_buffer_t* input, cuda_buffer_t* scale, cuda_buffer_t* output, int rows, int cols, float eps) {
     hc_state_t* st = state_of(ctx);
-    if (!st || !input || !scale || !output) return;
+    if (!st || !input || !scale || !output || rows < 0 || cols < 0) return;
     char name[80];
     snprintf(name, sizeof(name), "rmsnorm [%dx%d]", rows, cols);
+    if (!fits(st, name, 3, FIT(input, (size_t)rows * cols), FIT(scale, cols), FIT(output, (size_t)rows * cols))) return;
     RUN(st, name, 0, (size_t)8 * rows * cols, seraph_rmsnorm(input->data, scale->data, output->data, rows, cols, eps, st->stream));
 }
 void cuda_train_rope(cuda_train_context_t* ctx, cuda_buffer_t* x_in, cuda_buffer_t* x_out, int seq_len, int num_heads, int head_dim, float rope_theta) {
     hc_state_t* st = state_of(ctx);
-    if (st && x_in && x_out) RUN(st, "rope_fwd", 0, (size_t)8 * seq_len * num_heads * head_dim,
+    if (st && x_in && x_out && seq_len >= 0 && num_heads >= 0 && head_dim >= 0 &&
+        fits(st, "rope_fwd", 2, FIT(x_in, (size_t)seq_len * num_heads * head_dim), FIT(x_out, (size_t)seq_len * num_heads * head_dim)))
+        RUN(st, "rope_fwd", 0, (size_t)8 * seq_len * num_heads * head_dim,
                                  seraph_rope(x_in->data, x_out->data, NULL, 1, seq_len, num_heads, head_dim, rope_theta, 0, st->stream));
 }
 void cuda_train_rope_packed(cuda_train_context_t* ctx, cuda_buffer_t* x_in, cuda_buffer_t* x_out, cuda_buffer_t* seq_starts,
                             int total_tokens, int batch_size, int num_heads, int head_dim, float rope_theta) {
     hc_state_t* st = state_of(ctx);
-    if (st && x_in && x_out && seq_starts)
+    if (st && x_in && x_out && seq_starts && total_tokens >= 0 && batch_size >= 0 && num_heads >= 0 && head_dim >= 0 &&
+        fits(st, "rope_fwd_packed", 3, FIT(x_in, (size_t)total_tokens * num_heads * head_dim), FIT(x_out, (size_t)total_tokens * num_heads * head_dim),
+             FIT(seq_starts, (size_t)batch_size + 1)))
         RUN(st, "rope_fwd_packed", 0, (size_t)8 * total_tokens * num_heads * head_dim,
             seraph_rope(x_in->data, x_out->data, (const uint32_t*)seq_starts->data, batch_size, total_tokens, num_heads, head_dim, rope_theta, 0, st->stream));
 }
 void cuda_train_add(cuda_train_context_t* ctx, cuda_buffer_t* A, cuda_buffer_t* B, cuda_buffer_t* C, size_t count) {
     hc_state_t* st = state_of(ctx);
-    if (st && A && B && C) RUN(st, "add", 0, 12 * count, seraph_add(A->data, B->data, C->data, count, st->stream));
+    if (st && A && B && C && fits(st, "add", 3, FIT(A, count), FIT(B, count), FIT(C, count))) RUN(st, "add", 0, 12 * count, seraph_add(A->data, B->data, C->data, count, st->stream));
 }
 void cuda_train_mul(cuda_train_context_t* ctx, cuda_buffer_t* A, cuda_buffer_t* B, cuda_buffer_t* C, size_t count) {
     hc_state_t* st = state_of(ctx);
-    if (st && A && B && C) RUN(st, "mul", 0, 12 * count, seraph_mul(A->data, B->data, C->data, count, st->stream));
+    if (st && A && B && C && fits(st, "mul", 3, FIT(A, count), FIT(B, count), FIT(C, count))) RUN(st, "mul", 0, 12 * count, seraph_mul(A->data, B->data, C->data, count, st->stream));
 }
 void cuda_train_scale(cuda_train_context_t* ctx, cuda_buffer_t* A, size_t count, float alpha) {
     hc_state_t* st = state_of(ctx);
-    if (st && A) RUN(st, "scale", 0, 8 * count, seraph_scale(A->data, count, alpha, st->stream));
+    if (st && A && fits(st, "scale", 1, FIT(A, count))) RUN(st, "scale", 0, 8 * count, seraph_scale(A->data, count, alpha, st->stream));
 }
 
 static void attention_fwd(cuda_train_context_t* ctx, const char* name, cuda_buffer_t* Q, cuda_buffer_t* K, cuda_buffer_t* V,
                           cuda_buffer_t* out, cuda_buffer_t* lse_out, const uint32_t* starts, int batch, int T, int H, int KVH, int D) {
     hc_state_t* st = state_of(ctx);
-    if (!st || !Q || !K || !V || !out) return;
+    if (!st || !Q || !K || !V || !out || batch < 0 || T < 0 || H < 0 || KVH < 0 || D < 0) return;
+    if (!fits(st, name, 5, FIT(Q, (size_t)T * H * D), FIT(K, (size_t)T * KVH * D), FIT(V, (size_t)T * KVH * D), FIT(out, (size_t)T * H * D),
+              FIT(lse_out, (size_t)T * H)))
+        return;
     /* the reference's standard kernel ignores lse_out (:2855); writing it costs nothing here and lets the
      * backward skip its recomputation in both modes - same numbers either way */
     float* lse = lse_out ? lse_out->data : NULL;
@@ -486,7 +530,8 @@ void cuda_train_batch_attention_packed(cuda_train_context_t* ctx, cuda_buffer_t*
                                        cuda_buffer_t* lse_out, cuda_buffer_t* seq_starts, int total_tokens, int batch_size,
                                        int num_heads, int kv_heads, int head_dim, int max_seq_in_batch) {
     (void)max_seq_in_batch;
-    if (!seq_starts) return;
+    hc_state_t* st = state_of(ctx);
+    if (!st || !seq_starts || batch_size < 0 || !fits(st, "attn_fwd_packed", 1, FIT(seq_starts, (size_t)batch_size + 1))) return;
     attention_fwd(ctx, ctx && ctx->use_flash_attn ? "flash_attn_fwd_packed" : "attn_fwd_packed", Q, K, V, out, lse_out,
                   (const uint32_t*)seq_starts->data, batch_size, total_tokens, num_heads, kv_heads, head_dim);
 }
@@ -494,7 +539,8 @@ void cuda_train_batch_attention_packed(cuda_train_context_t* ctx, cuda_buffer_t*
 void cuda_train_embed_lookup(cuda_train_context_t* ctx, cuda_buffer_t* tokens_u32, cuda_buffer_t* embed_weight, cuda_buffer_t* out_hidden,
                              int seq_len, int hidden_size, int vocab_size) {
     hc_state_t* st = state_of(ctx);
-    if (st && tokens_u32 && embed_weight && out_hidden)
+    if (st && tokens_u32 && embed_weight && out_hidden && seq_len >= 0 && hidden_size >= 0 && vocab_size >= 0 &&
+        fits(st, "embed_lookup", 3, FIT(tokens_u32, seq_len), FIT(embed_weight, (size_t)vocab_size * hidden_size), FIT(out_hidden, (size_t)seq_len * hidden_size)))
         RUN(st, "embed_lookup", 0, (size_t)8 * seq_len * hidden_size,
             seraph_embed_lookup((const uint32_t*)tokens_u32->data, embed_weight->data, out_hidden->data, seq_len, hidden_size, vocab_size, st->stream));
 }
@@ -503,9 +549,10 @@ void cuda_train_embed_lookup(cuda_train_context_t* ctx, cuda_buffer_t* tokens_u3
 void cuda_train_cross_entropy_grad(cuda_train_context_t* ctx, cuda_buffer_t* logits, cuda_buffer_t* targets_u32, cuda_buffer_t* grad_logits,
                                    cuda_buffer_t* loss_rows, int rows, int cols) {
     hc_state_t* st = state_of(ctx);
-    if (!st || !logits || !targets_u32 || !grad_logits || !loss_rows) return;
+    if (!st || !logits || !targets_u32 || !grad_logits || !loss_rows || rows < 0 || cols < 0) return;
     char name[80];
     snprintf(name, sizeof(name), "cross_entropy [%dx%d]", rows, cols);
+    if (!fits(st, name, 4, FIT(logits, (size_t)rows * cols), FIT(targets_u32, rows), FIT(grad_logits, (size_t)rows * cols), FIT(loss_rows, rows))) return;
     RUN(st, name, 0, (size_t)rows * cols * 4 * 3,
         seraph_cross_entropy_grad(logits->data, (const uint32_t*)targets_u32->data, grad_logits->data, loss_rows->data, NULL, 1, rows, cols, rows, st->stream));
 }
@@ -513,30 +560,37 @@ void cuda_train_cross_entropy_grad_packed(cuda_train_context_t* ctx, cuda_buffer
                                           cuda_buffer_t* loss_rows, cuda_buffer_t* seq_starts, int total_tokens, int batch_size, int vocab_size,
                                           int num_valid_predictions) {
     hc_state_t* st = state_of(ctx);
-    if (!st || !logits || !targets_u32 || !grad_logits || !loss_rows || !seq_starts) return;
+    if (!st || !logits || !targets_u32 || !grad_logits || !loss_rows || !seq_starts || total_tokens < 0 || batch_size < 0 || vocab_size < 0) return;
+    if (!fits(st, "cross_entropy_packed", 5, FIT(logits, (size_t)total_tokens * vocab_size), FIT(targets_u32, total_tokens),
+              FIT(grad_logits, (size_t)total_tokens * vocab_size), FIT(loss_rows, total_tokens), FIT(seq_starts, (size_t)batch_size + 1)))
+        return;
     RUN(st, "cross_entropy_packed", 0, (size_t)total_tokens * vocab_size * 8,
         seraph_cross_entropy_grad(logits->data, (const uint32_t*)targets_u32->data, grad_logits->data, loss_rows->data,
                                   (const uint32_t*)seq_starts->data, batch_size, total_tokens, vocab_size, num_valid_predictions, st->stream));
 }
 void cuda_train_reduce_sum(cuda_train_context_t* ctx, cuda_buffer_t* in_buf, cuda_buffer_t* out_buf, size_t count) {
     hc_state_t* st = state_of(ctx);
-    if (st && in_buf && out_buf && count) RUN(st, "reduce_sum", 0, 4 * count, seraph_reduce_sum(in_buf->data, out_buf->data, count, st->stream));
+    if (st && in_buf && out_buf && count && fits(st, "reduce_sum", 2, FIT(in_buf, count), FIT(out_buf, (count + 511) / 512))) RUN(st, "reduce_sum", 0, 4 * count, seraph_reduce_sum(in_buf->data, out_buf->data, count, st->stream));
 }
 void cuda_train_silu_backward(cuda_train_context_t* ctx, cuda_buffer_t* input, cuda_buffer_t* grad_output, cuda_buffer_t* grad_input, size_t count) {
     hc_state_t* st = state_of(ctx);
-    if (st && input && grad_output && grad_input)
+    if (st && input && grad_output && grad_input && fits(st, "silu_bwd", 3, FIT(input, count), FIT(grad_output, count), FIT(grad_input, count)))
         RUN(st, "silu_bwd", 0, 12 * count, seraph_silu_backward(input->data, grad_output->data, grad_input->data, count, st->stream));
 }
 void cuda_train_elementwise_mul_backward(cuda_train_context_t* ctx, cuda_buffer_t* A, cuda_buffer_t* B, cuda_buffer_t* grad_C,
                                          cuda_buffer_t* grad_A, cuda_buffer_t* grad_B, size_t count) {
     hc_state_t* st = state_of(ctx);
-    if (st && A && B && grad_C && grad_A && grad_B)
+    if (st && A && B && grad_C && grad_A && grad_B &&
+        fits(st, "mul_bwd", 5, FIT(A, count), FIT(B, count), FIT(grad_C, count), FIT(grad_A, count), FIT(grad_B, count)))
         RUN(st, "mul_bwd", 0, 20 * count, seraph_mul_backward(A->data, B->data, grad_C->data, grad_A->data, grad_B->data, count, st->stream));
 }
 void cuda_train_rmsnorm_backward_batch(cuda_train_context_t* ctx, cuda_buffer_t* input, cuda_buffer_t* scale, cuda_buffer_t* grad_output,
                                        cuda_buffer_t* grad_input, cuda_buffer_t* grad_scale, int rows, int cols, float eps) {
     hc_state_t* st = state_of(ctx);
-    if (!st || !input || !scale || !grad_output || !grad_input || !grad_scale) return;
+    if (!st || !input || !scale || !grad_output || !grad_input || !grad_scale || rows < 0 || cols < 0) return;
+    if (!fits(st, "rmsnorm_bwd", 5, FIT(input, (size_t)rows * cols), FIT(scale, cols), FIT(grad_output, (size_t)rows * cols),
+              FIT(grad_input, (size_t)rows * cols), FIT(grad_scale, cols)))
+        return;
     void* ws = scratch(st, seraph_rmsnorm_backward_ws_bytes(rows, cols));
     if (!ws) return;
     char name[80];
@@ -546,13 +600,17 @@ void cuda_train_rmsnorm_backward_batch(cuda_train_context_t* ctx, cuda_buffer_t*
 }
 void cuda_train_rope_backward(cuda_train_context_t* ctx, cuda_buffer_t* x_in, cuda_buffer_t* x_out, int seq_len, int num_heads, int head_dim, float rope_theta) {
     hc_state_t* st = state_of(ctx);
-    if (st && x_in && x_out) RUN(st, "rope_bwd", 0, (size_t)8 * seq_len * num_heads * head_dim,
+    if (st && x_in && x_out && seq_len >= 0 && num_heads >= 0 && head_dim >= 0 &&
+        fits(st, "rope_bwd", 2, FIT(x_in, (size_t)seq_len * num_heads * head_dim), FIT(x_out, (size_t)seq_len * num_heads * head_dim)))
+        RUN(st, "rope_bwd", 0, (size_t)8 * seq_len * num_heads * head_dim,
                                  seraph_rope(x_in->data, x_out->data, NULL, 1, seq_len, num_heads, head_dim, rope_theta, 1, st->stream));
 }
 void cuda_train_rope_backward_packed(cuda_train_context_t* ctx, cuda_buffer_t* x_in, cuda_buffer_t* x_out, cuda_buffer_t* seq_starts,
                                      int total_tokens, int batch_size, int num_heads, int head_dim, float rope_theta) {
     hc_state_t* st = state_of(ctx);
-    if (st && x_in && x_out && seq_starts)
+    if (st && x_in && x_out && seq_starts && total_tokens >= 0 && batch_size >= 0 && num_heads >= 0 && head_dim >= 0 &&
+        fits(st, "rope_bwd_packed", 3, FIT(x_in, (size_t)total_tokens * num_heads * head_dim), FIT(x_out, (size_t)total_tokens * num_heads * head_dim),
+             FIT(seq_starts, (size_t)batch_size + 1)))
         RUN(st, "rope_bwd_packed", 0, (size_t)8 * total_tokens * num_heads * head_dim,
             seraph_rope(x_in->data, x_out->data, (const uint32_t*)seq_starts->data, batch_size, total_tokens, num_heads, head_dim, rope_theta, 1, st->stream));
 }
@@ -561,7 +619,11 @@ static void attention_bwd(cuda_train_context_t* ctx, const char* name, cuda_buff
                           cuda_buffer_t* attn_out, cuda_buffer_t* lse, cuda_buffer_t* grad_out, cuda_buffer_t* gQ, cuda_buffer_t* gK,
                           cuda_buffer_t* gV, const uint32_t* starts, int batch, int T, int H, int KVH, int D, int max_seq) {
     hc_state_t* st = state_of(ctx);
-    if (!st || !Q || !K || !V || !grad_out || !gQ || !gK || !gV) return;
+    if (!st || !Q || !K || !V || !grad_out || !gQ || !gK || !gV || batch < 0 || T < 0 || H < 0 || KVH < 0 || D < 0) return;
+    const size_t nq = (size_t)T * H * D, nkv = (size_t)T * KVH * D;
+    if (!fits(st, name, 9, FIT(Q, nq), FIT(K, nkv), FIT(V, nkv), FIT(attn_out, nq), FIT(lse, (size_t)T * H), FIT(grad_out, nq), FIT(gQ, nq),
+              FIT(gK, nkv), FIT(gV, nkv)))
+        return;
     const int saved = attn_out && lse;             /* both come from attention_fwd above; else recomputed */
     size_t need = seraph_attention_backward_ws_bytes_banded(T, H, KVH, D, max_seq);
     if (need > ((size_t)8 << 30)) need = seraph_attention_backward_ws_bytes(T, H, KVH, D);
@@ -582,7 +644,8 @@ void cuda_train_batch_attention_backward_packed(cuda_train_context_t* ctx, cuda_
                                                 cuda_buffer_t* attn_out, cuda_buffer_t* lse, cuda_buffer_t* grad_out, cuda_buffer_t* grad_Q,
                                                 cuda_buffer_t* grad_K, cuda_buffer_t* grad_V, cuda_buffer_t* seq_starts, int total_tokens,
                                                 int batch_size, int num_heads, int kv_heads, int head_dim, int max_seq_in_batch) {
-    if (!seq_starts) return;
+    hc_state_t* st = state_of(ctx);
+    if (!st || !seq_starts || batch_size < 0 || !fits(st, "attn_bwd_packed", 1, FIT(seq_starts, (size_t)batch_size + 1))) return;
     attention_bwd(ctx, ctx && ctx->use_flash_attn ? "flash_attn_bwd_packed" : "attn_bwd_packed", Q, K, V, attn_out, lse, grad_out, grad_Q,
                   grad_K, grad_V, (const uint32_t*)seq_starts->data, batch_size, total_tokens, num_heads, kv_heads, head_dim,
                   max_seq_in_batch > 0 ? max_seq_in_batch : total_tokens);
@@ -591,7 +654,9 @@ void cuda_train_batch_attention_backward_packed(cuda_train_context_t* ctx, cuda_
 void cuda_train_embedding_backward(cuda_train_context_t* ctx, cuda_buffer_t* tokens_u32, cuda_buffer_t* grad_hidden, cuda_buffer_t* grad_embed,
                                    int seq_len, int hidden_size, int vocab_size) {
     hc_state_t* st = state_of(ctx);
-    if (!st || !tokens_u32 || !grad_hidden || !grad_embed) return;
+    if (!st || !tokens_u32 || !grad_hidden || !grad_embed || seq_len < 0 || hidden_size < 0 || vocab_size < 0) return;
+    if (!fits(st, "embed_bwd", 3, FIT(tokens_u32, seq_len), FIT(grad_hidden, (size_t)seq_len * hidden_size), FIT(grad_embed, (size_t)vocab_size * hidden_size)))
+        return;
     void* ws = scratch(st, seraph_embedding_backward_ws_bytes(seq_len, vocab_size));
     if (!ws) return;
     RUN(st, "embed_bwd", 0, (size_t)12 * seq_len * hidden_size,
@@ -607,12 +672,13 @@ void cuda_train_adamw_update(cuda_train_context_t* ctx, cuda_buffer_t* weight, c
     char name[80];
     if (cols > 0) snprintf(name, sizeof(name), "adamw %s [%dx%d]", tensor_name ? tensor_name : "", rows, cols);
     else snprintf(name, sizeof(name), "adamw %s [%d]", tensor_name ? tensor_name : "", rows);
+    if (!fits(st, name, 4, FIT(weight, size), FIT(grad, size), FIT(m, size), FIT(v, size))) return;
     RUN(st, name, 0, size * 4 * 4, seraph_adamw(weight->data, grad->data, m->data, v->data, size, lr, beta1, beta2, weight_decay, eps, step, 0.0f, st->stream));
 }
 
 void cuda_train_nan_check(cuda_train_context_t* ctx, cuda_buffer_t* input, size_t count_floats, cuda_buffer_t* flags_u32, uint32_t flag_index) {
     hc_state_t* st = state_of(ctx);
-    if (st && input && flags_u32) RUN(st, "nan_check", 0, 4 * count_floats,
+    if (st && input && flags_u32 && fits(st, "nan_check", 2, FIT(input, count_floats), FIT(flags_u32, (size_t)flag_index + 1))) RUN(st, "nan_check", 0, 4 * count_floats,
                                       seraph_nan_check(input->data, count_floats, (uint32_t*)flags_u32->data, flag_index, st->stream));
 }
 
@@ -623,6 +689,12 @@ void cuda_train_lora_backward(cuda_train_context_t* ctx, cuda_buffer_t* grad_out
                               float scale) {
     if (!grad_output || !input || !A || !B || !gA || !gB || !hidden_tmp) return;
     const size_t n = (size_t)seq_len * (size_t)rank;
+    /* all four products or none: a half-updated adapter would be worse than an untouched one */
+    if (!gemm_fits(ctx, "lora_recompute", input, A, hidden_tmp, seq_len, rank, in_dim) ||
+        !gemm_fits(ctx, "lora_gB", grad_output, hidden_tmp, gB, out_dim, rank, seq_len) ||
+        !gemm_fits(ctx, "lora_grad_hidden", grad_output, B, hidden_tmp, seq_len, rank, out_dim) ||
+        !gemm_fits(ctx, "lora_gA", hidden_tmp, input, gA, rank, in_dim, seq_len))
+        return;
     gemm_op(ctx, "lora_recompute", input->data, A->data, hidden_tmp->data, seq_len, rank, in_dim, 0, 1, 0);
     cuda_train_scale(ctx, hidden_tmp, n, scale);
     gemm_op(ctx, "lora_gB", grad_output->data, hidden_tmp->data, gB->data, out_dim, rank, seq_len, 1, 0, 1);

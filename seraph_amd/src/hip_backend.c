@@ -27,6 +27,25 @@ int hip_backend_error_count(vulkan_context_t* ctx) {
     return st ? st->errors : -1;
 }
 
+int hip_backend_fits(vulkan_context_t* ctx, const char* op, int pairs, ...) {
+    va_list ap;
+    va_start(ap, pairs);
+    int ok = 1;
+    for (int i = 0; i < pairs; i++) {
+        const vulkan_buffer_t* buf = va_arg(ap, const vulkan_buffer_t*);
+        const size_t n = va_arg(ap, size_t);
+        if (!buf || n <= buf->size / 4) continue;              /* NULL: an optional operand the op goes without */
+        if (ok) {
+            hip_state_t* st = hip_state(ctx);
+            if (st && st->errors++ < 20)
+                fprintf(stderr, "ERROR: %s refused: operand %d has %zu bytes, the shape needs %zu\n", op, i, buf->size, n * 4);
+        }
+        ok = 0;
+    }
+    va_end(ap);
+    return ok;
+}
+
 void* hip_backend_scratch(vulkan_context_t* ctx, size_t bytes) {
     hip_state_t* st = hip_state(ctx);
     if (!st) return NULL;
@@ -328,6 +347,7 @@ void vulkan_nan_check(vulkan_context_t* ctx, vulkan_buffer_t* input, size_t coun
     hip_state_t* st = hip_state(ctx);
     if (!st || !input || !flags_u32 || count_floats == 0) return;
     if ((size_t)(flag_index + 1) * 4 > flags_u32->size) return;
+    if (!hip_backend_fits(ctx, "nan_check", 1, FIT(input, count_floats))) return;
     HIP_OP(ctx, "nan_check", seraph_nan_check(FPTR(input), count_floats, UPTR(flags_u32), flag_index, st->stream));
 }
 
@@ -345,7 +365,8 @@ static void backend_gemm(vulkan_context_t* ctx, hip_state_t* st, const char* wha
 void hip_matmul_scaled(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C,
                        int M, int N, int K, int transpose_A, int transpose_B, int accumulate, float alpha) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !A || !B || !C) return;
+    if (!st || !A || !B || !C || M < 0 || N < 0 || K < 0) return;
+    if (!hip_backend_fits(ctx, "matmul_scaled", 3, FIT(A, (size_t)M * K), FIT(B, (size_t)K * N), FIT(C, (size_t)M * N))) return;
     const size_t need = seraph_gemm_scaled_ws_bytes(M, N, K, transpose_A, transpose_B);
     void* ws = need ? hip_backend_scratch(ctx, need) : NULL;
     HIP_OPF(ctx, seraph_gemm_scaled(FPTR(A), FPTR(B), FPTR(C), M, N, K, transpose_A, transpose_B, accumulate, alpha,
@@ -354,51 +375,54 @@ void hip_matmul_scaled(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_
 
 void vulkan_matmul(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C, int M, int N, int K) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !A || !B || !C) return;
+    if (!st || !A || !B || !C || M < 0 || N < 0 || K < 0) return;
+    if (!hip_backend_fits(ctx, "matmul", 3, FIT(A, (size_t)M * K), FIT(B, (size_t)K * N), FIT(C, (size_t)M * N))) return;
     backend_gemm(ctx, st, "matmul", FPTR(A), FPTR(B), FPTR(C), M, N, K, 0, 0, 0);
 }
 
 void vulkan_matmul_transpose(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C,
                              int M, int N, int K, int transpose_A, int transpose_B, int accumulate) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !A || !B || !C) return;
+    if (!st || !A || !B || !C || M < 0 || N < 0 || K < 0) return;
+    if (!hip_backend_fits(ctx, "matmul_t", 3, FIT(A, (size_t)M * K), FIT(B, (size_t)K * N), FIT(C, (size_t)M * N))) return;
     backend_gemm(ctx, st, "matmul_t", FPTR(A), FPTR(B), FPTR(C), M, N, K, transpose_A, transpose_B, accumulate);
 }
 
 void vulkan_add(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C, size_t count) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !A || !B || !C) return;
+    if (!st || !A || !B || !C || !hip_backend_fits(ctx, "add", 3, FIT(A, count), FIT(B, count), FIT(C, count))) return;
     HIP_OP(ctx, "add", seraph_add(FPTR(A), FPTR(B), FPTR(C), count, st->stream));
 }
 
 void vulkan_mul(vulkan_context_t* ctx, vulkan_buffer_t* A, vulkan_buffer_t* B, vulkan_buffer_t* C, size_t count) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !A || !B || !C) return;
+    if (!st || !A || !B || !C || !hip_backend_fits(ctx, "mul", 3, FIT(A, count), FIT(B, count), FIT(C, count))) return;
     HIP_OP(ctx, "mul", seraph_mul(FPTR(A), FPTR(B), FPTR(C), count, st->stream));
 }
 
 void vulkan_scale(vulkan_context_t* ctx, vulkan_buffer_t* A, size_t count, float alpha) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !A) return;
+    if (!st || !A || !hip_backend_fits(ctx, "scale", 1, FIT(A, count))) return;
     HIP_OP(ctx, "scale", seraph_scale(FPTR(A), count, alpha, st->stream));
 }
 
 void vulkan_silu(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* output, size_t count) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !input || !output) return;
+    if (!st || !input || !output || !hip_backend_fits(ctx, "silu", 2, FIT(input, count), FIT(output, count))) return;
     HIP_OP(ctx, "silu", seraph_silu(FPTR(input), FPTR(output), count, st->stream));
 }
 
 void hip_swiglu(vulkan_context_t* ctx, vulkan_buffer_t* gate, vulkan_buffer_t* up, vulkan_buffer_t* out, size_t count) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !gate || !up || !out) return;
+    if (!st || !gate || !up || !out || !hip_backend_fits(ctx, "silu_mul", 3, FIT(gate, count), FIT(up, count), FIT(out, count))) return;
     HIP_OP(ctx, "silu_mul", seraph_swiglu(FPTR(gate), FPTR(up), FPTR(out), count, st->stream));
 }
 
 void vulkan_rmsnorm(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* scale, vulkan_buffer_t* output,
                     int rows, int cols, float eps) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !input || !scale || !output) return;
+    if (!st || !input || !scale || !output || rows < 0 || cols < 0) return;
+    if (!hip_backend_fits(ctx, "rmsnorm", 3, FIT(input, (size_t)rows * cols), FIT(scale, cols), FIT(output, (size_t)rows * cols))) return;
     HIP_OPF(ctx, seraph_rmsnorm(FPTR(input), FPTR(scale), FPTR(output), rows, cols, eps, st->stream), "rmsnorm [%dx%d] %u-thr", rows, cols, ctx->wg_size_1d);
 }
 
@@ -407,28 +431,36 @@ void vulkan_rmsnorm(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer
 void hip_add_rmsnorm(vulkan_context_t* ctx, vulkan_buffer_t* input, vulkan_buffer_t* addend, vulkan_buffer_t* sum,
                      vulkan_buffer_t* scale, vulkan_buffer_t* output, int rows, int cols, float eps) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !input || !addend || !sum || !scale || !output) return;
+    if (!st || !input || !addend || !sum || !scale || !output || rows < 0 || cols < 0) return;
+    const size_t rc = (size_t)rows * cols;
+    if (!hip_backend_fits(ctx, "add+rmsnorm", 5, FIT(input, rc), FIT(addend, rc), FIT(sum, rc), FIT(scale, cols), FIT(output, rc))) return;
     HIP_OPF(ctx, seraph_add_rmsnorm(FPTR(input), FPTR(addend), FPTR(sum), FPTR(scale), FPTR(output), rows, cols, eps, st->stream), "add+rmsnorm [%dx%d] %u-thr", rows, cols, ctx->wg_size_1d);
 }
 
 void vulkan_rope(vulkan_context_t* ctx, vulkan_buffer_t* x_in, vulkan_buffer_t* x_out,
                  int seq_len, int num_heads, int head_dim, float rope_theta) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !x_in || !x_out) return;
+    if (!st || !x_in || !x_out || seq_len < 0 || num_heads < 0 || head_dim < 0) return;
+    const size_t n = (size_t)seq_len * num_heads * head_dim;
+    if (!hip_backend_fits(ctx, "rope_fwd", 2, FIT(x_in, n), FIT(x_out, n))) return;
     HIP_OP(ctx, "rope_fwd", seraph_rope(FPTR(x_in), FPTR(x_out), NULL, 1, seq_len, num_heads, head_dim, rope_theta, 0, st->stream));
 }
 
 void hip_rope_packed(vulkan_context_t* ctx, vulkan_buffer_t* x_in, vulkan_buffer_t* x_out, vulkan_buffer_t* seq_starts,
                      int total_tokens, int batch_size, int num_heads, int head_dim, float rope_theta) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !x_in || !x_out || !seq_starts) return;
+    if (!st || !x_in || !x_out || !seq_starts || total_tokens < 0 || batch_size < 0 || num_heads < 0 || head_dim < 0) return;
+    const size_t n = (size_t)total_tokens * num_heads * head_dim;
+    if (!hip_backend_fits(ctx, "rope_fwd_packed", 3, FIT(x_in, n), FIT(x_out, n), FIT(seq_starts, (size_t)batch_size + 1))) return;
     HIP_OP(ctx, "rope_fwd_packed", seraph_rope(FPTR(x_in), FPTR(x_out), UPTR(seq_starts), batch_size, total_tokens, num_heads, head_dim, rope_theta, 0, st->stream));
 }
 
 void vulkan_batch_attention(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulkan_buffer_t* K, vulkan_buffer_t* V,
                             vulkan_buffer_t* out, int seq_len, int num_heads, int kv_heads, int head_dim) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !Q || !K || !V || !out) return;
+    if (!st || !Q || !K || !V || !out || seq_len < 0 || num_heads < 0 || kv_heads < 0 || head_dim < 0) return;
+    const size_t nq = (size_t)seq_len * num_heads * head_dim, nkv = (size_t)seq_len * kv_heads * head_dim;
+    if (!hip_backend_fits(ctx, "attn_fwd", 4, FIT(Q, nq), FIT(K, nkv), FIT(V, nkv), FIT(out, nq))) return;
     float scale = 1.0f / sqrtf((float)head_dim);          /* src/vulkan_backend.c:2980-2984 */
     HIP_OPF(ctx, seraph_attention_forward(FPTR(Q), FPTR(K), FPTR(V), FPTR(out), NULL, NULL, 1, seq_len,
                                                             num_heads, kv_heads, head_dim, scale, st->stream), "attn_fwd [seq=%d h=%d hd=%d]", seq_len, num_heads, head_dim);
@@ -438,7 +470,10 @@ void hip_batch_attention_packed(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulka
                                 vulkan_buffer_t* out, vulkan_buffer_t* lse_out, vulkan_buffer_t* seq_starts,
                                 int total_tokens, int batch_size, int num_heads, int kv_heads, int head_dim) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !Q || !K || !V || !out || !seq_starts) return;
+    if (!st || !Q || !K || !V || !out || !seq_starts || total_tokens < 0 || batch_size < 0 || num_heads < 0 || kv_heads < 0 || head_dim < 0) return;
+    const size_t nq = (size_t)total_tokens * num_heads * head_dim, nkv = (size_t)total_tokens * kv_heads * head_dim;
+    if (!hip_backend_fits(ctx, "attn_fwd_packed", 6, FIT(Q, nq), FIT(K, nkv), FIT(V, nkv), FIT(out, nq),
+                          FIT(lse_out, (size_t)total_tokens * num_heads), FIT(seq_starts, (size_t)batch_size + 1))) return;
     float scale = 1.0f / sqrtf((float)head_dim);
     HIP_OPF(ctx, seraph_attention_forward(FPTR(Q), FPTR(K), FPTR(V), FPTR(out), lse_out ? FPTR(lse_out) : NULL,
                                                                    UPTR(seq_starts), batch_size, total_tokens,
@@ -448,13 +483,16 @@ void hip_batch_attention_packed(vulkan_context_t* ctx, vulkan_buffer_t* Q, vulka
 void vulkan_embed_lookup(vulkan_context_t* ctx, vulkan_buffer_t* tokens_u32, vulkan_buffer_t* embed_weight,
                          vulkan_buffer_t* out_hidden, int seq_len, int hidden_size, int vocab_size) {
     hip_state_t* st = hip_state(ctx);
-    if (!st || !tokens_u32 || !embed_weight || !out_hidden) return;
+    if (!st || !tokens_u32 || !embed_weight || !out_hidden || seq_len < 0 || hidden_size < 0 || vocab_size < 0) return;
+    if (!hip_backend_fits(ctx, "embed_lookup", 3, FIT(tokens_u32, seq_len), FIT(embed_weight, (size_t)vocab_size * hidden_size),
+                          FIT(out_hidden, (size_t)seq_len * hidden_size))) return;
     HIP_OP(ctx, "embed_lookup", seraph_embed_lookup(UPTR(tokens_u32), FPTR(embed_weight), FPTR(out_hidden), seq_len, hidden_size, vocab_size, st->stream));
 }
 
 void vulkan_qk_norm(vulkan_context_t* ctx, vulkan_buffer_t* qk, int seq_len, int num_heads, int head_dim, int use_qk_norm, float eps) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !qk || !use_qk_norm) return;               /* src/vulkan_backend.c:3481 */
+    if (seq_len < 0 || num_heads < 0 || head_dim < 0 || !hip_backend_fits(ctx, "qk_norm", 1, FIT(qk, (size_t)seq_len * num_heads * head_dim))) return;
     HIP_OP(ctx, "qk_norm", seraph_qk_norm(FPTR(qk), seq_len, num_heads, head_dim, use_qk_norm, eps, st->stream));
 }
 
@@ -464,6 +502,7 @@ void hip_adamw_update_clipped(vulkan_context_t* ctx, vulkan_buffer_t* weight, vu
                               int step, size_t size, float clip) {
     hip_state_t* st = hip_state(ctx);
     if (!st || !weight || !grad || !m || !v || size == 0) return;
+    if (!hip_backend_fits(ctx, "adamw", 4, FIT(weight, size), FIT(grad, size), FIT(m, size), FIT(v, size))) return;
     HIP_OPF(ctx, seraph_adamw(FPTR(weight), FPTR(grad), FPTR(m), FPTR(v), size, lr, beta1, beta2, weight_decay, eps, step, clip, st->stream), "adamw [%zu] %u-thr", (size_t)size, ctx->wg_size_1d);
 }
 
@@ -477,6 +516,7 @@ void hip_adamw_update_multi(vulkan_context_t* ctx, int count, vulkan_buffer_t* c
     int k = 0;
     for (int i = 0; i < count; i++) {
         if (!weights[i] || !grads[i] || !m[i] || !v[i] || sizes[i] == 0) continue;      /* as vulkan_adamw_update: silently */
+        if (!hip_backend_fits(ctx, "adamw", 4, FIT(weights[i], sizes[i]), FIT(grads[i], sizes[i]), FIT(m[i], sizes[i]), FIT(v[i], sizes[i]))) continue;
         list[k].w = FPTR(weights[i]); list[k].g = FPTR(grads[i]); list[k].m = FPTR(m[i]); list[k].v = FPTR(v[i]);
         list[k].n = sizes[i];
         k++;

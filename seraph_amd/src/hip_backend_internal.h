@@ -35,6 +35,12 @@ void hip_backend_report(vulkan_context_t* ctx, const char* op, int rc);
 void hip_prof_begin(vulkan_context_t* ctx, const char* name);
 void hip_prof_end(vulkan_context_t* ctx);
 
+/* 1 when each of the `pairs` (buffer, number of 4-byte values) arguments that follow fits its buffer.  Otherwise the op
+ * is reported as refused and counted as an error, and the caller returns without launching anything: a shape that
+ * reaches past the end of a buffer is a memory fault on this device, which can take more than the process with it. */
+int hip_backend_fits(vulkan_context_t* ctx, const char* op, int pairs, ...);
+#define FIT(buf, n) (const vulkan_buffer_t*)(buf), (size_t)(n)
+
 /* Runs one kernel-library call for op `name`: timing when profiling, error report when it fails. */
 #define HIP_OP(ctx, name, call)                       \
     do {                                              \

@@ -297,3 +297,57 @@ def test_adamw_update_multi_equals_per_tensor_updates(vk, orc):
         for b in bufs:
             if b is not None:
                 lib.vulkan_buffer_free(ctx, b)
+
+
+def test_shapes_that_do_not_fit_their_buffers_are_refused():
+    """An op whose shape reaches past the end of one of its buffers is not launched: the op reports an error, counts it
+    and leaves every buffer as it was.  (Elsewhere such a call reads garbage; on this device it would be a memory fault.)
+    A context of its own, because the error count is the context's."""
+    from seraph_amd._lib import backend
+    lib = backend()
+    lib.vulkan_init_ex.restype = C.c_void_p
+    lib.vulkan_buffer_create.restype = C.POINTER(Buf)
+    lib.vulkan_buffer_create.argtypes = [C.c_void_p, C.c_size_t]
+    ctx = C.c_void_p(lib.vulkan_init_ex(0, -1))
+    me = (lib, ctx)
+    r = rng(90)
+    T, h, w = 24, 32, 48
+    a = r.standard_normal((T, h)).astype(np.float32)
+    b = r.standard_normal((h, w)).astype(np.float32)
+    stale = np.full((T, h), 3.0, np.float32)                     # T x h where the product needs T x w
+    A, B, Csmall, tok = up(me, a), up(me, b), up(me, stale), up(me, np.arange(T, dtype=np.uint32))
+    errors = 0
+    calls = [
+        lambda: lib.vulkan_matmul(ctx, A, B, Csmall, T, w, h),
+        lambda: lib.vulkan_matmul_transpose(ctx, A, B, Csmall, T, w, h, 0, 0, 1),
+        lambda: lib.vulkan_add(ctx, A, A, Csmall, C.c_size_t(T * h + 1)),
+        lambda: lib.vulkan_scale(ctx, Csmall, C.c_size_t(T * w), C.c_float(2.0)),
+        lambda: lib.vulkan_silu(ctx, A, Csmall, C.c_size_t(T * w)),
+        lambda: lib.vulkan_rmsnorm(ctx, A, B, Csmall, T, w, C.c_float(1e-5)),
+        lambda: lib.vulkan_rope(ctx, Csmall, Csmall, T, 2, 32, C.c_float(10000.0)),
+        lambda: lib.vulkan_batch_attention(ctx, A, A, A, Csmall, T, 2, 2, 32),
+        lambda: lib.vulkan_embed_lookup(ctx, tok, B, Csmall, T, w, h),
+        lambda: lib.vulkan_cross_entropy_grad(ctx, A, tok, Csmall, Csmall, T, w, T),
+        lambda: lib.vulkan_rmsnorm_backward_batch(ctx, A, B, A, Csmall, B, T, w, C.c_float(1e-5)),
+        lambda: lib.vulkan_batch_attention_backward(ctx, A, A, A, A, Csmall, Csmall, Csmall, T, 2, 2, 32),
+        lambda: lib.vulkan_embedding_backward(ctx, tok, A, Csmall, T, h, w),
+        lambda: lib.vulkan_silu_backward(ctx, A, A, Csmall, C.c_size_t(T * w)),
+        lambda: lib.vulkan_adamw_update(ctx, Csmall, A, A, A, C.c_float(1e-3), C.c_float(0.9), C.c_float(0.999), C.c_float(0.01),
+                                        C.c_float(1e-8), 1, C.c_size_t(T * w)),
+    ]
+    lib.vulkan_cmd_begin(ctx)
+    for i, call in enumerate(calls):
+        call()
+        errors += 1
+        assert lib.hip_backend_error_count(ctx) == errors, i
+    assert lib.vulkan_cmd_end_submit(ctx) == 1
+    assert (down(me, Csmall, (T, h)) == stale).all() and (down(me, A, (T, h)) == a).all()
+    # the same ops with shapes that fit still run
+    lib.vulkan_cmd_begin(ctx)
+    lib.vulkan_matmul(ctx, A, B, Csmall, T, h // 2, h)            # T x 16 of B's first rows: inside every buffer
+    lib.vulkan_cmd_end_submit(ctx)
+    assert lib.hip_backend_error_count(ctx) == errors
+    assert not (down(me, Csmall, (T, h)) == stale).all()
+    for buf in (A, B, Csmall, tok):
+        lib.vulkan_buffer_free(ctx, buf)
+    lib.vulkan_free(ctx)

@@ -408,6 +408,12 @@ def test_reference_batched_trainer_profile_and_lora(tmp_path, orc, binary):
     assert len(got) == len(batches) and abs(got[0] - base_loss) < 1.5e-4
     assert all(np.isfinite(got))
     assert os.path.exists(tmp_path / "q" / "checkpoint_final.bin")
+    # The reference's batched LoRA backward gives every adapter the final hidden gradient as its output gradient
+    # (src/train_cuda.c:2596-2644).  For the query adapter of this shape (q_dim 128, hidden 64) that product would read
+    # past the end of the buffer: the backend refuses it with a message and leaves the adapter alone; the value adapter
+    # (kv_dim 64) fits and runs.
+    assert "lora_gB [128x4" in err and "skipped: operand 0" in err, err[-1500:]
+    assert "lora_gB [64x4" not in err
 
 
 def test_nan_detection_writes_the_dump_files_the_reference_inspector_reads(tr, orc, tmp_path):

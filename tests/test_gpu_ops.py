@@ -278,7 +278,8 @@ def test_gemm_scaled_grouped_equals_the_single_calls(ops, orc, tA, tB, shapes, a
 @pytest.mark.parametrize("M,N,Ks", [(2048, 512, (1408, 1408)), (2048, 512, (512, 512, 512)), (1024, 2048, (2048, 1024, 1024)),
                                     (4100, 2048, (512, 256)),            # 128x128 tiles with a ragged edge
                                     (300, 260, (64, 32, 96)),            # edge tiles in both directions
-                                    (96, 64, (2048, 1024)),              # too few tiles: runs as single products
+                                    (96, 64, (2048, 1024)),              # few tiles, long K: 32x32 tiles whose waves share out K
+                                    (40, 36, (96, 64, 128)),             # the same with ragged 32x32 tiles
                                     (130, 70, (36, 64)),                 # a K that is not whole stages: single products
                                     (512, 512, (128,))])
 def test_gemm_chain(ops, orc, tA, tB, M, N, Ks):
@@ -297,9 +298,11 @@ def test_gemm_chain(ops, orc, tA, tB, M, N, Ks):
     out = ops.gemm_chain(terms, M, N, tA, tB, out=dev(C0), accumulate=True)
     parity(out, (ref + C0).astype(np.float32), f"gemm chain {M}x{N}x{Ks}, accumulate", atol=1e-4)
     name = ops.gemm_chain_kernel_name(terms, out, M, N, tA, tB)
-    few_tiles = ((M + 63) // 64) * ((N + 63) // 64) < 256             # with a long K such an output is cut along K instead
-    one_launch = len(Ks) > 1 and all(K % 32 == 0 for K in Ks) and not (few_tiles and sum(Ks) >= 256)
+    one_launch = len(Ks) > 1 and all(K % 32 == 0 for K in Ks)
     assert ("chain_kernel" in name) == one_launch, name
+    t64 = ((M + 63) // 64) * ((N + 63) // 64)                         # few 64x64 tiles and a long K: the waves share out K
+    if one_launch and t64 < 256 and sum(Ks) >= 256:
+        assert "splitk_chain_kernel" in name, name
 
 
 # ------------------------------------------------------------------ rmsnorm
