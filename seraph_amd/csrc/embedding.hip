@@ -183,17 +183,10 @@ __device__ __forceinline__ void emb_sum_slabs(const uint32_t* __restrict__ token
 
 // VPL float4 per lane make the first pass over a row; EXACT: the row holds at least that many and the pass needs no
 // test against its end (the tests cost 8 us of 66 at 16384 x 2048: the loads of a pass no longer issue back to back).
-typedef float emb_f4v __attribute__((ext_vector_type(4)));
-template <bool STREAM> __device__ __forceinline__ float4 emb_ld(const float4* p) {
-    if (STREAM) { const emb_f4v v = __builtin_nontemporal_load(reinterpret_cast<const emb_f4v*>(p)); return make_float4(v.x, v.y, v.z, v.w); }
-    return *p;
-}
-template <bool STREAM> __device__ __forceinline__ void emb_st(float4* p, float4 v) {
-    if (STREAM) { const emb_f4v r = {v.x, v.y, v.z, v.w}; __builtin_nontemporal_store(r, reinterpret_cast<emb_f4v*>(p)); }
-    else *p = v;
-}
-
-template <int VPL, bool EXACT, bool STREAM>
+// Streamed (nontemporal) accesses for the row read-modify-write were measured and are not used: with table rows that no
+// earlier call left in the last-level cache they change nothing (87.5 against 87.2 us at 16384 x 2048 into 151936 rows),
+// with rows that are still there they lose them (87.1 against 69.6 us).
+template <int VPL, bool EXACT>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8)))
 void emb_sum_kernel(const uint32_t* __restrict__ tokens, EmbEntry* tab, const uint32_t* __restrict__ link,
                     const float* __restrict__ dH, float* __restrict__ grad_embed,
@@ -208,7 +201,7 @@ void emb_sum_kernel(const uint32_t* __restrict__ tokens, EmbEntry* tab, const ui
 #pragma unroll
         for (int k = 0; k < VPL; k++) {
             const int64_t i = lane + 64 * k;
-            own[k] = (EXACT || i < n4) ? emb_ld<STREAM>(reinterpret_cast<const float4*>(dH + p * hidden) + i) : make_float4(0, 0, 0, 0);
+            own[k] = (EXACT || i < n4) ? reinterpret_cast<const float4*>(dH + p * hidden)[i] : make_float4(0, 0, 0, 0);
         }
     }
     const uint32_t tok = tokens[p];
@@ -230,7 +223,7 @@ void emb_sum_kernel(const uint32_t* __restrict__ tokens, EmbEntry* tab, const ui
 #pragma unroll
         for (int k = 0; k < VPL; k++) {
             const int64_t i = lane + 64 * k;
-            old[k] = (EXACT || i < n4) ? emb_ld<STREAM>(reinterpret_cast<const float4*>(row) + i) : make_float4(0, 0, 0, 0);
+            old[k] = (EXACT || i < n4) ? reinterpret_cast<const float4*>(row)[i] : make_float4(0, 0, 0, 0);
         }
     }
     const uint32_t count = emb_value(tab[tok].count, epoch, 0u);
@@ -244,7 +237,7 @@ void emb_sum_kernel(const uint32_t* __restrict__ tokens, EmbEntry* tab, const ui
 #pragma unroll
         for (int k = 0; k < VPL; k++) {
             const int64_t i = lane + 64 * k;
-            if (EXACT || i < n4) emb_st<STREAM>(reinterpret_cast<float4*>(row) + i, make_float4(old[k].x + own[k].x, old[k].y + own[k].y, old[k].z + own[k].z, old[k].w + own[k].w));
+            if (EXACT || i < n4) reinterpret_cast<float4*>(row)[i] = make_float4(old[k].x + own[k].x, old[k].y + own[k].y, old[k].z + own[k].z, old[k].w + own[k].w);
         }
         for (int64_t i0 = 64 * VPL; i0 < n4; i0 += 64) {       // what the first pass left of the row
             const int64_t i = i0 + lane;
@@ -326,11 +319,6 @@ void emb_sum_kernel(const uint32_t* __restrict__ tokens, EmbEntry* tab, const ui
     }
 }
 
-// Streamed (nontemporal) accesses for the row read-modify-write were measured and are off: with table rows that no
-// earlier call left in the last-level cache they change nothing (87.5 against 87.2 us at 16384 x 2048 into 151936 rows),
-// with rows that are still there they lose them (87.1 against 69.6 us).
-static int g_emb_streamed = 0;
-
 // device address of the library's tables on the current device
 static int emb_tables(EmbEntry** out, int* device) {
     static std::mutex mu;
@@ -361,8 +349,6 @@ int seraph_embed_lookup(const uint32_t* tokens, const float* embed, float* out,
     SERAPH_LAUNCH_CHECK();
     return SERAPH_OK;
 }
-
-void seraph_embedding_backward_streamed(int on) { g_emb_streamed = on ? 1 : 0; }
 
 size_t seraph_embedding_backward_ws_bytes(int64_t T, int64_t vocab) {
     if (T <= 0 || vocab <= 0) return 0;
@@ -413,9 +399,8 @@ int seraph_embedding_backward(const uint32_t* tokens, const float* dH, float* gr
     int vec = (hidden % 4 == 0) && aligned16(dH) && aligned16(grad_embed);
     // first pass over a row: as many float4 per lane as fit it exactly, up to 8 (2048 floats)
     const int64_t whole = vec && hidden % 256 == 0 ? hidden / 256 : 0;
-#define SUM(VPL, EXACT) do { \
-        if (g_emb_streamed) hipLaunchKernelGGL((emb_sum_kernel<VPL, EXACT, true>), dim3((unsigned)T), dim3(64), 0, st, tokens, tab, w.link, dH, grad_embed, T, hidden, vocab, epoch, vec); \
-        else hipLaunchKernelGGL((emb_sum_kernel<VPL, EXACT, false>), dim3((unsigned)T), dim3(64), 0, st, tokens, tab, w.link, dH, grad_embed, T, hidden, vocab, epoch, vec); } while (0)
+#define SUM(VPL, EXACT) \
+    hipLaunchKernelGGL((emb_sum_kernel<VPL, EXACT>), dim3((unsigned)T), dim3(64), 0, st, tokens, tab, w.link, dH, grad_embed, T, hidden, vocab, epoch, vec)
     if (whole >= 8) SUM(8, true);
     else if (whole >= 4) SUM(4, true);
     else if (whole >= 2) SUM(2, true);

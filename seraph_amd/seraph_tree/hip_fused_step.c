@@ -164,6 +164,12 @@ static hip_trainer_t* fused_trainer(train_state_t* state, cuda_train_context_t* 
     return t;
 }
 
+/* An op-by-op step updates the per-tensor buffers, so from then on the fused step's arenas would be stale - unless the
+ * step belongs to another model than the one the fused trainer serves, whose arenas it does not touch. */
+static void took_opbyop_step(const train_state_t* state) {
+    if (!g.t || g.state == state) g.opbyop = 1;
+}
+
 /* hip_cuda_backend.c calls this from cuda_train_free when it is linked in */
 void hip_fused_step_release(cuda_train_context_t* ctx) {
     if (g.t && g.ctx == ctx) { hip_trainer_free(g.t); memset(&g, 0, sizeof(g)); }
@@ -174,7 +180,7 @@ float cuda_train_step_gpu_full_batch(train_state_t* state, int* tokens_packed, i
     if (!state || !state->full_weights || !state->config || !ctx) return -1.0f;      /* src/train_cuda.c:1970 */
     hip_trainer_t* t = fused_trainer(state, ctx, total_tokens, batch_size);
     if (!t) {
-        g.opbyop = 1;
+        took_opbyop_step(state);
         return cuda_train_step_gpu_full_batch_opbyop(state, tokens_packed, total_tokens, seq_starts, batch_size, ctx);
     }
     const double t0 = now_ms();
@@ -216,7 +222,7 @@ float cuda_train_step_gpu_full_batch(train_state_t* state, int* tokens_packed, i
 float cuda_train_step_gpu_full(train_state_t* state, int* tokens, int num_tokens, cuda_train_context_t* ctx) {
     if (!state || !state->full_weights || !state->config || !ctx) return -1.0f;
     if (!fused_trainer(state, ctx, num_tokens, 1)) {
-        g.opbyop = 1;
+        took_opbyop_step(state);
         return cuda_train_step_gpu_full_opbyop(state, tokens, num_tokens, ctx);
     }
     int starts[2] = {0, num_tokens};
