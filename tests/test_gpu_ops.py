@@ -481,6 +481,23 @@ def test_embedding_backward_float_and_odd_hidden(ops, orc):
     assert (a == b).all()
 
 
+def test_embedding_backward_vocabulary_larger_than_the_library_tables(ops, orc):
+    """Vocabularies of more than 2^18 tokens do not fit the token tables that the library keeps: the table is then part of
+    the caller's scratch and is cleared by a launch of its own in every call.  Twice with different tokens through the same
+    scratch pattern, with repeated tokens on both sides of 2^18 and ids past the vocabulary; bit-exact (integer values)."""
+    r = rng(19)
+    T, V, h = 3000, 300000, 8
+    base = r.integers(-3, 4, (V, h)).astype(np.float32)
+    for seed in (1, 2):
+        tok = rng(seed).integers(0, V + 1000, T).astype(np.uint32)
+        tok[:40] = 5
+        tok[40:80] = 262144 + 17
+        tok[80:100] = V - 1
+        dH = rng(seed + 10).integers(-8, 9, (T, h)).astype(np.float32)
+        got = host(ops.embedding_backward(dev(tok.view(np.int32)), dev(dH), dev(base)))
+        assert (got == orc.embedding_backward(tok, dH, base)).all()
+
+
 # ------------------------------------------------------------------ AdamW
 @pytest.mark.parametrize("n", [1, 1000, 100003])
 @pytest.mark.parametrize("clip", [0.0, 1.0])
@@ -744,7 +761,7 @@ def test_cross_entropy_long_rows_are_deterministic_and_alias_safe(ops, rows, col
     assert float(g_ref[~live].abs().max()) == 0 if (~live).any() else True
 
 
-@pytest.mark.parametrize("h", [256, 520, 2048])
+@pytest.mark.parametrize("h", [256, 520, 1024, 2048, 4096])
 @pytest.mark.parametrize("case", ["one token", "few tokens", "pairs", "mixed"])
 def test_embedding_backward_repeated_tokens(ops, orc, case, h):
     """Groups of every size: a batch that is one token repeated (a padding-dominated batch), a handful of tokens, every
@@ -776,7 +793,9 @@ def test_embedding_backward_repeated_tokens(ops, orc, case, h):
     a = ops.embedding_backward(dev(tok.view(np.int32)), dev(dF), dev(base))
     b = ops.embedding_backward(dev(tok.view(np.int32)), dev(dF), dev(base))
     assert torch.equal(a, b)
-    parity(a, orc.embedding_backward(tok, dF, base), "embedding backward", atol=1e-4)
+    # a row that collects up to 5000 N(0,1) terms has partial sums of about 70, whose float spacing is 8e-6: two orders of
+    # addition differ by some 1e-4 in absolute terms wherever the total happens to land near zero
+    parity(a, orc.embedding_backward(tok, dF, base), "embedding backward", atol=1e-3)
 
 
 def test_embedding_backward_more_column_slabs_than_positions(ops, orc):
