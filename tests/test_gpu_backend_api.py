@@ -351,3 +351,113 @@ def test_shapes_that_do_not_fit_their_buffers_are_refused():
     for buf in (A, B, Csmall, tok):
         lib.vulkan_buffer_free(ctx, buf)
     lib.vulkan_free(ctx)
+
+
+def test_packed_and_fused_additions_through_the_backend(vk, orc):
+    """The entry points the backend adds for packed batches and fused ops (arguments of include/cuda_train_context.h:273-288),
+    and the single-op forms the reference's step does not reach in the slices above, each against the oracle: one layer's
+    worth of a packed batch, forward and backward, in issue order between cmd_begin and cmd_end_submit."""
+    lib, ctx = vk
+    r = rng(31)
+    f = C.c_float
+    starts = np.array([0, 40, 41, 100], np.uint32)
+    T, batch, H, KVH, D, V, ffn = 100, 3, 4, 2, 32, 211, 96
+    hdim, qd, kvd = 64, H * D, KVH * D
+    theta, eps = 10000.0, 1e-6
+    tok = r.integers(0, V, T).astype(np.uint32)
+    E = r.standard_normal((V, hdim)).astype(np.float32)
+    q, k, v = (0.5 * r.standard_normal((T, w)).astype(np.float32) for w in (qd, kvd, kvd))
+    d_out = (0.1 * r.standard_normal((T, qd))).astype(np.float32)
+    logits = (2 * r.standard_normal((T, V))).astype(np.float32)
+    gate, upv, d_h = (r.standard_normal((T, ffn)).astype(np.float32) for _ in range(3))
+    dk0, dv0 = (r.standard_normal((T, kvd)).astype(np.float32) for _ in range(2))
+    ge0 = r.standard_normal((V, hdim)).astype(np.float32)
+    d_hidden = r.standard_normal((T, hdim)).astype(np.float32)
+
+    B = {n: up(vk, a) for n, a in dict(tok=tok, E=E, q=q, k=k, v=v, d_out=d_out, logits=logits, gate=gate, up=upv, d_h=d_h,
+                                       starts=starts, dk=dk0, dv=dv0, dk2=dk0, dv2=dv0, ge=ge0, d_hidden=d_hidden).items()}
+    for n, shape in dict(hid=(T, hdim), qn=(T, qd), qr=(T, qd), kr=(T, kvd), att=(T, qd), lse=(T, H), dq=(T, qd), dq2=(T, qd),
+                         dqr=(T, qd), dqn=(T, qd), gl=(T, V), loss=(T,), act=(T, ffn), sil=(T, ffn), g_gate=(T, ffn), g_up=(T, ffn),
+                         g_sil=(T, ffn), g_a=(T, ffn), g_b=(T, ffn), copy=(T, qd), att1=(T, qd)).items():
+        B[n] = up(vk, np.full(shape, 7.0, np.float32))
+    B["flags"] = up(vk, np.zeros(4, np.uint32))
+    n_valid = T - batch
+
+    assert lib.vulkan_cmd_begin(ctx) == 1
+    lib.vulkan_embed_lookup(ctx, B["tok"], B["E"], B["hid"], T, hdim, V)
+    lib.vulkan_copy_buffer(ctx, B["q"], B["qn"], C.c_size_t(T * qd * 4))
+    lib.vulkan_qk_norm(ctx, B["qn"], T, H, D, 1, f(eps))
+    lib.hip_rope_packed(ctx, B["qn"], B["qr"], B["starts"], T, batch, H, D, f(theta))
+    lib.hip_rope_packed(ctx, B["k"], B["kr"], B["starts"], T, batch, KVH, D, f(theta))
+    lib.hip_batch_attention_packed(ctx, B["qr"], B["kr"], B["v"], B["att"], B["lse"], B["starts"], T, batch, H, KVH, D)
+    lib.vulkan_copy_buffer_cache(ctx, B["att"], B["copy"], C.c_size_t(T * qd * 4))
+    lib.hip_cross_entropy_grad_packed(ctx, B["logits"], B["tok"], B["gl"], B["loss"], B["starts"], T, batch, V, n_valid)
+    lib.hip_batch_attention_backward_packed(ctx, B["qr"], B["kr"], B["v"], B["att"], B["lse"], B["d_out"], B["dq"], B["dk"], B["dv"],
+                                            B["starts"], T, batch, H, KVH, D)
+    lib.hip_batch_attention_backward_packed(ctx, B["qr"], B["kr"], B["v"], None, None, B["d_out"], B["dq2"], B["dk2"], B["dv2"],
+                                            B["starts"], T, batch, H, KVH, D)             # nothing saved: recomputed
+    lib.hip_rope_backward_packed(ctx, B["dq"], B["dqr"], B["starts"], T, batch, H, D, f(theta))
+    lib.hip_qk_norm_backward(ctx, B["q"], B["dqr"], B["dqn"], T, H, D, f(eps))
+    lib.hip_swiglu(ctx, B["gate"], B["up"], B["act"], C.c_size_t(T * ffn))
+    lib.hip_swiglu_backward(ctx, B["gate"], B["up"], B["d_h"], B["g_gate"], B["g_up"], C.c_size_t(T * ffn))
+    lib.vulkan_silu(ctx, B["gate"], B["sil"], C.c_size_t(T * ffn))                        # the reference's two ops for the same
+    lib.vulkan_mul(ctx, B["sil"], B["up"], B["sil"], C.c_size_t(T * ffn))
+    lib.vulkan_elementwise_mul_backward(ctx, B["gate"], B["up"], B["d_h"], B["g_a"], B["g_b"], C.c_size_t(T * ffn))
+    lib.vulkan_silu_backward(ctx, B["gate"], B["d_h"], B["g_sil"], C.c_size_t(T * ffn))
+    lib.vulkan_embedding_backward(ctx, B["tok"], B["d_hidden"], B["ge"], T, hdim, V)
+    lib.vulkan_nan_check(ctx, B["att"], C.c_size_t(T * qd), B["flags"], 2)
+    lib.vulkan_barrier_transfer_to_compute(ctx)
+    assert lib.vulkan_cmd_end_submit(ctx) == 1
+    # one sequence through the unpacked forms (outside a recording: synchronous)
+    lib.vulkan_rope(ctx, B["q"], B["dq2"], T, H, D, f(theta))
+    lib.vulkan_batch_attention(ctx, B["q"], B["k"], B["v"], B["att1"], T, H, KVH, D)
+    assert lib.hip_backend_error_count(ctx) == 0
+
+    assert (down(vk, B["hid"], (T, hdim)) == orc.embed_lookup(tok, E)).all()
+    qn = orc.qk_norm(q, H, D, eps)
+    close(down(vk, B["qn"], (T, qd)), qn)
+    qr, kr = orc.rope(qn, H, D, theta, starts), orc.rope(k, KVH, D, theta, starts)
+    close(down(vk, B["qr"], (T, qd)), qr); close(down(vk, B["kr"], (T, kvd)), kr)
+    att, lse = orc.attention_forward(qr, kr, v, H, KVH, D, starts)
+    close(down(vk, B["att"], (T, qd)), att); close(down(vk, B["lse"], (T, H)), lse)
+    assert (down(vk, B["copy"], (T, qd)) == down(vk, B["att"], (T, qd))).all()
+    gl, loss = orc.cross_entropy_grad_packed(logits, tok, starts, n_valid)
+    close(down(vk, B["gl"], (T, V)), gl, atol=1e-7); close(down(vk, B["loss"], (T,)), loss)
+    dq, dk, dv = orc.attention_backward(qr, kr, v, d_out, H, KVH, D, starts, dK0=dk0, dV0=dv0)
+    for a, b, ref, shape in (("dq", "dq2", dq, (T, qd)), ("dk", "dk2", dk, (T, kvd)), ("dv", "dv2", dv, (T, kvd))):
+        if a != "dq":
+            close(down(vk, B[b], shape), ref)                      # dq2 was reused by vulkan_rope below
+        close(down(vk, B[a], shape), ref)
+    dqr = orc.rope(dq, H, D, theta, starts, backward=True)
+    close(down(vk, B["dqr"], (T, qd)), dqr)
+    close(down(vk, B["dqn"], (T, qd)), orc.qk_norm_backward(q, dqr, H, D, eps), atol=2e-5)
+    act = orc.silu(gate) * upv
+    close(down(vk, B["act"], (T, ffn)), act); close(down(vk, B["sil"], (T, ffn)), act)
+    gg, gu = orc.swiglu_backward(gate, upv, d_h)
+    close(down(vk, B["g_gate"], (T, ffn)), gg); close(down(vk, B["g_up"], (T, ffn)), gu)
+    ga, gb = orc.mul_backward(gate, upv, d_h)
+    assert (down(vk, B["g_a"], (T, ffn)) == ga).all() and (down(vk, B["g_b"], (T, ffn)) == gb).all()
+    close(down(vk, B["g_sil"], (T, ffn)), orc.silu_backward(gate, d_h))
+    close(down(vk, B["ge"], (V, hdim)), orc.embedding_backward(tok, d_hidden, ge0))
+    assert (down(vk, B["flags"], 4, np.uint32) == 0).all()
+    close(down(vk, B["dq2"], (T, qd)), orc.rope(q, H, D, theta))
+    close(down(vk, B["att1"], (T, qd)), orc.attention_forward(q, k, v, H, KVH, D)[0])
+    for b in B.values():
+        lib.vulkan_buffer_free(ctx, b)
+
+
+def test_video_mode_ops_report_that_they_are_not_provided():
+    """The four video-only symbols exist so that train.o links (include/vulkan_backend.h:600-642); calling one is an error
+    that is reported and counted, nothing more.  A context of its own (vulkan_init, the pool-size form), because the error
+    count is the context's."""
+    from seraph_amd._lib import backend
+    lib = backend()
+    lib.vulkan_init.restype = C.c_void_p
+    ctx = C.c_void_p(lib.vulkan_init(0))
+    assert ctx
+    lib.vulkan_patch_extract(ctx, None, None, 1, 1, 1, 1, 1, 1)
+    lib.vulkan_add_bias(ctx, None, None, 1, 1)
+    lib.vulkan_bce_loss_grad(ctx, None, None, None, None, C.c_size_t(1))
+    lib.vulkan_sum_cols(ctx, None, None, 1, 1)
+    assert lib.hip_backend_error_count(ctx) == 4
+    lib.vulkan_free(ctx)

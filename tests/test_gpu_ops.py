@@ -102,7 +102,8 @@ def test_fill_nan_reduce(ops, orc):
 
 
 # ------------------------------------------------------------------ cross entropy
-@pytest.mark.parametrize("rows,cols", [(9, 8192), (5, 1000), (4, 40000), (3, 33001), (2, 151936), (6, 4), (1030, 32772), (3, 1300000)])
+@pytest.mark.parametrize("rows,cols", [(9, 8192), (5, 1000), (4, 40000), (3, 33001), (2, 151936), (6, 4), (1030, 32772), (3, 1300000),
+                                       (7, 12000), (5, 30000), (3, 32768)])    # 16 and 32 float4 per lane in one workgroup's registers
 def test_cross_entropy_grad(ops, orc, rows, cols):
     r = rng(rows * 100003 + cols)
     x = (2 * r.standard_normal((rows, cols))).astype(np.float32)
@@ -157,7 +158,7 @@ def test_gemm_forms(ops, orc, tA, tB, M, N, K):
 
 @pytest.mark.parametrize("tA,tB,M,N,K", [(0, 1, 2048, 16, 2048), (0, 0, 2048, 16, 1024), (1, 0, 2048, 16, 2048),
                                           (1, 0, 16, 2048, 2048), (1, 0, 8, 1024, 4096), (0, 1, 300, 20, 1000),
-                                          (0, 1, 64, 64, 64)])
+                                          (0, 1, 64, 64, 64), (1, 1, 2048, 16, 2048), (1, 1, 40, 2048, 1024)])
 @pytest.mark.parametrize("scratch", [True, False])
 def test_gemm_scaled(ops, orc, tA, tB, M, N, K, scratch):
     """alpha * product, also accumulated, with K cut into runs (scratch) and as product + scale (no scratch)."""
@@ -253,6 +254,7 @@ def test_gemm_grouped(ops, orc, tA, tB, shapes, K):
     (1, 0, [(16, 2048, 2048)] * 4),                                                       # (dY B)^T x: the A gradients
     (0, 1, [(2048, 2048, 16), (2048, 1024, 16), (2048, 1024, 16)]),                       # (x A^T) B^T onto q, k, v: rank-sized K
     (0, 1, [(300, 20, 1000), (64, 64, 64)]),                                              # shapes that share no launch: single calls
+    (1, 1, [(2048, 16, 2048), (16, 1024, 2048), (512, 16, 1024)]),                        # both operands transposed (no call site in the step)
 ])
 @pytest.mark.parametrize("accumulate,alpha", [(False, 2.0), (True, 1.0)])
 def test_gemm_scaled_grouped_equals_the_single_calls(ops, orc, tA, tB, shapes, accumulate, alpha):
@@ -306,7 +308,7 @@ def test_gemm_chain(ops, orc, tA, tB, M, N, Ks):
 
 
 # ------------------------------------------------------------------ rmsnorm
-@pytest.mark.parametrize("rows,cols", [(33, 512), (17, 2048), (5, 4096), (9, 100), (4, 8192), (1, 4)])
+@pytest.mark.parametrize("rows,cols", [(33, 512), (17, 2048), (5, 4096), (9, 100), (4, 8192), (1, 4), (21, 1024), (11, 1408), (6, 256)])
 def test_rmsnorm_forward_backward(ops, orc, rows, cols):
     r = rng(rows + cols)
     x = r.standard_normal((rows, cols)).astype(np.float32)
@@ -409,7 +411,8 @@ def test_qk_norm(ops, orc):
     parity(ops.qk_norm_backward(dev(x), dev(dy), 4, 64, 1e-6), orc.qk_norm_backward(x, dy, 4, 64, 1e-6), "qk_norm bwd")
 
 
-@pytest.mark.parametrize("T,heads,D", [(37, 4, 64), (300, 16, 128), (5, 3, 6), (1000, 8, 128), (64, 2, 32)])
+@pytest.mark.parametrize("T,heads,D", [(37, 4, 64), (300, 16, 128), (5, 3, 6), (1000, 8, 128), (64, 2, 32), (50, 4, 128), (20, 32, 128),
+                                       (9, 40, 128)])           # 512, 4096 and 5120 values per token: two and sixteen float4 per lane, and the loop
 def test_qk_norm_saved_pair(ops, orc, T, heads, D):
     """The pair the training step uses: the forward that also leaves each token's rms, and the backward from the
     normalised output and that rms.  Same derivative as the backward from the input (the oracle's), also in place, also
@@ -591,6 +594,51 @@ def test_attention_backward_assign_checks_the_host_offsets(ops):
     for bad in ([0, 40, 90], [1, 40, 100], [0, 60, 50, 100][:3]):
         with pytest.raises(SeraphError):
             ops.attention_backward_assign(dev(Q), dev(K), dev(V), dev(dO), 2, 2, 32, sd, bad)
+
+
+def test_scratch_that_is_missing_or_too_small_is_refused(ops):
+    """Entry points that take caller-owned scratch return SERAPH_ERR_WORKSPACE (-3) before they touch anything when it is
+    missing, misaligned or smaller than their *_ws_bytes() query says; the outputs keep what they held."""
+    import ctypes as C
+    from seraph_amd._lib import kernels
+    k = kernels()
+    k.seraph_hip_last_error.restype = C.c_char_p
+    i64, sz, f32, p = C.c_int64, C.c_size_t, C.c_float, lambda t: C.c_void_p(t.data_ptr())
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    T, h, V, H, D = 64, 256, 300, 2, 32
+    x, dy = torch.randn(T, h, device="cuda"), torch.randn(T, h, device="cuda")
+    w = torch.ones(h, device="cuda")
+    dx, gs = torch.full((T, h), 5.0, device="cuda"), torch.full((h,), 5.0, device="cuda")
+    small = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    nparts = C.c_int(0)
+    tok = torch.randint(0, V, (T,), device="cuda", dtype=torch.int32)
+    ge = torch.full((V, h), 5.0, device="cuda")
+    q = torch.randn(T, H * D, device="cuda")
+    dq, dk, dv = (torch.full((T, H * D), 5.0, device="cuda") for _ in range(3))
+    calls = {
+        "rmsnorm_backward": lambda ws, n: k.seraph_rmsnorm_backward(p(x), p(w), p(dy), p(dx), p(gs), i64(T), i64(h), f32(1e-5), ws, sz(n), st),
+        "rmsnorm_backward_rows": lambda ws, n: k.seraph_rmsnorm_backward_rows(p(x), p(w), p(dy), None, p(dx), i64(T), i64(h), f32(1e-5), ws, sz(n),
+                                                                            C.byref(nparts), st),
+        "embedding_backward": lambda ws, n: k.seraph_embedding_backward(p(tok), p(dy), p(ge), i64(T), i64(h), i64(V), ws, sz(n), st),
+        "attention_backward": lambda ws, n: k.seraph_attention_backward(p(q), p(q), p(q), p(q), None, None, p(dq), p(dk), p(dv), None, 1, i64(T),
+                                                                      H, H, D, f32(D ** -0.5), ws, sz(n), st),
+    }
+    for name, call in calls.items():
+        assert call(None, 0) == -3, name
+        assert call(p(small), 64) == -3, name
+        assert b"scratch" in k.seraph_hip_last_error(), name
+    torch.cuda.synchronize()
+    for t in (dx, gs, ge, dq, dk, dv):
+        assert (t == 5.0).all()
+    # the non-banded attention backward with scratch of the size it asks for: the sum into dK / dV, dQ overwritten
+    k.seraph_attention_backward_ws_bytes.restype = C.c_size_t
+    need = k.seraph_attention_backward_ws_bytes(i64(T), H, H, D)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    dk.zero_(); dv.zero_()
+    assert calls["attention_backward"](p(ws), need) == 0
+    ref = ops.attention_backward(q, q, q, q, H, H, D)
+    for got, want in zip((dq, dk, dv), ref):
+        assert torch.allclose(got, want, rtol=1e-4, atol=1e-5)
 
 
 def test_rope_and_cross_entropy_many_short_sequences(ops, orc):
