@@ -416,6 +416,34 @@ def test_reference_batched_trainer_profile_and_lora(tmp_path, orc, binary):
     assert "lora_gB [64x4" not in err
 
 
+def test_front_end_stops_on_a_nan_and_says_where(tmp_path, orc):
+    """--debug-nan-check through the stand-alone front end, as tools/seraph_train_cuda.c:457-476 behaves: a model whose
+    first query projection holds a NaN stops at step 1 with exit status 2, the optimizer is skipped, the report names the
+    first poisoned buffers and no checkpoint of poisoned weights is left behind."""
+    import glob
+    from safetensors.torch import load_file, save_file
+    mdir, ckpt = str(tmp_path / "model"), str(tmp_path / "ckpt")
+    make_model_dir(mdir, orc, SHAPE, seed=81)
+    f = os.path.join(mdir, "model.safetensors")
+    tensors = load_file(f)
+    name = [k for k in tensors if "layers.0." in k and "q_proj" in k][0]
+    tensors[name][0, 3] = float("nan")
+    save_file(tensors, f)
+    write_ttok(os.path.join(mdir, "train.ttok"), make_samples(82, 6, SHAPE["vocab"], lo=5), vocab=SHAPE["vocab"])
+    before = set(glob.glob("/tmp/seraph_nan_step_1_*"))
+    rc, out, err = run_cli([mdir, os.path.join(mdir, "train.ttok"), "--full-training", "--batch", 2, "--max-seq", 24, "--log-every", 1,
+                            "--debug-nan-check", "--checkpoint", ckpt])
+    try:
+        assert rc == 2, (out[-800:], err[-1500:])
+        assert "[NAN] detected at step=1" in err and "(optimizer skipped)" in err
+        assert "  - buffer: " in err and "[FATAL] NaN detected at step 1 - stopping training" in err
+        assert not step_losses(out)                               # the step is not logged as a training step
+        assert not os.path.exists(os.path.join(ckpt, "checkpoint_final.safetensors"))
+    finally:
+        for dump in set(glob.glob("/tmp/seraph_nan_step_1_*")) - before:
+            os.remove(dump)
+
+
 def test_nan_detection_writes_the_dump_files_the_reference_inspector_reads(tr, orc, tmp_path):
     """A step that detects a NaN writes the step's buffers as the reference does (src/train.c:5562-5653).  The files are
     read back with a restatement of what tools/nan_dump_inspect.c does with them (sizes from the token file and the model
