@@ -22,6 +22,8 @@
  *
  * LoRA steps are not forwarded: the reference's CUDA LoRA step keeps running op by op over cuda_train_*.
  * Video models (num_queries > 0) and SERAPH_HIP_FUSED_STEP=0 in the environment take the op-by-op step too.
+ * SERAPH_HIP_FUSED_TOKENS=n sets the room the fused trainer starts with (default: batch size x longest sequence of the
+ * training configuration).
  */
 #include <math.h>
 #include <stdio.h>
@@ -113,7 +115,13 @@ static hip_trainer_t* fused_trainer(train_state_t* state, cuda_train_context_t* 
     hip_optim_config_t o = {state->learning_rate, 0.9f, 0.999f, 0.01f, 1e-8f, 0.0f, 100,
                             state->gradient_accumulation_steps < 1 ? 1 : state->gradient_accumulation_steps};
     int want_tokens = total_tokens, want_batch = batch_size;
-    if (state->train_cfg && state->train_cfg->batch_size > 0 && state->train_cfg->max_seq_len > 0) {
+    /* Room for the largest batch the training configuration allows, so that the trainer is created once.
+     * SERAPH_HIP_FUSED_TOKENS=n in the environment starts with room for n tokens instead (activation memory for the
+     * batches that actually arrive); a batch that does not fit makes a larger trainer and carries the arenas over. */
+    const char* room = getenv("SERAPH_HIP_FUSED_TOKENS");
+    if (room && atol(room) > 0 && atol(room) < (1L << 30)) {
+        if (atol(room) > want_tokens) want_tokens = (int)atol(room);
+    } else if (state->train_cfg && state->train_cfg->batch_size > 0 && state->train_cfg->max_seq_len > 0) {
         const long cap = (long)state->train_cfg->batch_size * (long)state->train_cfg->max_seq_len;
         if (cap > want_tokens && cap < (1L << 30)) want_tokens = (int)cap;
         if (state->train_cfg->batch_size > want_batch) want_batch = state->train_cfg->batch_size;
@@ -146,6 +154,7 @@ static hip_trainer_t* fused_trainer(train_state_t* state, cuda_train_context_t* 
     }
     if (keep[0]) {
         for (int a = 0; a < 4; a++) { hip_trainer_upload(t, a, keep[a], n); free(keep[a]); }
+        fprintf(stderr, "[HIP] fused training step: room grown to %d tokens in %d sequences\n", want_tokens, want_batch);
     } else {
         /* weights (and moments, zero in a fresh state) of every tensor into its place in the arenas */
         int ns = 0;

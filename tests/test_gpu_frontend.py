@@ -553,3 +553,35 @@ def test_fused_front_end_validation_accumulation_and_the_switch_back(tmp_path, o
     from seraph_amd import io as sio
     saved = sio.checkpoint_load(str(tmp_path / "fused" / "checkpoint_final.safetensors"), cfg)
     assert np.all(np.abs(saved - rp) <= 2.0 ** -7 * np.abs(rp) + 1e-6)
+
+
+@pytest.mark.skipif(not os.path.exists(FUSED_BIN), reason="fused front end not built")
+def test_fused_front_end_grows_with_the_batches_and_takes_single_sequences(tmp_path, orc):
+    """Two more ways into the fused step from the reference's front end.  (1) SERAPH_HIP_FUSED_TOKENS=1: the fused trainer
+    starts with room for the first batch only; the samples get longer, so later batches make a larger trainer and the four
+    arenas (weights, the gradients of an open accumulation window, both Adam moments) travel to it.  (2) A batch that
+    holds a single sequence - the thirteenth sample is left over - goes through cuda_train_step_gpu_full
+    (tools/seraph_train_cuda.c:431-435).  The losses and the final weights are the oracle's."""
+    mdir = str(tmp_path / "model")
+    ocfg, cfg, p0 = make_model_dir(mdir, orc, SHAPE, seed=95)
+    add_tokenizer(mdir, SHAPE["vocab"])
+    r = np.random.default_rng(96)
+    samples = [r.integers(0, SHAPE["vocab"], n).astype(np.int32) for n in (5, 6, 8, 9, 12, 13, 17, 18, 24, 25, 31, 32, 20)]
+    ttok = os.path.join(mdir, "train.ttok")
+    write_ttok(ttok, samples, vocab=SHAPE["vocab"])
+    tokens = np.concatenate(samples)
+    offsets = np.concatenate([[0], np.cumsum([len(s) for s in samples])]).tolist()
+    batches = reference_pack(tokens.tolist(), offsets, 2, 32)
+    assert len(batches) == 7 and len(batches[-1][1]) == 2            # the last batch: one sequence
+    args = [mdir, ttok, "--full-training", "--batch", 2, "--max-seq", 32, "--lr", 2e-3, "--log-every", 1, "--save-every", 0,
+            "--accum", 2, "--checkpoint", tmp_path / "ckpt"]
+    rc, out, err = run_ref(args, binary=FUSED_BIN, env={"SERAPH_HIP_FUSED_TOKENS": "1"})
+    assert rc == 0, (out[-1500:], err[-1500:])
+    assert "[HIP] fused training step" in err and err.count("room grown to") >= 3, err[-1500:]
+    ref_losses, rp, _, _ = oracle_run(orc, ocfg, p0.copy(), batches, 2e-3, accum=2)
+    got = [l for _, l in step_losses(out)]
+    assert len(got) == len(batches) and np.allclose(got, ref_losses, atol=1.5e-4), (got, ref_losses)
+    from seraph_amd import io as sio
+    saved = sio.checkpoint_load(str(tmp_path / "ckpt" / "checkpoint_final.safetensors"), cfg)
+    assert np.all(np.abs(saved - rp) <= 2.0 ** -7 * np.abs(rp) + 1e-6)
+    assert np.abs(rp - p0).max() > 1e-6
