@@ -116,6 +116,9 @@ float hip_evaluate(hip_trainer_t* t, const int* val_tokens, int num_val_tokens, 
 /* Resume support: the learning rate and the two counters of src/train.c:5439-5463
  * (state->optimizer_step, state->accumulation_counter); a negative counter is left unchanged. */
 void  hip_trainer_set_schedule(hip_trainer_t* t, float learning_rate, int optimizer_step, int accumulation_counter);
+/* The number of training steps run so far (state->current_step of the reference): the step number in the names of
+ * the NaN dump files and in their metadata is this plus one. */
+void  hip_trainer_set_step_counter(hip_trainer_t* t, int steps_run);
 int   hip_trainer_accumulation_counter(const hip_trainer_t* t);
 
 /* NaN/Inf flag lattice of the reference's --debug-nan-check (src/train.c:4499-4546): with it on,

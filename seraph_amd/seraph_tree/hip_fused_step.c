@@ -54,6 +54,7 @@ static struct {
     hip_trainer_t* t;
     int max_tokens, max_batch;
     int opbyop;                     /* this state has taken an op-by-op step: its weights live in the per-tensor buffers */
+    int nan_check;                  /* the trainer's NaN checks are on */
 } g;
 
 static double now_ms(void) {
@@ -170,6 +171,7 @@ static hip_trainer_t* fused_trainer(train_state_t* state, cuda_train_context_t* 
                 (long long)n, want_tokens, want_batch);
     }
     g.t = t; g.ctx = ctx; g.state = state; g.max_tokens = want_tokens; g.max_batch = want_batch;
+    g.nan_check = 0;                                                /* a new trainer starts without them */
     return t;
 }
 
@@ -196,6 +198,11 @@ float cuda_train_step_gpu_full_batch(train_state_t* state, int* tokens_packed, i
     if (total_tokens - batch_size <= 0) return 0.0f;                                 /* :1990-1991 */
     /* the state's counters and learning rate are the truth (a resume sets them): src/train_cuda.c:2287-2303 */
     hip_trainer_set_schedule(t, state->learning_rate, state->optimizer_step, state->accumulation_counter);
+    /* --debug-nan-check: the flag lattice, the held-back optimizer and the dump files of the reference's single-sequence
+     * step (src/train_cuda.c:633-661, :1080-1187), for packed batches as well (the reference's packed step has no checks) */
+    const int want_nan = state->debug_nan_check ? 1 : 0;
+    if (want_nan != g.nan_check && hip_trainer_enable_nan_check(t, want_nan) == 0) g.nan_check = want_nan;
+    if (g.nan_check) hip_trainer_set_step_counter(t, state->current_step);
     /* --profile: the fused step has no per-call ops to bracket; its kernels are timed per class (event pairs around
      * every kernel-library call of this one step) and each class goes to the front end's profiler as one entry, named so
      * that the profiler's substring categories (src/cuda_profiler.cu:152-172) file it where the op-by-op step's ops go */
@@ -216,6 +223,15 @@ float cuda_train_step_gpu_full_batch(train_state_t* state, int* tokens_packed, i
             hip_cuda_profiler_add(prof, label, (float)stats[i].ms, (size_t)stats[i].flops, (size_t)stats[i].bytes);
         }
         hip_trainer_enable_op_timing(t, 0);
+    }
+    if (g.nan_check && hip_trainer_nan_detected(t)) {                                /* src/train_cuda.c:1097-1183 */
+        fprintf(stderr, "[NAN] detected at step=%d seq=%d (optimizer skipped)\n", state->current_step + 1, total_tokens);
+        fprintf(stderr, "  - lr(base)=%g opt_step=%d accum=%d/%d\n", (double)state->learning_rate, state->optimizer_step,
+                state->accumulation_counter, state->gradient_accumulation_steps);
+        hip_trainer_nan_report(t, stderr);
+        fprintf(stderr, "[NAN-DUMP] wrote buffers with prefix /tmp/seraph_nan_step_%d_*\n", state->current_step + 1);
+        state->nan_detected = 1;
+        return NAN;
     }
     state->optimizer_step = hip_trainer_optimizer_step(t);
     state->accumulation_counter = hip_trainer_accumulation_counter(t);

@@ -522,6 +522,10 @@ void hip_trainer_set_schedule(hip_trainer_t* t, float learning_rate, int optimiz
     if (accumulation_counter >= 0) t->accumulation_counter = accumulation_counter;
 }
 
+void hip_trainer_set_step_counter(hip_trainer_t* t, int steps_run) {
+    if (t && steps_run >= 0) t->step_counter = steps_run;
+}
+
 int hip_trainer_accumulation_counter(const hip_trainer_t* t) { return t ? t->accumulation_counter : -1; }
 
 int64_t hip_trainer_arena_count(hip_trainer_t* t, int which) {

@@ -416,19 +416,64 @@ def test_reference_batched_trainer_profile_and_lora(tmp_path, orc, binary):
     assert "lora_gB [64x4" not in err
 
 
-def test_front_end_stops_on_a_nan_and_says_where(tmp_path, orc):
-    """--debug-nan-check through the stand-alone front end, as tools/seraph_train_cuda.c:457-476 behaves: a model whose
-    first query projection holds a NaN stops at step 1 with exit status 2, the optimizer is skipped, the report names the
-    first poisoned buffers and no checkpoint of poisoned weights is left behind."""
-    import glob
+def poison_first_query_projection(mdir):
     from safetensors.torch import load_file, save_file
-    mdir, ckpt = str(tmp_path / "model"), str(tmp_path / "ckpt")
-    make_model_dir(mdir, orc, SHAPE, seed=81)
     f = os.path.join(mdir, "model.safetensors")
     tensors = load_file(f)
     name = [k for k in tensors if "layers.0." in k and "q_proj" in k][0]
     tensors[name][0, 3] = float("nan")
     save_file(tensors, f)
+
+
+@needs_ref
+@pytest.mark.parametrize("binary", BINARIES)
+def test_reference_front_end_with_debug_nan_check(tmp_path, orc, binary):
+    """--debug-nan-check through the reference's front end.  Its single-sequence step checks its buffers
+    (src/train_cuda.c:633-661, :1080-1187), its packed step does not; the fused step checks in both.  A clean model trains
+    to the same losses with the checks on; a model with a NaN in its first query projection is stopped by the fused
+    step at step 1 (report, dump files, the front end's [FATAL] lines, tools/seraph_train_cuda.c:472-476), with packed
+    batches too."""
+    import glob
+    mdir = str(tmp_path / "model")
+    ocfg, cfg, p0 = make_model_dir(mdir, orc, SHAPE, seed=85)
+    add_tokenizer(mdir, SHAPE["vocab"])
+    samples = make_samples(86, 6, SHAPE["vocab"], lo=6, hi=24)
+    ttok = os.path.join(mdir, "train.ttok")
+    write_ttok(ttok, samples, vocab=SHAPE["vocab"])
+    args = [mdir, ttok, "--full-training", "--batch", 2, "--max-seq", 32, "--lr", 2e-3, "--log-every", 1, "--save-every", 0,
+            "--debug-nan-check"]
+    rc, out, err = run_ref(args + ["--checkpoint", tmp_path / "clean"], binary=binary)
+    assert rc == 0, (out[-1500:], err[-1500:])
+    tokens = np.concatenate(samples)
+    offsets = np.concatenate([[0], np.cumsum([len(s) for s in samples])]).tolist()
+    batches = reference_pack(tokens.tolist(), offsets, 2, 32)
+    ref_losses, _, _, _ = oracle_run(orc, ocfg, p0.copy(), batches, 2e-3)
+    assert np.allclose([l for _, l in step_losses(out)], ref_losses, atol=1.5e-4)
+    assert "[NAN]" not in err
+    if binary != FUSED_BIN:
+        return                                                   # the reference's packed step has no checks to trip
+    poison_first_query_projection(mdir)
+    before = set(glob.glob("/tmp/seraph_nan_step_1_*"))
+    rc, out, err = run_ref(args + ["--checkpoint", tmp_path / "poisoned"], binary=binary)
+    try:
+        assert "[NAN] detected at step=1" in err and "(optimizer skipped)" in err, err[-1500:]
+        assert "  - buffer: " in err and "[FATAL] NaN detected at step 1 - stopping training" in err
+        dumps = set(glob.glob("/tmp/seraph_nan_step_1_*")) - before
+        assert any(d.endswith("_meta.txt") for d in dumps), dumps
+        assert not step_losses(out)
+    finally:
+        for dump in set(glob.glob("/tmp/seraph_nan_step_1_*")) - before:
+            os.remove(dump)
+
+
+def test_front_end_stops_on_a_nan_and_says_where(tmp_path, orc):
+    """--debug-nan-check through the stand-alone front end, as tools/seraph_train_cuda.c:457-476 behaves: a model whose
+    first query projection holds a NaN stops at step 1 with exit status 2, the optimizer is skipped, the report names the
+    first poisoned buffers and no checkpoint of poisoned weights is left behind."""
+    import glob
+    mdir, ckpt = str(tmp_path / "model"), str(tmp_path / "ckpt")
+    make_model_dir(mdir, orc, SHAPE, seed=81)
+    poison_first_query_projection(mdir)
     write_ttok(os.path.join(mdir, "train.ttok"), make_samples(82, 6, SHAPE["vocab"], lo=5), vocab=SHAPE["vocab"])
     before = set(glob.glob("/tmp/seraph_nan_step_1_*"))
     rc, out, err = run_cli([mdir, os.path.join(mdir, "train.ttok"), "--full-training", "--batch", 2, "--max-seq", 24, "--log-every", 1,
