@@ -129,9 +129,18 @@ def gemm_table(w):
     from seraph_amd import ops
     ops.init(0)
 
-    def timeit(fn, iters=5, warm=2):
-        for _ in range(warm):
+    def timeit(fn):
+        # about 30 ms of untimed calls first (a row that follows allocations and host work would otherwise be timed on
+        # clocks that have not come back up: the first row of either table read 6-10 % slow for both libraries), then
+        # at least 5 calls and 50 ms under one event pair
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        once = max(time.perf_counter() - t0, 1e-5)
+        for _ in range(min(200, max(2, int(0.03 / once)))):
             fn()
+        iters = min(200, max(5, int(0.05 / once)))
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         a.record()
