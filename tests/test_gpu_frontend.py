@@ -437,7 +437,7 @@ def test_reference_front_end_with_debug_nan_check(tmp_path, orc, binary):
     mdir = str(tmp_path / "model")
     ocfg, cfg, p0 = make_model_dir(mdir, orc, SHAPE, seed=85)
     add_tokenizer(mdir, SHAPE["vocab"])
-    samples = make_samples(86, 6, SHAPE["vocab"], lo=6, hi=24)
+    samples = make_samples(86, 7, SHAPE["vocab"], lo=6, hi=24)      # the seventh is a batch of its own: the single-sequence step
     ttok = os.path.join(mdir, "train.ttok")
     write_ttok(ttok, samples, vocab=SHAPE["vocab"])
     args = [mdir, ttok, "--full-training", "--batch", 2, "--max-seq", 32, "--lr", 2e-3, "--log-every", 1, "--save-every", 0,
