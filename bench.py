@@ -101,11 +101,88 @@ def cpu_baseline(w, budget_tokens=192):
                         C.c_float(0.999), C.c_float(0.01), C.c_float(1e-8), C.c_int(1), C.c_float(w["clip"]))
     opt = time.perf_counter() - t0
     del arrs
-    return dict(value=round(T / (full + opt), 3), unit="tok/s", cores=orc.num_threads(), kind="port",
+    model, cpus = host_cpu()
+    return dict(value=round(T / (full + opt), 3), unit="tok/s", cores=orc.num_threads(), kind="port", cpu_model=model, host_cpus=cpus,
                 sample=(f"oracle step (fwd+loss+bwd) on {T} tokens in 1 sequence at full width and vocabulary, "
                         f"1 layer {best[1]:.2f}s and 3 layers {best[3]:.2f}s (best of 2); LM-head/embedding cost "
                         f"{head:.2f}s + {per_layer:.2f}s per layer scaled to {w['layers']} layers = {full:.1f}s, plus one "
                         f"AdamW pass over all {n} trainable parameters, {opt:.2f}s (timed once)"))
+
+
+def host_cpu():
+    """(model name, logical CPUs the process may run on) of the host."""
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    try:
+        n = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        n = os.cpu_count() or 0
+    return model, n
+
+
+def cpu_ops():
+    """The oracle's own loops for the single-op configurations, on the host cores, each on a bounded part of the
+    configuration (fewer rows, heads or sequences: the ops are independent per row / head / sequence) and scaled to the whole:
+    name -> dict(ms, sample).  Best of two runs each; a few seconds in all."""
+    import ctypes as C
+    from oracle import oracle as orc
+    r = np.random.default_rng(3)
+    out = {}
+
+    def best_of_2(fn):
+        b = 1e30
+        for _ in range(2):
+            t0 = time.perf_counter()
+            fn()
+            b = min(b, time.perf_counter() - t0)
+        return b
+
+    def put(name, seconds, factor, sample):
+        out[name] = dict(ms=round(1e3 * seconds * factor, 2), unit="ms", cores=orc.num_threads(), kind="port",
+                         sample=f"{sample}: {1e3 * seconds:.2f} ms, x {factor:g}")
+
+    # attention at B8 H16 S1024 D64: one sequence, two heads of the sixteen
+    S, H, D = 1024, 2, 64
+    q, k, v, do = (r.standard_normal((S, H * D)).astype(np.float32) / 8 for _ in range(4))
+    put("attention_backward_b8_h16_s1024_d64", best_of_2(lambda: orc.attention_backward(q, k, v, do, H, H, D)), 8 * 16 / H,
+        "one sequence of 1024 tokens, 2 heads")
+    put("attention_forward_b8_h16_s1024_d64", best_of_2(lambda: orc.attention_forward(q, k, v, H, H, D)), 8 * 16 / H,
+        "one sequence of 1024 tokens, 2 heads")
+    # the bandwidth-bound chain: half of the 16384 rows (1/64 for the cross entropy, 1/8 for SwiGLU, half of the AdamW elements)
+    rows, cols, V = 16384, 2048, 151936
+    x = 2 * r.standard_normal((rows // 64, V), dtype=np.float32)
+    t = r.integers(0, V, rows // 64).astype(np.uint32)
+    put("cross_entropy_grad_16384_x_151936", best_of_2(lambda: orc.cross_entropy_grad(x, t)), 64, "256 rows of 151936")
+    del x
+    n = rows // 2
+    a, b = r.standard_normal((n, cols), dtype=np.float32), 1e-2 * r.standard_normal((n, cols), dtype=np.float32)
+    gains = (1 + 0.02 * r.standard_normal(cols)).astype(np.float32)
+    put("rmsnorm_backward_16384_x_2048", best_of_2(lambda: orc.rmsnorm_backward_batch(a, gains, b, 1e-6)), 2, "8192 rows of 2048")
+    put("qk_norm_backward_16384_x_16_heads_128", best_of_2(lambda: orc.qk_norm_backward(a, b, 16, 128, 1e-6)), 2, "8192 tokens, 16 heads of 128")
+    put("rope_backward_16384_x_16_heads_128", best_of_2(lambda: orc.rope(a, 16, 128, 1e6, backward=True)), 2, "8192 tokens, 16 heads of 128")
+    table = np.zeros((V, cols), np.float32)
+    tok = r.integers(0, V, n).astype(np.uint32)
+    f32p = lambda arr: arr.ctypes.data_as(C.POINTER(C.c_float))
+    put("embedding_backward_16384_x_2048_into_151936_rows",
+        best_of_2(lambda: orc.lib().orc_embedding_backward(tok.ctypes.data_as(C.POINTER(C.c_uint32)), f32p(a), f32p(table), C.c_int64(n),
+                                                           C.c_int64(cols), C.c_int64(V))), 2, "8192 tokens into the 151936-row table, in place")
+    del table
+    g3 = [r.standard_normal((rows // 8, 6144), dtype=np.float32) for _ in range(3)]
+    put("swiglu_backward_16384_x_6144", best_of_2(lambda: orc.swiglu_backward(*g3)), 8, "2048 rows of 6144")
+    del g3
+    m = 25_000_000
+    arrs = [np.full(m, val, np.float32) for val in (0.01, 1e-3, 0.0, 0.0)]
+    for clip in (0.0, 1.0):
+        put(f"adamw_50m_clip_{clip:g}",
+            best_of_2(lambda: orc.lib().orc_adamw(*[f32p(z) for z in arrs], C.c_int64(m), C.c_float(3.14e-4), C.c_float(0.9), C.c_float(0.999),
+                                                  C.c_float(0.01), C.c_float(1e-8), C.c_int(1), C.c_float(clip))), 2, "25 M elements, in place")
+    return out
 
 
 def measured_traffic(kernel, workload):
@@ -666,6 +743,9 @@ def main():
             ref = reference_cpu_step(c1)
             if ref is not None:
                 out["workloads"]["c1"]["cpu_baseline_reference"] = ref
+            for name, cpu in cpu_ops().items():
+                if name in out["ops"]:
+                    out["ops"][name]["cpu_baseline"] = cpu
     out.update(contract)
     summary = {args.workload: [head["value"], head["ms_per_step"]]}
     for key, r in out.get("workloads", {}).items():
